@@ -1,0 +1,177 @@
+/*
+ * planmoe_hip.h -- C ABI of libplanmoe_hip.so: the per-GPU MoE data path of PlanMoE
+ * (top-k gating with capacity slots, dispatch / combine kernels with their backward
+ * passes, the "int8" and zfp fixed-rate codecs) as hand-written HIP kernels for gfx950.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the parameter name ends in _host;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); every call only
+ *     enqueues work on that stream and returns without synchronising;
+ *   - the library never allocates device memory: callers pass outputs and, where a call
+ *     needs scratch, a workspace sized by the matching *_workspace_bytes() query;
+ *   - return value 0 = success; anything else is an error whose text is available from
+ *     planmoe_last_error() (thread local).  Nothing is enqueued when an error is returned;
+ *   - choice planes: per-token routing data of the k choices are k planes of `samples`
+ *     elements, plane j starting at base + j * plane_stride (elements, >= samples).  This is
+ *     the list-of-k-tensors of the reference (fast_dispatch.py:99-101) laid out in one buffer.
+ *   - a (token, choice) pair is LIVE iff location < capacity and index >= 0
+ *     (jit_kernels/sparse.py:29,50,78; custom_kernel.cpp:73,84,101).
+ *
+ * File:line citations name the interface of the reference (PlanMoE/...) each entry
+ * point replaces.
+ */
+#ifndef PLANMOE_HIP_H
+#define PLANMOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PLANMOE_ABI_VERSION 1
+
+typedef enum planmoe_dtype {
+    PLANMOE_F32 = 0,
+    PLANMOE_BF16 = 1,
+    PLANMOE_F16 = 2
+} planmoe_dtype;
+
+/* ---------------------------------------------------------------- housekeeping */
+
+int planmoe_abi_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). Host pointer. */
+const char *planmoe_last_error(void);
+
+/* ---------------------------------------------------------------- capacity cumsum
+ * Replaces torch.ops.tutel_ops.cumsum / warp_cumsum (custom/custom_kernel.cpp:331-385),
+ * reached through fast_cumsum_sub_one (jit_kernels/gating.py:17-22).
+ * out[t][c] = (sum of in[0..t][c]) - 1 for an int32 row-major [samples, columns] matrix.
+ * Workspace: planmoe_cumsum_workspace_bytes(samples, columns). */
+size_t planmoe_cumsum_workspace_bytes(int samples, int columns);
+int planmoe_cumsum_sub_one(const int32_t *in, int32_t *out, int samples, int columns,
+                           void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------- routing
+ * Replaces extract_critical (impls/fast_dispatch.py:140-195) for the capacity_factor > 0,
+ * non-batch-prioritised case, together with the softmax of the layer's routing closure
+ * (impls/moe_layer.py:239) and the GShard auxiliary loss (impls/losses.py:12-19).
+ */
+
+/* capacity = k * int(cf * ceil(T / E)) rounded up to `alignment`  (fast_dispatch.py:179-190).
+ * Host-only arithmetic; capacity_factor must be > 0. */
+int planmoe_capacity(int samples, int experts, int top_k, double capacity_factor,
+                     int alignment, int *capacity_host);
+
+size_t planmoe_route_workspace_bytes(int samples, int experts, int top_k);
+
+/* input        [samples, experts] row-major in `dtype` (F32 or BF16): softmax scores, or
+ *              gate logits when input_is_logits != 0 (softmax over experts is then applied
+ *              first, in fp32, rounded to `dtype`).
+ * logit_bias   optional fp32 [experts] added to the logits before the softmax (NULL = none;
+ *              only with input_is_logits).
+ * indices      out int32 k planes   expert id of the j-th largest score (ties: lower id)
+ * locations    out int32 k planes   slot inside that expert; all first choices of an expert
+ *              come first in token order, then all second choices, ...
+ * gates        out `dtype` k planes score of the chosen expert, divided by
+ *              clamp(sum over the k choices, eps(dtype)) when normalize_gate and k > 1
+ * scores_out   optional out [samples, experts] `dtype`: the scores routing was done on
+ * l_aux        optional out fp32 scalar: sum_e(me[e] * ce[e]) / samples with me = column sums
+ *              of the scores and ce = (experts / samples) * number of first choices of e
+ * expert_counts optional out int32 [top_k, experts]: tokens whose j-th choice is e
+ * top_k is clamped to `experts` (fast_dispatch.py:142); planes beyond the clamp are untouched.
+ */
+int planmoe_route_topk(const void *input, int dtype, int input_is_logits, const float *logit_bias,
+                       int samples, int experts, int top_k, int normalize_gate,
+                       int32_t *indices, int32_t *locations, void *gates, int64_t plane_stride,
+                       void *scores_out, float *l_aux, int32_t *expert_counts,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
+/* Gate logits  logits[samples, experts] = x[samples, model_dim] . wg[experts, model_dim]^T
+ * (gates/top.py:20-26).  x and wg are in `dtype` (BF16: MFMA with fp32 accumulation; F32:
+ * fp32 FMA); logits are written in `out_dtype` (F32 = the fp32_gate flow, or `dtype`). */
+int planmoe_gate_logits(const void *x, const void *wg, int dtype, void *logits, int out_dtype,
+                        int samples, int model_dim, int experts, void *stream);
+
+/* ---------------------------------------------------------------- dispatch / combine
+ * Replace the JIT kernels of jit_kernels/sparse.py (create_forward :17-35,
+ * create_backward_data :38-64, create_backward_gate :67-134), their CPU twins
+ * invoke_cpu_fp32 (custom/custom_kernel.cpp:57-112) and the per-choice launch loops of
+ * GatingEncoder / GatingDecoder (impls/fast_dispatch.py:16-79).
+ * Tensors are in `dtype` (F32, BF16 or F16); arithmetic is fp32 with one rounding per
+ * operation, as the reference's dispatcher computes (fast_dispatch.py:91-93,121-131).
+ * `gates` are fp32 planes or NULL for the all-ones helper (fast_dispatch.py:24,57).
+ */
+
+size_t planmoe_dispatch_workspace_bytes(int experts, int capacity);
+
+/* GatingEncoder.forward (fast_dispatch.py:18-29) == GatingDecoder.backward's scatter (:66-71):
+ *   dispatched[(idx*capacity + loc), :] = 0 + gate * x[t, :]   for every live pair,
+ *   every other row of dispatched[experts*capacity, model_dim] = 0.
+ * Live pairs must address distinct slots (true for planmoe_route_topk's output); when two
+ * pairs collide the later write wins instead of the reference's sum. */
+int planmoe_dispatch_fwd(const void *x, int dtype, const float *gates, const int32_t *indices,
+                         const int32_t *locations, int64_t plane_stride, int top_k,
+                         int samples, int model_dim, int experts, int capacity,
+                         void *dispatched, void *workspace, size_t workspace_bytes, void *stream);
+
+/* GatingDecoder.forward (fast_dispatch.py:51-64) == GatingEncoder.backward's data path (:33-38):
+ *   out[t, :] = sum over j (left to right) of (live_j ? gate_j * dispatched[slot_j, :] : 0). */
+int planmoe_combine_fwd(const void *dispatched, int dtype, const float *gates,
+                        const int32_t *indices, const int32_t *locations, int64_t plane_stride,
+                        int top_k, int samples, int model_dim, int capacity, void *out,
+                        void *stream);
+
+/* create_backward_gate for all k planes at once (fast_dispatch.py:40-45, 73-78):
+ *   grad_gates[j][t] = live ? <dispatched[slot_j, :], x[t, :]> : 0    (fp32 planes) */
+int planmoe_bwd_gate(const void *x, const void *dispatched, int dtype, const int32_t *indices,
+                     const int32_t *locations, int64_t plane_stride, int top_k, int samples,
+                     int model_dim, int capacity, float *grad_gates, void *stream);
+
+/* ---------------------------------------------------------------- "int8" codec
+ * Replaces Int8Compressor::compress / ::decompress (custom/compressor/int8.cpp:7-60).
+ * Per row of row_len elements: bias = min, scale = max - min,
+ *   code = uint8(((x - bias) / scale) * 255)      three roundings in `dtype`, truncation;
+ *   rows with scale == 0 (e.g. empty capacity slots) encode to 0.
+ * bias and scale are written in `dtype` (one element per row).
+ *   out  = ((code / 255) * scale) + bias          three roundings in `dtype`. */
+int planmoe_int8_compress(const void *x, int dtype, int64_t rows, int row_len, uint8_t *codes,
+                          void *bias, void *scale, void *stream);
+int planmoe_int8_decompress(const uint8_t *codes, const void *bias, const void *scale, int dtype,
+                            int64_t rows, int row_len, void *out, void *stream);
+
+/* Dispatch and compress in one pass (fast_encode followed by Compress.apply with "int8":
+ * impls/moe_layer.py:265 then impls/overlap.py:12-16): the codes/bias/scale that
+ * planmoe_int8_compress would produce from planmoe_dispatch_fwd's output, without the
+ * intermediate [experts*capacity, model_dim] tensor ever reaching memory. */
+int planmoe_dispatch_int8(const void *x, int dtype, const float *gates, const int32_t *indices,
+                          const int32_t *locations, int64_t plane_stride, int top_k,
+                          int samples, int model_dim, int experts, int capacity,
+                          uint8_t *codes, void *bias, void *scale,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------- zfp fixed-rate codec
+ * Replaces ZfpCompressor::compress / ::decompress (custom/compressor/zfpc.cpp:23-86), i.e.
+ * zfp_compress / zfp_decompress of the third-party zfp library in fixed-rate mode on fp32.
+ * The stream is bit-identical to stock zfp 0.5.5 (64-bit words, no header).
+ *   dims = 2: the reference's call, field nx = fastest axis, ny rows, 4x4 blocks;
+ *   dims = 1: the nx*ny values as one array, blocks of 4.
+ * nx and ny must be multiples of 4 (zfpc.cpp:26-28); maxbits = floor(4^dims * rate + 0.5)
+ * must be a multiple of 32 (rate 8, the reference's default zfpc.h:17, qualifies in both). */
+
+/* zfp_stream_maximum_size for the field: what the reference sizes its buffer with (zfpc.cpp:39) */
+size_t planmoe_zfp_max_bytes(int dims, int64_t nx, int64_t ny, double rate);
+/* bytes zfp_compress returns (`length`, zfpc.cpp:48) */
+size_t planmoe_zfp_stream_bytes(int dims, int64_t nx, int64_t ny, double rate);
+
+int planmoe_zfp_compress(const float *field, int dims, int64_t nx, int64_t ny, double rate,
+                         void *stream_out, size_t stream_capacity, void *stream);
+int planmoe_zfp_decompress(const void *stream_in, int dims, int64_t nx, int64_t ny, double rate,
+                           float *field, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PLANMOE_HIP_H */

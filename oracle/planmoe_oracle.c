@@ -1,0 +1,571 @@
+/*
+ * CPU oracle for the PlanMoE per-GPU MoE data path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file restates, on the CPU and in plain C, the
+ * arithmetic of the reference's hot path so that the HIP kernels can be checked
+ * against it.  Nothing the product ships may link, load or call it: only the test
+ * suite, the smoke check and the benchmark's cpu_baseline leg do.
+ *
+ * Each function names the reference lines it follows (paths relative to the
+ * reference checkout, PlanMoE/...).  None of the reference's source is copied; the
+ * loops below are written from its observable semantics.
+ *
+ * Parity pins (what each function is checked against before it is trusted):
+ *   orc_dispatch_* / orc_combine_* / orc_bwd_gate_*  torch index_put/gather closed
+ *        forms, the dense GShard einsum on tiny shapes, fp64 autograd identities
+ *   orc_cumsum_sub_one                               torch.cumsum - 1, brute force
+ *   orc_route_*                                      torch.topk / scatter / cumsum chain
+ *        on tie-free inputs, O(T*E) brute force, slot-uniqueness invariants
+ *   orc_int8_*                                       literal torch-CPU op chain in the
+ *        input dtype, exhaustive bf16 sweep, min->0 / max->255 invariants
+ *   orc_zfp_*                                        golden bitstreams and decoded fields
+ *        from stock libzfp 0.5.5 (serial), cross-decode both ways
+ *
+ * Build: gcc -O2 -fPIC -shared -ffp-contract=off -fno-fast-math (see oracle/Makefile).
+ */
+#include <stdint.h>
+#include <stddef.h>
+#include <string.h>
+#include <math.h>
+#include <float.h>
+#include <stdlib.h>
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ bf16 helpers */
+
+static inline float bf16_to_f32(uint16_t h)
+{
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* round-to-nearest-even float -> bf16, the conversion torch applies after every
+ * bf16 ATen op */
+static inline uint16_t f32_to_bf16(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u)          /* NaN stays NaN (quiet) */
+        return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+static inline float rbf(float f) { return bf16_to_f32(f32_to_bf16(f)); }
+
+/* ------------------------------------------------------------------ dispatch / combine
+ * Semantics of the three sparse kernels, CPU flavour:
+ *   custom/custom_kernel.cpp:57-112 (invoke_cpu<T>, kernel_type 0/1/2) and the GPU twins
+ *   jit_kernels/sparse.py:24-34, 45-63, 74-133.
+ * A (token, choice) pair is live iff  location < capacity  and  expert index >= 0.
+ */
+
+/* kernel_type 0: dispatched[slot] += gate * x[token]   (custom_kernel.cpp:72-81) */
+#define DEF_DISPATCH(NAME, T)                                                          \
+ORC_API void NAME(const T *gate, const int32_t *idx, const int32_t *loc, const T *x,  \
+                  T *dispatched, int samples, int hidden, int capacity)                \
+{                                                                                      \
+    for (int t = 0; t < samples; ++t) {                                                \
+        if (!(loc[t] < capacity && idx[t] >= 0)) continue;                             \
+        T *dst = dispatched + ((int64_t)idx[t] * capacity + loc[t]) * hidden;          \
+        const T *src = x + (int64_t)t * hidden;                                        \
+        const T g = gate[t];                                                           \
+        for (int j = 0; j < hidden; ++j) dst[j] += g * src[j];                         \
+    }                                                                                  \
+}
+DEF_DISPATCH(orc_dispatch_f32, float)
+DEF_DISPATCH(orc_dispatch_f64, double)
+
+/* kernel_type 1: out[token] = gate * dispatched[slot], zeros when dropped
+ * (custom_kernel.cpp:82-97) */
+#define DEF_GATHER(NAME, T)                                                            \
+ORC_API void NAME(const T *gate, const int32_t *idx, const int32_t *loc, T *out,      \
+                  const T *dispatched, int samples, int hidden, int capacity)          \
+{                                                                                      \
+    for (int t = 0; t < samples; ++t) {                                                \
+        T *dst = out + (int64_t)t * hidden;                                            \
+        if (loc[t] < capacity && idx[t] >= 0) {                                        \
+            const T *src = dispatched + ((int64_t)idx[t] * capacity + loc[t]) * hidden;\
+            const T g = gate[t];                                                       \
+            for (int j = 0; j < hidden; ++j) dst[j] = g * src[j];                      \
+        } else {                                                                       \
+            for (int j = 0; j < hidden; ++j) dst[j] = 0;                               \
+        }                                                                              \
+    }                                                                                  \
+}
+DEF_GATHER(orc_gather_f32, float)
+DEF_GATHER(orc_gather_f64, double)
+
+/* kernel_type 2: grad_gate[token] = <dispatched[slot], x[token]>, sequential sum in T
+ * (custom_kernel.cpp:98-111) */
+#define DEF_BWD_GATE(NAME, T)                                                          \
+ORC_API void NAME(T *grad_gate, const int32_t *idx, const int32_t *loc, const T *x,   \
+                  const T *dispatched, int samples, int hidden, int capacity)          \
+{                                                                                      \
+    for (int t = 0; t < samples; ++t) {                                                \
+        T acc = 0;                                                                     \
+        if (loc[t] < capacity && idx[t] >= 0) {                                        \
+            const T *a = dispatched + ((int64_t)idx[t] * capacity + loc[t]) * hidden;  \
+            const T *b = x + (int64_t)t * hidden;                                      \
+            for (int j = 0; j < hidden; ++j) acc += a[j] * b[j];                       \
+        }                                                                              \
+        grad_gate[t] = acc;                                                            \
+    }                                                                                  \
+}
+DEF_BWD_GATE(orc_bwd_gate_f32, float)
+DEF_BWD_GATE(orc_bwd_gate_f64, double)
+
+/* ------------------------------------------------------------------ capacity cumsum
+ * jit_kernels/gating.py:13-22 and custom_kernel.cpp:331-383: column-wise inclusive
+ * prefix sum minus one of an int [samples, cols] matrix. */
+ORC_API void orc_cumsum_sub_one(const int32_t *in, int32_t *out, int samples, int cols)
+{
+    for (int c = 0; c < cols; ++c) {
+        int32_t run = -1;
+        for (int t = 0; t < samples; ++t) {
+            run += in[(int64_t)t * cols + c];
+            out[(int64_t)t * cols + c] = run;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ routing
+ * impls/fast_dispatch.py:140-195 (extract_critical) with impls/losses.py:7-19.
+ *
+ * scores: [samples, experts] row-major, fp32 (is_bf16 = 0) or bf16 bit patterns in
+ * uint16 (is_bf16 = 1).  Outputs are k planes of [samples]:
+ *   indices[j][t]   expert of the j-th largest score of token t       (:143-145,174)
+ *   locations[j][t] slot inside that expert: first choices of an expert take slots in
+ *                   token order, then second choices, ...               (:156-168)
+ *   gates[j][t]     scores[t, indices[j][t]], divided by clamp(sum_j, eps) when
+ *                   normalize and k > 1; every step rounded in the scores dtype (:148,170-172)
+ * counts[j][e]     number of tokens whose j-th choice is e (what mask_j.sum(0) holds, :164)
+ * Ties between equal scores are resolved towards the lower expert index; torch.topk
+ * leaves that order unspecified, so parity on indices is only defined for tie-free rows.
+ */
+static inline float load_score(const void *scores, int is_bf16, int64_t i)
+{
+    return is_bf16 ? bf16_to_f32(((const uint16_t *)scores)[i]) : ((const float *)scores)[i];
+}
+
+ORC_API void orc_route_topk(const void *scores, int is_bf16, int samples, int experts, int top_k,
+                            int normalize_gate, int32_t *indices, int32_t *locations,
+                            void *gates, int32_t *counts)
+{
+    int k = top_k < experts ? top_k : experts;
+    int64_t *seen = (int64_t *)calloc((size_t)experts, sizeof(int64_t));
+    uint8_t *taken = (uint8_t *)malloc((size_t)experts);
+    float *g = (float *)malloc(sizeof(float) * (size_t)k);
+    memset(counts, 0, sizeof(int32_t) * (size_t)k * experts);
+
+    for (int t = 0; t < samples; ++t) {
+        memset(taken, 0, (size_t)experts);
+        for (int j = 0; j < k; ++j) {
+            int best = -1;
+            float bv = 0.f;
+            for (int e = 0; e < experts; ++e) {
+                if (taken[e]) continue;
+                float v = load_score(scores, is_bf16, (int64_t)t * experts + e);
+                if (best < 0 || v > bv) { best = e; bv = v; }
+            }
+            taken[best] = 1;
+            indices[(int64_t)j * samples + t] = best;
+            g[j] = bv;
+            counts[j * experts + best] += 1;
+        }
+        if (k > 1 && normalize_gate) {
+            /* python sum(): ((0 + g0) + g1) + ...; clamp(min = eps of the dtype); divide */
+            float denom = g[0];
+            for (int j = 1; j < k; ++j) { denom = denom + g[j]; if (is_bf16) denom = rbf(denom); }
+            float eps = is_bf16 ? 0.0078125f : FLT_EPSILON;
+            if (denom < eps) denom = eps;
+            for (int j = 0; j < k; ++j) { g[j] = g[j] / denom; if (is_bf16) g[j] = rbf(g[j]); }
+        }
+        for (int j = 0; j < k; ++j) {
+            if (is_bf16) ((uint16_t *)gates)[(int64_t)j * samples + t] = f32_to_bf16(g[j]);
+            else ((float *)gates)[(int64_t)j * samples + t] = g[j];
+        }
+    }
+    /* slot numbers: running count per expert, choice plane after choice plane */
+    for (int j = 0; j < k; ++j) {
+        for (int t = 0; t < samples; ++t) {
+            int e = indices[(int64_t)j * samples + t];
+            locations[(int64_t)j * samples + t] = (int32_t)seen[e];
+            seen[e] += 1;
+        }
+    }
+    free(seen); free(taken); free(g);
+}
+
+/* capacity closed form, capacity_factor > 0 branch plus alignment round-up
+ * (fast_dispatch.py:179-190) */
+ORC_API int orc_capacity(int samples, int experts, int top_k, double capacity_factor, int alignment)
+{
+    int k = top_k < experts ? top_k : experts;
+    int per_expert = (samples + experts - 1) / experts;
+    int cap = k * (int)(capacity_factor * per_expert);
+    int rem = cap % alignment;
+    if (rem > 0) cap += alignment - rem;
+    return cap;
+}
+
+/* GShard auxiliary loss (losses.py:12-19) evaluated in double: sum_e(me[e]*ce[e]) / T with
+ * me = column sums of scores and ce = (E/T) * #first-choices of e.  Tolerance-level pin. */
+ORC_API double orc_gshard_loss(const void *scores, int is_bf16, const int32_t *first_choice,
+                               int samples, int experts)
+{
+    double *me = (double *)calloc((size_t)experts, sizeof(double));
+    double *ce = (double *)calloc((size_t)experts, sizeof(double));
+    for (int t = 0; t < samples; ++t) {
+        for (int e = 0; e < experts; ++e)
+            me[e] += load_score(scores, is_bf16, (int64_t)t * experts + e);
+        ce[first_choice[t]] += (double)experts / samples;
+    }
+    double s = 0;
+    for (int e = 0; e < experts; ++e) s += me[e] * ce[e];
+    free(me); free(ce);
+    return s / samples;
+}
+
+/* softmax over the expert axis (impls/moe_layer.py:239), double math rounded to float.
+ * Tolerance-level pin only: torch's vectorised expf is not bit-defined. */
+ORC_API void orc_softmax_f32(const float *logits, float *scores, int samples, int experts)
+{
+    for (int t = 0; t < samples; ++t) {
+        const float *l = logits + (int64_t)t * experts;
+        float m = l[0];
+        for (int e = 1; e < experts; ++e) if (l[e] > m) m = l[e];
+        double s = 0;
+        for (int e = 0; e < experts; ++e) s += exp((double)l[e] - m);
+        for (int e = 0; e < experts; ++e)
+            scores[(int64_t)t * experts + e] = (float)(exp((double)l[e] - m) / s);
+    }
+}
+
+/* gate logits x[T,M] . wg[E,M]^T (gates/top.py:20-26), double accumulation.
+ * is_bf16 selects bf16 bit patterns for both operands. */
+ORC_API void orc_gate_logits(const void *x, const void *wg, int is_bf16, double *logits,
+                             int samples, int model_dim, int experts)
+{
+    for (int t = 0; t < samples; ++t)
+        for (int e = 0; e < experts; ++e) {
+            double acc = 0;
+            for (int m = 0; m < model_dim; ++m)
+                acc += (double)load_score(x, is_bf16, (int64_t)t * model_dim + m) *
+                       (double)load_score(wg, is_bf16, (int64_t)e * model_dim + m);
+            logits[(int64_t)t * experts + e] = acc;
+        }
+}
+
+/* ------------------------------------------------------------------ "int8" codec
+ * custom/compressor/int8.cpp:10-16 (compress) and :55-58 (decompress).
+ * Per row: bias = min, scale = max - min, code = uint8(((x - bias) / scale) * 255), three
+ * separately rounded ops in the tensor's dtype.  A row with scale == 0 gives 0/0 = NaN,
+ * which torch-CPU converts to code 0. */
+static inline uint8_t to_u8(float q)
+{
+    if (!(q == q)) return 0;
+    if (q <= 0.f) return 0;
+    if (q >= 255.f) return 255;
+    return (uint8_t)q;
+}
+
+ORC_API void orc_int8_compress_f32(const float *x, int64_t rows, int row_len, uint8_t *codes,
+                                   float *bias, float *scale)
+{
+    for (int64_t r = 0; r < rows; ++r) {
+        const float *p = x + r * row_len;
+        float mn = p[0], mx = p[0];
+        for (int j = 1; j < row_len; ++j) { if (p[j] < mn) mn = p[j]; if (p[j] > mx) mx = p[j]; }
+        float sc = mx - mn;
+        bias[r] = mn; scale[r] = sc;
+        for (int j = 0; j < row_len; ++j) {
+            float d = p[j] - mn;
+            float q = d / sc;
+            float m = q * 255.0f;
+            codes[r * row_len + j] = to_u8(m);
+        }
+    }
+}
+
+ORC_API void orc_int8_compress_bf16(const uint16_t *x, int64_t rows, int row_len, uint8_t *codes,
+                                    uint16_t *bias, uint16_t *scale)
+{
+    for (int64_t r = 0; r < rows; ++r) {
+        const uint16_t *p = x + r * row_len;
+        float mn = bf16_to_f32(p[0]), mx = mn;
+        for (int j = 1; j < row_len; ++j) {
+            float v = bf16_to_f32(p[j]);
+            if (v < mn) mn = v;
+            if (v > mx) mx = v;
+        }
+        float sc = rbf(mx - mn);
+        bias[r] = f32_to_bf16(mn); scale[r] = f32_to_bf16(sc);
+        for (int j = 0; j < row_len; ++j) {
+            float d = rbf(bf16_to_f32(p[j]) - mn);
+            float q = rbf(d / sc);
+            float m = rbf(q * 255.0f);
+            codes[r * row_len + j] = to_u8(m);
+        }
+    }
+}
+
+/* out = ((code / 255) * scale) + bias, each op rounded in the dtype (int8.cpp:55-58);
+ * division is a true division as on torch-CPU */
+ORC_API void orc_int8_decompress_f32(const uint8_t *codes, const float *bias, const float *scale,
+                                     int64_t rows, int row_len, float *out)
+{
+    for (int64_t r = 0; r < rows; ++r)
+        for (int j = 0; j < row_len; ++j) {
+            float v = (float)codes[r * row_len + j];
+            v = v / 255.0f;
+            v = v * scale[r];
+            v = v + bias[r];
+            out[r * row_len + j] = v;
+        }
+}
+
+ORC_API void orc_int8_decompress_bf16(const uint8_t *codes, const uint16_t *bias,
+                                      const uint16_t *scale, int64_t rows, int row_len,
+                                      uint16_t *out)
+{
+    for (int64_t r = 0; r < rows; ++r) {
+        float b = bf16_to_f32(bias[r]), s = bf16_to_f32(scale[r]);
+        for (int j = 0; j < row_len; ++j) {
+            float v = (float)codes[r * row_len + j];     /* exact in bf16 (<= 8 bits) */
+            v = rbf(v / 255.0f);
+            v = rbf(v * s);
+            v = rbf(v + b);
+            out[r * row_len + j] = f32_to_bf16(v);
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ zfp fixed-rate codec
+ * The reference calls the third-party zfp library (custom/compressor/zfpc.cpp:31-51 and
+ * :66-84; not vendored, version unpinned).  This is a restatement of the published zfp
+ * 0.5.5 fixed-rate float codec for 1-D and 2-D fields: block-floating-point cast, the
+ * decorrelating lifting transform, negabinary reordering and the embedded group-tested
+ * bit-plane coder, written to a header-less stream of 64-bit little-endian words.
+ * The reference uses dims = 2 with nx = model_dim, ny = experts*capacity (zfpc.cpp:32-37).
+ */
+typedef struct { uint8_t *base; uint64_t bitpos; } bitw_t;
+
+static inline void put_bit(bitw_t *w, uint32_t b)
+{
+    if (b) w->base[w->bitpos >> 3] |= (uint8_t)(1u << (w->bitpos & 7));
+    w->bitpos++;
+}
+static inline void put_bits(bitw_t *w, uint64_t v, int n)
+{
+    for (int i = 0; i < n; ++i) put_bit(w, (uint32_t)((v >> i) & 1u));
+}
+static inline uint32_t get_bit(const uint8_t *base, uint64_t *pos)
+{
+    uint32_t b = (base[*pos >> 3] >> (*pos & 7)) & 1u;
+    (*pos)++;
+    return b;
+}
+
+static void fwd_lift(int32_t *p, int s)
+{
+    int32_t x = p[0], y = p[s], z = p[2 * s], w = p[3 * s];
+    x += w; x >>= 1; w -= x;
+    z += y; z >>= 1; y -= z;
+    x += z; x >>= 1; z -= x;
+    w += y; w >>= 1; y -= w;
+    w += y >> 1; y -= w >> 1;
+    p[0] = x; p[s] = y; p[2 * s] = z; p[3 * s] = w;
+}
+static void inv_lift(int32_t *p, int s)
+{
+    int32_t x = p[0], y = p[s], z = p[2 * s], w = p[3 * s];
+    y += w >> 1; w -= y >> 1;
+    y += w; w = (int32_t)((uint32_t)w << 1); w -= y;
+    z += x; x = (int32_t)((uint32_t)x << 1); x -= z;
+    y += z; z = (int32_t)((uint32_t)z << 1); z -= y;
+    w += x; x = (int32_t)((uint32_t)x << 1); x -= w;
+    p[0] = x; p[s] = y; p[2 * s] = z; p[3 * s] = w;
+}
+
+static const uint8_t PERM1[4] = {0, 1, 2, 3};
+static const uint8_t PERM2[16] = {0, 1, 4, 5, 2, 8, 6, 9, 3, 12, 10, 7, 13, 11, 14, 15};
+
+static int zfp_maxbits(int dims, double rate)
+{
+    int n = dims == 1 ? 4 : 16;
+    int bits = (int)floor(n * rate + 0.5);
+    if (bits < 1 + 8) bits = 1 + 8;
+    return bits;
+}
+
+static void zfp_encode_block(bitw_t *w, const float *f, int dims, int maxbits)
+{
+    const int n = dims == 1 ? 4 : 16;
+    const uint8_t *perm = dims == 1 ? PERM1 : PERM2;
+    const uint64_t start = w->bitpos;
+    float m = 0.f;
+    for (int i = 0; i < n; ++i) { float a = fabsf(f[i]); if (a > m) m = a; }
+    int emax = -127;
+    if (m > 0.f) { int e; frexpf(m, &e); emax = e > -126 ? e : -126; }
+    int prec = emax + 1074 + 2 * (dims + 1);
+    if (prec > 64) prec = 64;
+    if (prec < 0) prec = 0;
+    uint32_t e = prec ? (uint32_t)(emax + 127) : 0u;
+    if (!e) { w->bitpos = start + (uint64_t)maxbits; return; }   /* '0' flag + zero padding */
+    put_bits(w, 2u * e + 1u, 9);
+
+    int32_t q[16];
+    float s = ldexpf(1.0f, 30 - emax);
+    for (int i = 0; i < n; ++i) {
+        float v = f[i] * s;
+        /* out-of-range products take the x86 conversion result (INT_MIN) */
+        q[i] = (v >= 2147483648.0f || v < -2147483648.0f || v != v) ? INT32_MIN : (int32_t)v;
+    }
+    if (dims == 1) fwd_lift(q, 1);
+    else {
+        for (int y = 0; y < 4; ++y) fwd_lift(q + 4 * y, 1);
+        for (int x = 0; x < 4; ++x) fwd_lift(q + x, 4);
+    }
+    uint32_t u[16];
+    for (int i = 0; i < n; ++i)
+        u[i] = ((uint32_t)q[perm[i]] + 0xaaaaaaaau) ^ 0xaaaaaaaau;
+
+    int bits = maxbits - 9;
+    int kmin = prec >= 32 ? 0 : 32 - prec;
+    int nsig = 0;
+    for (int k = 31; bits > 0 && k >= kmin; --k) {
+        uint64_t x = 0;
+        for (int i = 0; i < n; ++i) x += (uint64_t)((u[i] >> k) & 1u) << i;
+        int mm = nsig < bits ? nsig : bits;
+        bits -= mm;
+        put_bits(w, x, mm);
+        x >>= mm;
+        while (nsig < n && bits > 0) {
+            bits--; put_bit(w, x != 0);
+            if (x == 0) break;
+            while (nsig < n - 1 && bits > 0) {
+                bits--; put_bit(w, (uint32_t)(x & 1u));
+                if (x & 1u) break;
+                x >>= 1; nsig++;
+            }
+            x >>= 1; nsig++;
+        }
+    }
+    w->bitpos = start + (uint64_t)maxbits;
+}
+
+static void zfp_decode_block(const uint8_t *base, uint64_t start, float *f, int dims, int maxbits)
+{
+    const int n = dims == 1 ? 4 : 16;
+    const uint8_t *perm = dims == 1 ? PERM1 : PERM2;
+    uint64_t pos = start;
+    if (!get_bit(base, &pos)) { for (int i = 0; i < n; ++i) f[i] = 0.f; return; }
+    uint32_t e = 0;
+    for (int i = 0; i < 8; ++i) e |= get_bit(base, &pos) << i;
+    int emax = (int)e - 127;
+    int prec = emax + 1074 + 2 * (dims + 1);
+    if (prec > 64) prec = 64;
+    int kmin = prec >= 32 ? 0 : 32 - prec;
+    uint32_t u[16];
+    for (int i = 0; i < n; ++i) u[i] = 0;
+    int bits = maxbits - 9;
+    int nsig = 0;
+    for (int k = 31; bits > 0 && k >= kmin; --k) {
+        int mm = nsig < bits ? nsig : bits;
+        bits -= mm;
+        uint64_t x = 0;
+        for (int i = 0; i < mm; ++i) x |= (uint64_t)get_bit(base, &pos) << i;
+        while (nsig < n && bits > 0) {
+            bits--;
+            if (!get_bit(base, &pos)) break;
+            while (nsig < n - 1 && bits > 0) {
+                bits--;
+                if (get_bit(base, &pos)) break;
+                nsig++;
+            }
+            x += (uint64_t)1 << nsig;
+            nsig++;
+        }
+        for (int i = 0; x; ++i, x >>= 1) u[i] += (uint32_t)(x & 1u) << k;
+    }
+    int32_t q[16];
+    for (int i = 0; i < n; ++i)
+        q[perm[i]] = (int32_t)((u[i] ^ 0xaaaaaaaau) - 0xaaaaaaaau);
+    if (dims == 1) inv_lift(q, 1);
+    else {
+        for (int x = 0; x < 4; ++x) inv_lift(q + x, 4);
+        for (int y = 0; y < 4; ++y) inv_lift(q + 4 * y, 1);
+    }
+    float s = ldexpf(1.0f, emax - 30);
+    for (int i = 0; i < n; ++i) f[i] = (float)q[i] * s;
+}
+
+/* bytes zfp_stream_maximum_size reports for a float field (header allowance + whole words) */
+ORC_API uint64_t orc_zfp_max_bytes(int dims, int64_t nx, int64_t ny, double rate)
+{
+    int64_t blocks = dims == 1 ? (nx * ny + 3) / 4 : ((nx + 3) / 4) * ((ny + 3) / 4);
+    uint64_t bits = 148u + (uint64_t)blocks * (uint64_t)zfp_maxbits(dims, rate);
+    return ((bits + 63u) / 64u) * 8u;
+}
+
+/* payload bytes of a fixed-rate stream (what zfp_compress returns after flushing) */
+ORC_API uint64_t orc_zfp_stream_bytes(int dims, int64_t nx, int64_t ny, double rate)
+{
+    int64_t blocks = dims == 1 ? (nx * ny) / 4 : (nx / 4) * (ny / 4);
+    uint64_t bits = (uint64_t)blocks * (uint64_t)zfp_maxbits(dims, rate);
+    return ((bits + 63u) / 64u) * 8u;
+}
+
+/* field: ny rows of nx floats (nx fastest).  dims = 1 treats it as one array of nx*ny.
+ * nx and ny must be multiples of 4 (zfpc.cpp:26-28).  out must be zero-initialised and hold
+ * orc_zfp_stream_bytes(). */
+ORC_API int orc_zfp_compress(const float *field, int dims, int64_t nx, int64_t ny, double rate,
+                             uint8_t *out)
+{
+    const int maxbits = zfp_maxbits(dims, rate);
+    bitw_t w = {out, 0};
+    if (dims == 1) {
+        int64_t n = nx * ny;
+        if (n % 4) return -1;
+        for (int64_t b = 0; b < n / 4; ++b) zfp_encode_block(&w, field + 4 * b, 1, maxbits);
+    } else {
+        if (nx % 4 || ny % 4) return -1;
+        for (int64_t by = 0; by < ny / 4; ++by)
+            for (int64_t bx = 0; bx < nx / 4; ++bx) {
+                float blk[16];
+                for (int j = 0; j < 4; ++j)
+                    for (int i = 0; i < 4; ++i)
+                        blk[i + 4 * j] = field[(4 * by + j) * nx + 4 * bx + i];
+                zfp_encode_block(&w, blk, 2, maxbits);
+            }
+    }
+    return 0;
+}
+
+ORC_API int orc_zfp_decompress(const uint8_t *in, int dims, int64_t nx, int64_t ny, double rate,
+                               float *field)
+{
+    const int maxbits = zfp_maxbits(dims, rate);
+    if (dims == 1) {
+        int64_t n = nx * ny;
+        if (n % 4) return -1;
+        for (int64_t b = 0; b < n / 4; ++b)
+            zfp_decode_block(in, (uint64_t)b * maxbits, field + 4 * b, 1, maxbits);
+    } else {
+        if (nx % 4 || ny % 4) return -1;
+        int64_t b = 0;
+        for (int64_t by = 0; by < ny / 4; ++by)
+            for (int64_t bx = 0; bx < nx / 4; ++bx, ++b) {
+                float blk[16];
+                zfp_decode_block(in, (uint64_t)b * maxbits, blk, 2, maxbits);
+                for (int j = 0; j < 4; ++j)
+                    for (int i = 0; i < 4; ++i)
+                        field[(4 * by + j) * nx + 4 * bx + i] = blk[i + 4 * j];
+            }
+    }
+    return 0;
+}

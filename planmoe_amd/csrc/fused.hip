@@ -1,0 +1,199 @@
+// Dispatch fused with the "int8" codec: token rows go straight to uint8 codes in their
+// capacity slots, so the [experts*capacity, model_dim] tensor that fast_encode would hand to
+// Compress.apply (impls/moe_layer.py:265, impls/overlap.py:12-16, int8.cpp:10-24) never
+// exists in memory.  One wavefront owns one token: the row is read once into registers,
+// reduced to min/max across lanes, quantised, and the codes are written to every live slot
+// of the token.  With the all-ones gate helper every choice shares one set of codes.
+#include "rows.hpp"
+#include "int8_core.hpp"
+
+namespace pm {
+
+// CACHE = 16-byte vectors per lane held in registers (0: re-read the row from cache)
+template <int DT, int CACHE>
+__global__ __launch_bounds__(256) void dispatch_int8_kernel(
+    const void *__restrict__ x, const float *__restrict__ gates,
+    const int32_t *__restrict__ indices, const int32_t *__restrict__ locations, int64_t stride,
+    int top_k, int samples, int model_dim, int experts, int capacity,
+    uint8_t *__restrict__ codes, void *__restrict__ bias_out, void *__restrict__ scale_out,
+    const uint32_t *__restrict__ flags, int token_blocks)
+{
+    using E = Elem<DT>;
+    constexpr int V = E::VEC;
+    const int wave = threadIdx.x >> 6, lane = lane_id();
+    const int units = model_dim / V;
+
+    if ((int)blockIdx.x >= token_blocks) {
+        // slots no live pair addresses: all-zero row -> codes 0, bias 0, scale 0
+        const int slots = experts * capacity;
+        const int nwaves = (gridDim.x - token_blocks) * 4;
+        for (int s = (blockIdx.x - token_blocks) * 4 + wave; s < slots; s += nwaves) {
+            if (flags[s]) continue;
+            uint8_t *row = codes + (int64_t)s * model_dim;
+            for (int u = lane; u < units; u += WAVE) {
+                if constexpr (V == 8) reinterpret_cast<uint2 *>(row)[u] = make_uint2(0u, 0u);
+                else reinterpret_cast<uint32_t *>(row)[u] = 0u;
+            }
+            if (lane == 0) { E::store(bias_out, s, 0.f); E::store(scale_out, s, 0.f); }
+        }
+        return;
+    }
+
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= samples) return;
+    const uint4 *src = reinterpret_cast<const uint4 *>((const char *)x + (int64_t)t * model_dim * (int64_t)sizeof(typename E::store_t));
+
+    uint4 cache[CACHE > 0 ? CACHE : 1];
+    if constexpr (CACHE > 0) {
+#pragma unroll
+        for (int c = 0; c < CACHE; ++c) {
+            const int u = c * WAVE + lane;
+            if (u < units) cache[c] = src[u];
+        }
+    }
+
+    // the row as the dispatcher would store it for gate g: round(0 + g * x)
+    auto reduce = [&](float g, float &mn, float &mx) {
+        mn = INFINITY; mx = -INFINITY;
+        auto visit = [&](const uint4 &raw) {
+            float f[V];
+            E::unpack(raw, f);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                const float d = E::round(0.f + g * f[i]);
+                mn = nan_min(mn, d); mx = nan_max(mx, d);
+            }
+        };
+        if constexpr (CACHE > 0) {
+#pragma unroll
+            for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) visit(cache[c]);
+        } else {
+            for (int u = lane; u < units; u += WAVE) visit(src[u]);
+        }
+        mn = wave_allreduce(mn, [](float a, float b) { return nan_min(a, b); });
+        mx = wave_allreduce(mx, [](float a, float b) { return nan_max(a, b); });
+    };
+    auto encode = [&](const uint4 &raw, float g, float mn, float scale, uint32_t *w) {
+        float f[V];
+        E::unpack(raw, f);
+#pragma unroll
+        for (int i = 0; i < V; ++i) f[i] = E::round(0.f + g * f[i]);
+#pragma unroll
+        for (int i = 0; i < V / 4; ++i)
+            w[i] = quantise<DT>(f[4 * i], mn, scale) | (quantise<DT>(f[4 * i + 1], mn, scale) << 8) |
+                   (quantise<DT>(f[4 * i + 2], mn, scale) << 16) | (quantise<DT>(f[4 * i + 3], mn, scale) << 24);
+    };
+    auto put = [&](int s, int u, const uint32_t *w) {
+        uint8_t *row = codes + (int64_t)s * model_dim;
+        if constexpr (V == 8) reinterpret_cast<uint2 *>(row)[u] = make_uint2(w[0], w[1]);
+        else reinterpret_cast<uint32_t *>(row)[u] = w[0];
+    };
+
+    for (int j0 = 0; j0 < top_k; j0 += WAVE) {
+        const int np = min(top_k - j0, WAVE);
+        int slot; float gate;
+        fetch_planes(gates, indices, locations, stride, t, j0, np, experts, capacity, slot, gate);
+        if (__ballot(slot >= 0) == 0) continue;
+
+        if (!gates) {
+            // one code row shared by all live choices
+            float mn, mx;
+            reduce(1.f, mn, mx);
+            const float scale = E::round(mx - mn);
+            if (lane < np && slot >= 0) { E::store(bias_out, slot, mn); E::store(scale_out, slot, scale); }
+            auto emit = [&](int u, const uint4 &raw) {
+                uint32_t w[2];
+                encode(raw, 1.f, mn, scale, w);
+                for (int j = 0; j < np; ++j) {
+                    const int s = rl_i(slot, j);
+                    if (s >= 0) put(s, u, w);
+                }
+            };
+            if constexpr (CACHE > 0) {
+#pragma unroll
+                for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) emit(c * WAVE + lane, cache[c]);
+            } else {
+                for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
+            }
+        } else {
+            for (int j = 0; j < np; ++j) {
+                const int s = rl_i(slot, j);
+                if (s < 0) continue;
+                const float g = rl_f(gate, j);
+                float mn, mx;
+                reduce(g, mn, mx);
+                const float scale = E::round(mx - mn);
+                if (lane == 0) { E::store(bias_out, s, mn); E::store(scale_out, s, scale); }
+                auto emit = [&](int u, const uint4 &raw) {
+                    uint32_t w[2];
+                    encode(raw, g, mn, scale, w);
+                    put(s, u, w);
+                };
+                if constexpr (CACHE > 0) {
+#pragma unroll
+                    for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) emit(c * WAVE + lane, cache[c]);
+                } else {
+                    for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
+                }
+            }
+        }
+    }
+}
+
+template <int DT>
+static void launch_dispatch_int8(int per_lane, unsigned grid, hipStream_t st, const void *x,
+                                 const float *gates, const int32_t *indices, const int32_t *locations,
+                                 int64_t stride, int top_k, int samples, int model_dim, int experts,
+                                 int capacity, uint8_t *codes, void *bias, void *scale,
+                                 const uint32_t *flags, int token_blocks)
+{
+#define PM_DI8(CACHE)                                                                            \
+    dispatch_int8_kernel<DT, CACHE><<<grid, 256, 0, st>>>(x, gates, indices, locations, stride,  \
+        top_k, samples, model_dim, experts, capacity, codes, bias, scale, flags, token_blocks)
+    if (per_lane <= 2) PM_DI8(2);
+    else if (per_lane <= 4) PM_DI8(4);
+    else if (per_lane <= 8) PM_DI8(8);
+    else if (per_lane <= 16) PM_DI8(16);
+    else PM_DI8(0);
+#undef PM_DI8
+}
+
+} // namespace pm
+
+using namespace pm;
+
+extern "C" int planmoe_dispatch_int8(const void *x, int dtype, const float *gates,
+                                     const int32_t *indices, const int32_t *locations,
+                                     int64_t plane_stride, int top_k, int samples, int model_dim,
+                                     int experts, int capacity, uint8_t *codes, void *bias,
+                                     void *scale, void *workspace, size_t workspace_bytes,
+                                     void *stream)
+{
+    if (check_planes("planmoe_dispatch_int8", indices, locations, plane_stride, top_k, samples)) return 1;
+    PM_REQUIRE(dtype_ok(dtype), "planmoe_dispatch_int8: bad dtype %d", dtype);
+    PM_REQUIRE(model_dim >= 1 && experts >= 1 && capacity >= 0, "planmoe_dispatch_int8: bad shape");
+    PM_REQUIRE((int64_t)experts * capacity < (1ll << 31), "planmoe_dispatch_int8: experts*capacity overflows int32");
+    PM_REQUIRE((int64_t)samples * top_k < (1ll << 31), "planmoe_dispatch_int8: samples*top_k overflows int32");
+    const int slots = experts * capacity;
+    if (slots == 0) return 0;
+    PM_REQUIRE(x || samples == 0, "planmoe_dispatch_int8: x is NULL");
+    PM_REQUIRE(codes && bias && scale, "planmoe_dispatch_int8: NULL output");
+    PM_REQUIRE(workspace && workspace_bytes >= planmoe_dispatch_workspace_bytes(experts, capacity),
+               "planmoe_dispatch_int8: workspace too small");
+    const int vec = dtype == PLANMOE_F32 ? 4 : 8;
+    PM_REQUIRE(model_dim % vec == 0 && aligned16(x) && ((uintptr_t)codes % 8 == 0),
+               "planmoe_dispatch_int8: model_dim must be a multiple of %d and buffers 16-byte aligned; "
+               "use planmoe_dispatch_fwd + planmoe_int8_compress otherwise", vec);
+    hipStream_t st = (hipStream_t)stream;
+    uint32_t *flags = (uint32_t *)workspace;
+    launch_slot_flags(flags, indices, locations, plane_stride, top_k, samples, experts, capacity, st);
+    const int token_blocks = (samples + 3) / 4;
+    const int fill_blocks = min((slots + 3) / 4, 2048);
+    const int per_lane = (model_dim / vec + WAVE - 1) / WAVE;
+    PM_DTYPE_SWITCH(dtype, DT,
+        launch_dispatch_int8<DT>(per_lane, (unsigned)(token_blocks + fill_blocks), st, x, gates, indices,
+                                 locations, plane_stride, top_k, samples, model_dim, experts, capacity,
+                                 codes, bias, scale, flags, token_blocks));
+    PM_LAUNCH_CHECK("planmoe_dispatch_int8");
+    return 0;
+}

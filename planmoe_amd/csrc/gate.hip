@@ -1,0 +1,91 @@
+// Gate logits: logits[T, E] = x[T, M] . wg[E, M]^T  (gates/top.py:20-26).
+//
+// The GEMM is skinny (E is 2..64) and bound by reading x once from HBM; the matrix cores
+// (MFMA 16x16 tiles, fp32 accumulation) keep the arithmetic off the critical path.
+// A work-group of 4 waves owns 16*TPW tokens; the K axis is dealt to the 4 waves in 16-vector
+// steps (round robin, so the group streams 1 KB of every token row at a time) and the 4
+// partial tiles meet in LDS, summed in a fixed order.  Both MFMA operands use the same
+// lane -> k mapping, chosen so that each lane reads 64 contiguous bytes of its row per step.
+#include "gate_core.hpp"
+
+namespace pm {
+
+template <int DT, int NT, int TPW>
+__global__ __launch_bounds__(256) void gate_logits_kernel(
+    const void *__restrict__ x, const void *__restrict__ wg, void *__restrict__ logits, int out_dt,
+    int samples, int model_dim, int experts)
+{
+    __shared__ float part[4][16 * TPW][16 * NT + 1];
+    const int t0 = blockIdx.x * 16 * TPW;
+    gate_tile_partials<DT, NT, TPW>(x, wg, t0, samples, model_dim, experts, part);
+    __syncthreads();
+    for (int i = threadIdx.x; i < 16 * TPW * experts; i += 256) {
+        const int r = i / experts, e = i - r * experts;
+        const int t = t0 + r;
+        if (t >= samples) continue;
+        const float v = ((part[0][r][e] + part[1][r][e]) + part[2][r][e]) + part[3][r][e];
+        const int64_t o = (int64_t)t * experts + e;
+        if (out_dt == PLANMOE_F32) ((float *)logits)[o] = v;
+        else if (out_dt == PLANMOE_BF16) ((uint16_t *)logits)[o] = (uint16_t)f32_to_bf16(v);
+        else ((uint16_t *)logits)[o] = (uint16_t)f32_to_f16(v);
+    }
+}
+
+// any shape / alignment: one thread per logit
+template <int DT>
+__global__ __launch_bounds__(256) void gate_logits_naive_kernel(
+    const void *__restrict__ x, const void *__restrict__ wg, void *__restrict__ logits, int out_dt,
+    int samples, int model_dim, int experts)
+{
+    using E = Elem<DT>;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)samples * experts) return;
+    const int64_t t = i / experts; const int e = (int)(i - t * experts);
+    float acc = 0.f;
+    for (int m = 0; m < model_dim; ++m)
+        acc = fmaf(E::load(x, t * model_dim + m), E::load(wg, (int64_t)e * model_dim + m), acc);
+    if (out_dt == PLANMOE_F32) ((float *)logits)[i] = acc;
+    else if (out_dt == PLANMOE_BF16) ((uint16_t *)logits)[i] = (uint16_t)f32_to_bf16(acc);
+    else ((uint16_t *)logits)[i] = (uint16_t)f32_to_f16(acc);
+}
+
+template <int DT>
+static void launch_gate_logits(const void *x, const void *wg, void *logits, int out_dt, int samples,
+                               int model_dim, int experts, bool mfma, hipStream_t st)
+{
+    if (!mfma) {
+        const int64_t n = (int64_t)samples * experts;
+        gate_logits_naive_kernel<DT><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(x, wg, logits, out_dt,
+                                                                                 samples, model_dim, experts);
+        return;
+    }
+#define PM_GATE(NT, TPW)                                                                     \
+    gate_logits_kernel<DT, NT, TPW><<<(samples + 16 * TPW - 1) / (16 * TPW), 256, 0, st>>>(  \
+        x, wg, logits, out_dt, samples, model_dim, experts)
+    if (experts <= 16) PM_GATE(1, 2);
+    else if (experts <= 32) PM_GATE(2, 2);
+    else PM_GATE(4, 2);
+#undef PM_GATE
+}
+
+} // namespace pm
+
+using namespace pm;
+
+extern "C" int planmoe_gate_logits(const void *x, const void *wg, int dtype, void *logits,
+                                   int out_dtype, int samples, int model_dim, int experts,
+                                   void *stream)
+{
+    PM_REQUIRE(dtype_ok(dtype) && dtype_ok(out_dtype), "planmoe_gate_logits: bad dtype");
+    PM_REQUIRE(out_dtype == PLANMOE_F32 || out_dtype == dtype,
+               "planmoe_gate_logits: out_dtype must be F32 or the input dtype");
+    PM_REQUIRE(samples >= 0 && model_dim >= 1 && experts >= 1, "planmoe_gate_logits: bad shape");
+    if (samples == 0) return 0;
+    PM_REQUIRE(x && wg && logits, "planmoe_gate_logits: NULL argument");
+    const int vec = dtype == PLANMOE_F32 ? 4 : 8;
+    const bool mfma = experts <= 64 && model_dim % vec == 0 && aligned16(x) && aligned16(wg);
+    PM_DTYPE_SWITCH(dtype, DT, launch_gate_logits<DT>(x, wg, logits, out_dtype, samples, model_dim,
+                                                      experts, mfma, (hipStream_t)stream));
+    PM_LAUNCH_CHECK("planmoe_gate_logits");
+    return 0;
+}

@@ -1,0 +1,452 @@
+// Top-k routing with capacity-slot assignment, and the stand-alone capacity cumsum.
+//
+// planmoe_route_topk takes the place of extract_critical (impls/fast_dispatch.py:140-195):
+// about 25 ATen launches over [samples, experts] one-hot matrices plus the E-block
+// Blelloch scan of custom_kernel.cpp:339-376 become three launches that never build a
+// one-hot matrix:
+//   route_tile_kernel   one thread per token, 256 tokens per tile: softmax (optional),
+//                       k-fold arg-max, rank of the token among the tile's tokens that
+//                       chose the same expert (wave ballots + an LDS table), per-tile
+//                       expert histograms and per-tile column sums of the scores
+//   route_scan_kernel   exclusive prefix of the histograms over tiles, choice plane after
+//                       choice plane, so that all first choices precede all second choices
+//   route_finish_kernel location = rank in tile + prefix; GShard loss
+//
+// Workspace layout (int32 words): hist[tiles][k][E] then me[tiles][E] (fp32).
+#include "common.hpp"
+
+namespace pm {
+
+constexpr int TILE = 256;         // tokens per tile = threads per block
+constexpr int ROUTE_MAX_E = 2048; // LDS table is 4 waves x experts counters
+
+__device__ __forceinline__ uint64_t lanemask_lt()
+{
+    return ((uint64_t)1 << lane_id()) - 1;
+}
+
+template <int DT>
+struct ScoreRow {
+    using E = Elem<DT>;
+    const void *in;
+    const float *bias;
+    int64_t base;
+    int experts;
+    bool logits;
+    float mx, sum;
+
+    __device__ __forceinline__ float logit(int e) const
+    {
+        float l = E::load(in, base + e);
+        if (bias) l = E::round(l + bias[e]);
+        return l;
+    }
+    __device__ void prepare()
+    {
+        if (!logits) return;
+        mx = -INFINITY;
+        for (int e = 0; e < experts; ++e) mx = fmaxf(mx, logit(e));
+        sum = 0.f;
+        for (int e = 0; e < experts; ++e) sum += expf(logit(e) - mx);
+    }
+    // score of expert e in the routing dtype
+    __device__ __forceinline__ float score(int e) const
+    {
+        if (!logits) return E::load(in, base + e);
+        return E::round(expf(logit(e) - mx) / sum);
+    }
+};
+
+// CAP > 0: the row (<= CAP scores) lives in registers; CAP == 0: every pass recomputes
+// the scores from memory.
+template <int DT, int CAP>
+__global__ __launch_bounds__(TILE) void route_tile_kernel(
+    const void *__restrict__ input, int input_is_logits, const float *__restrict__ logit_bias,
+    int samples, int experts, int k, int normalize_gate,
+    int32_t *__restrict__ indices, int32_t *__restrict__ locations, void *__restrict__ gates,
+    int64_t stride, void *__restrict__ scores_out, int32_t *__restrict__ hist,
+    float *__restrict__ me_part)
+{
+    using E = Elem<DT>;
+    extern __shared__ int32_t wave_cnt[];           // [4][experts]
+    const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
+    const int t = blockIdx.x * TILE + tid;
+    const bool valid = t < samples;
+
+    ScoreRow<DT> row;
+    row.in = input; row.bias = logit_bias; row.base = (int64_t)t * experts;
+    row.experts = experts; row.logits = input_is_logits != 0;
+
+    float s[CAP > 0 ? CAP : 1];
+    if (valid) {
+        row.prepare();
+        if constexpr (CAP > 0) {
+#pragma unroll
+            for (int e = 0; e < CAP; ++e) s[e] = (e < experts) ? row.score(e) : -INFINITY;
+        }
+        if (scores_out) {
+            if constexpr (CAP > 0) {
+#pragma unroll
+                for (int e = 0; e < CAP; ++e) if (e < experts) E::store(scores_out, row.base + e, s[e]);
+            } else {
+                for (int e = 0; e < experts; ++e) E::store(scores_out, row.base + e, row.score(e));
+            }
+        }
+    }
+
+    // per-tile column sums of the scores (for the GShard loss), fixed reduction order
+    if (me_part) {
+        float *wsum = reinterpret_cast<float *>(wave_cnt);
+        if constexpr (CAP > 0) {
+#pragma unroll
+            for (int e = 0; e < CAP; ++e) {
+                if (e >= experts) break;
+                const float v = wave_sum(valid ? s[e] : 0.f);
+                if (lane == 0) wsum[wave * experts + e] = v;
+            }
+        } else {
+            for (int e = 0; e < experts; ++e) {
+                const float v = wave_sum(valid ? row.score(e) : 0.f);
+                if (lane == 0) wsum[wave * experts + e] = v;
+            }
+        }
+        __syncthreads();
+        for (int e = tid; e < experts; e += TILE)
+            me_part[(int64_t)blockIdx.x * experts + e] =
+                ((wsum[e] + wsum[experts + e]) + wsum[2 * experts + e]) + wsum[3 * experts + e];
+        __syncthreads();
+    }
+
+    // k-fold arg-max: lower expert id wins among equal scores
+    float denom = 0.f;
+    uint64_t taken_lo = 0;                       // experts < 64 already chosen (CAP path)
+    for (int j = 0; j < k; ++j) {
+        int best = -1; float bv = -INFINITY;
+        if (valid) {
+            if constexpr (CAP > 0) {
+#pragma unroll
+                for (int e = 0; e < CAP; ++e) {
+                    const bool free_ = !((taken_lo >> e) & 1u) && e < experts;
+                    if (free_ && (best < 0 || s[e] > bv)) { best = e; bv = s[e]; }
+                }
+                taken_lo |= (uint64_t)1 << best;
+            } else {
+                // chosen experts of earlier planes are re-read from the output planes
+                for (int e = 0; e < experts; ++e) {
+                    bool free_ = true;
+                    for (int p = 0; p < j; ++p) free_ = free_ && (indices[(int64_t)p * stride + t] != e);
+                    const float v = row.score(e);
+                    if (free_ && (best < 0 || v > bv)) { best = e; bv = v; }
+                }
+            }
+            indices[(int64_t)j * stride + t] = best;
+            // raw gate now, normalised after the loop
+            E::store(gates, (int64_t)j * stride + t, bv);
+            denom = (j == 0) ? bv : E::round(denom + bv);
+        }
+
+        // rank of this token among the tile's tokens with the same j-th choice
+        for (int e = tid; e < 4 * experts; e += TILE) wave_cnt[e] = 0;
+        __syncthreads();
+        int rank = 0;
+        uint64_t todo = __ballot(valid);
+        while (todo) {
+            const int leader = __ffsll((unsigned long long)todo) - 1;
+            const int le = __builtin_amdgcn_readlane(best, leader);
+            const uint64_t m = __ballot(valid && best == le);
+            if (valid && best == le) rank = __popcll(m & lanemask_lt());
+            if (lane == leader) wave_cnt[wave * experts + le] = __popcll(m);
+            todo &= ~m;
+        }
+        __syncthreads();
+        if (valid) {
+            int before = 0;
+            for (int w = 0; w < wave; ++w) before += wave_cnt[w * experts + best];
+            locations[(int64_t)j * stride + t] = rank + before;
+        }
+        for (int e = tid; e < experts; e += TILE)
+            hist[((int64_t)blockIdx.x * k + j) * experts + e] =
+                wave_cnt[e] + wave_cnt[experts + e] + wave_cnt[2 * experts + e] + wave_cnt[3 * experts + e];
+        __syncthreads();
+    }
+
+    if (valid && k > 1 && normalize_gate) {
+        const float eps = DT == PLANMOE_F32 ? 1.1920928955078125e-07f
+                        : DT == PLANMOE_BF16 ? 0.0078125f : 0.0009765625f;
+        const float d = fmaxf(denom, eps);
+        for (int j = 0; j < k; ++j) {
+            const float g = E::load(gates, (int64_t)j * stride + t);
+            E::store(gates, (int64_t)j * stride + t, g / d);
+        }
+    }
+}
+
+// One block per group of up to 64 experts; 256 threads = expert lanes x tile chunks.
+// hist[tile][j][e] is replaced by the number of slots of expert e taken before tile `tile`
+// of plane j: all of planes < j plus the tiles before it in plane j.
+__global__ __launch_bounds__(256) void route_scan_kernel(int32_t *__restrict__ hist, int tiles,
+                                                         int k, int experts,
+                                                         int32_t *__restrict__ counts_out,
+                                                         int32_t *__restrict__ counts_ws)
+{
+    __shared__ int32_t part[256];
+    const int eb = min(64, experts);                 // expert lanes in this block
+    int lanes_e = 1; while (lanes_e < eb) lanes_e <<= 1;
+    const int chunks = 256 / lanes_e;
+    const int el = threadIdx.x % lanes_e, ch = threadIdx.x / lanes_e;
+    const int e = blockIdx.x * 64 + el;
+    const bool live = el < eb && e < experts;
+    const int per = (tiles + chunks - 1) / chunks;
+    const int t0 = min(ch * per, tiles), t1 = min(t0 + per, tiles);
+
+    int32_t carry = 0;
+    for (int j = 0; j < k; ++j) {
+        int32_t s = 0;
+        if (live)
+            for (int t = t0; t < t1; ++t) s += hist[((int64_t)t * k + j) * experts + e];
+        part[threadIdx.x] = s;
+        __syncthreads();
+        int32_t before = 0, total = 0;
+        for (int c = 0; c < chunks; ++c) {
+            const int32_t v = part[c * lanes_e + el];
+            before += (c < ch) ? v : 0;
+            total += v;
+        }
+        if (live) {
+            int32_t run = carry + before;
+            for (int t = t0; t < t1; ++t) {
+                const int64_t o = ((int64_t)t * k + j) * experts + e;
+                const int32_t v = hist[o];
+                hist[o] = run;
+                run += v;
+            }
+            if (ch == 0) {
+                if (counts_out) counts_out[j * experts + e] = total;
+                if (j == 0) counts_ws[e] = total;
+            }
+        }
+        carry += total;
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(TILE) void route_finish_kernel(
+    const int32_t *__restrict__ indices, int32_t *__restrict__ locations, int64_t stride,
+    int samples, int experts, int k, const int32_t *__restrict__ hist,
+    const float *__restrict__ me_part, const int32_t *__restrict__ counts_ws, int tiles,
+    float *__restrict__ l_aux)
+{
+    const int t = blockIdx.x * TILE + threadIdx.x;
+    if (t < samples) {
+        for (int j = 0; j < k; ++j) {
+            const int64_t o = (int64_t)j * stride + t;
+            locations[o] += hist[((int64_t)blockIdx.x * k + j) * experts + indices[o]];
+        }
+    }
+    if (l_aux && blockIdx.x == 0) {
+        // l_aux = sum_e(me[e] * ce[e]) / T, ce[e] = count0[e] * (E / T)
+        __shared__ float red[TILE / WAVE];
+        float acc = 0.f;
+        for (int e = threadIdx.x; e < experts; e += TILE) {
+            float me = 0.f;
+            for (int tl = 0; tl < tiles; ++tl) me += me_part[(int64_t)tl * experts + e];
+            const float ce = (float)counts_ws[e] * ((float)experts / (float)samples);
+            acc += me * ce;
+        }
+        acc = wave_sum(acc);
+        if (lane_id() == 0) red[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0) *l_aux = (((red[0] + red[1]) + red[2]) + red[3]) / (float)samples;
+    }
+}
+
+// ------------------------------------------------------------------ stand-alone cumsum
+// out = cumsum(in, dim 0) - 1 over an int32 [samples, columns] matrix, three phases:
+// per-tile column sums, prefix of the tile sums, per-tile rescan with the tile's offset.
+// A block covers 64-column groups with 256 threads = column lanes x row lanes; a thread
+// walks CS_ROWS consecutive rows of its column.
+constexpr int CS_ROWS = 16;
+
+struct CsGeom { int lanes_c, lanes_r, tile_rows; };
+__host__ __device__ inline CsGeom cs_geom(int columns)
+{
+    CsGeom g;
+    g.lanes_c = 1;
+    while (g.lanes_c < columns && g.lanes_c < 64) g.lanes_c <<= 1;
+    g.lanes_r = 256 / g.lanes_c;
+    g.tile_rows = g.lanes_r * CS_ROWS;
+    return g;
+}
+
+template <bool FINAL>
+__global__ __launch_bounds__(256) void cumsum_tile_kernel(const int32_t *__restrict__ in,
+                                                          int32_t *__restrict__ out, int samples,
+                                                          int columns, int32_t *__restrict__ tile_sums)
+{
+    __shared__ int32_t part[256];
+    const CsGeom g = cs_geom(columns);
+    const int cl = threadIdx.x % g.lanes_c, rl = threadIdx.x / g.lanes_c;
+    const int c = blockIdx.y * 64 + cl;
+    const bool live = c < columns;
+    const int r0 = blockIdx.x * g.tile_rows + rl * CS_ROWS;
+    int32_t v[CS_ROWS];
+    int32_t s = 0;
+#pragma unroll
+    for (int i = 0; i < CS_ROWS; ++i) {
+        const int r = r0 + i;
+        v[i] = (live && r < samples) ? in[(int64_t)r * columns + c] : 0;
+        s += v[i];
+    }
+    part[threadIdx.x] = s;
+    __syncthreads();
+    int32_t before = 0, total = 0;
+    for (int q = 0; q < g.lanes_r; ++q) {
+        const int32_t p = part[q * g.lanes_c + cl];
+        before += (q < rl) ? p : 0;
+        total += p;
+    }
+    if constexpr (!FINAL) {
+        if (live && rl == 0) tile_sums[(int64_t)blockIdx.x * columns + c] = total;
+    } else {
+        if (!live) return;
+        int32_t run = tile_sums[(int64_t)blockIdx.x * columns + c] + before - 1;
+#pragma unroll
+        for (int i = 0; i < CS_ROWS; ++i) {
+            const int r = r0 + i;
+            run += v[i];
+            if (r < samples) out[(int64_t)r * columns + c] = run;
+        }
+    }
+}
+
+// exclusive prefix over tiles, in place; same thread geometry as route_scan_kernel
+__global__ __launch_bounds__(256) void cumsum_scan_kernel(int32_t *__restrict__ tile_sums, int tiles,
+                                                          int columns)
+{
+    __shared__ int32_t part[256];
+    const int cb = min(64, columns);
+    int lanes_c = 1; while (lanes_c < cb) lanes_c <<= 1;
+    const int chunks = 256 / lanes_c;
+    const int cl = threadIdx.x % lanes_c, ch = threadIdx.x / lanes_c;
+    const int c = blockIdx.x * 64 + cl;
+    const bool live = cl < cb && c < columns;
+    const int per = (tiles + chunks - 1) / chunks;
+    const int t0 = min(ch * per, tiles), t1 = min(t0 + per, tiles);
+    int32_t s = 0;
+    if (live) for (int t = t0; t < t1; ++t) s += tile_sums[(int64_t)t * columns + c];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    int32_t before = 0;
+    for (int q = 0; q < ch; ++q) before += part[q * lanes_c + cl];
+    if (live) {
+        int32_t run = before;
+        for (int t = t0; t < t1; ++t) {
+            const int64_t o = (int64_t)t * columns + c;
+            const int32_t v = tile_sums[o];
+            tile_sums[o] = run;
+            run += v;
+        }
+    }
+}
+
+} // namespace pm
+
+using namespace pm;
+
+extern "C" size_t planmoe_cumsum_workspace_bytes(int samples, int columns)
+{
+    if (samples <= 0 || columns <= 0) return 16;
+    const CsGeom g = cs_geom(columns);
+    const size_t tiles = ((size_t)samples + g.tile_rows - 1) / g.tile_rows;
+    return round_up(tiles * (size_t)columns * sizeof(int32_t), 256);
+}
+
+extern "C" int planmoe_cumsum_sub_one(const int32_t *in, int32_t *out, int samples, int columns,
+                                      void *workspace, size_t workspace_bytes, void *stream)
+{
+    PM_REQUIRE(samples >= 0 && columns >= 0, "planmoe_cumsum_sub_one: bad shape");
+    if (samples == 0 || columns == 0) return 0;
+    PM_REQUIRE(in && out, "planmoe_cumsum_sub_one: NULL argument");
+    PM_REQUIRE(workspace && workspace_bytes >= planmoe_cumsum_workspace_bytes(samples, columns),
+               "planmoe_cumsum_sub_one: workspace too small");
+    const CsGeom g = cs_geom(columns);
+    const int tiles = (samples + g.tile_rows - 1) / g.tile_rows;
+    const int cgroups = (columns + 63) / 64;
+    PM_REQUIRE(cgroups <= 65535, "planmoe_cumsum_sub_one: too many columns");
+    hipStream_t st = (hipStream_t)stream;
+    int32_t *sums = (int32_t *)workspace;
+    cumsum_tile_kernel<false><<<dim3(tiles, cgroups), 256, 0, st>>>(in, out, samples, columns, sums);
+    cumsum_scan_kernel<<<cgroups, 256, 0, st>>>(sums, tiles, columns);
+    cumsum_tile_kernel<true><<<dim3(tiles, cgroups), 256, 0, st>>>(in, out, samples, columns, sums);
+    PM_LAUNCH_CHECK("planmoe_cumsum_sub_one");
+    return 0;
+}
+
+static inline size_t route_tiles(int samples) { return ((size_t)samples + TILE - 1) / TILE; }
+
+extern "C" size_t planmoe_route_workspace_bytes(int samples, int experts, int top_k)
+{
+    if (samples <= 0 || experts <= 0 || top_k <= 0) return 16;
+    const size_t k = (size_t)(top_k < experts ? top_k : experts);
+    const size_t tiles = route_tiles(samples);
+    // hist[tiles][k][E] + me[tiles][E] + count0[E]
+    return round_up((tiles * k * experts + tiles * experts + (size_t)experts) * 4, 256);
+}
+
+template <int DT>
+static int launch_route_tile(int cap, dim3 grid, size_t lds, hipStream_t st, const void *input,
+                             int is_logits, const float *bias, int samples, int experts, int k,
+                             int normalize, int32_t *indices, int32_t *locations, void *gates,
+                             int64_t stride, void *scores_out, int32_t *hist, float *me)
+{
+#define PM_ROUTE_LAUNCH(CAP)                                                                  \
+    route_tile_kernel<DT, CAP><<<grid, TILE, lds, st>>>(input, is_logits, bias, samples,      \
+        experts, k, normalize, indices, locations, gates, stride, scores_out, hist, me)
+    if (cap <= 8) PM_ROUTE_LAUNCH(8);
+    else if (cap <= 16) PM_ROUTE_LAUNCH(16);
+    else if (cap <= 64) PM_ROUTE_LAUNCH(64);
+    else PM_ROUTE_LAUNCH(0);
+#undef PM_ROUTE_LAUNCH
+    return 0;
+}
+
+extern "C" int planmoe_route_topk(const void *input, int dtype, int input_is_logits,
+                                  const float *logit_bias, int samples, int experts, int top_k,
+                                  int normalize_gate, int32_t *indices, int32_t *locations,
+                                  void *gates, int64_t plane_stride, void *scores_out, float *l_aux,
+                                  int32_t *expert_counts, void *workspace, size_t workspace_bytes,
+                                  void *stream)
+{
+    PM_REQUIRE(dtype == PLANMOE_F32 || dtype == PLANMOE_BF16 || dtype == PLANMOE_F16,
+               "planmoe_route_topk: bad dtype %d", dtype);
+    PM_REQUIRE(samples >= 0 && experts >= 1 && top_k >= 1, "planmoe_route_topk: bad shape");
+    PM_REQUIRE(experts <= ROUTE_MAX_E, "planmoe_route_topk: experts %d > supported %d", experts, ROUTE_MAX_E);
+    PM_REQUIRE(plane_stride >= samples, "planmoe_route_topk: plane_stride < samples");
+    PM_REQUIRE(!logit_bias || input_is_logits, "planmoe_route_topk: logit_bias needs input_is_logits");
+    const int k = top_k < experts ? top_k : experts;
+    hipStream_t st = (hipStream_t)stream;
+    if (samples == 0) {
+        if (expert_counts) fill_u32((uint32_t *)expert_counts, (size_t)k * experts, 0u, st);
+        // the loss of an empty batch is 0/0 in the reference; leave l_aux untouched
+        return 0;
+    }
+    PM_REQUIRE(input && indices && locations && gates, "planmoe_route_topk: NULL argument");
+    PM_REQUIRE(workspace && workspace_bytes >= planmoe_route_workspace_bytes(samples, experts, top_k),
+               "planmoe_route_topk: workspace too small (%zu < %zu)", workspace_bytes,
+               planmoe_route_workspace_bytes(samples, experts, top_k));
+    const int tiles = (int)route_tiles(samples);
+    int32_t *hist = (int32_t *)workspace;
+    float *me = (float *)(hist + (size_t)tiles * k * experts);
+    int32_t *count0 = (int32_t *)(me + (size_t)tiles * experts);
+    const size_t lds = sizeof(int32_t) * 4 * (size_t)experts;
+
+    PM_DTYPE_SWITCH(dtype, DT,
+        launch_route_tile<DT>(experts, dim3(tiles), lds, st, input, input_is_logits, logit_bias,
+                              samples, experts, k, normalize_gate, indices, locations, gates,
+                              plane_stride, scores_out, hist, l_aux ? me : nullptr));
+    route_scan_kernel<<<(experts + 63) / 64, 256, 0, st>>>(hist, tiles, k, experts, expert_counts, count0);
+    route_finish_kernel<<<tiles, TILE, 0, st>>>(indices, locations, plane_stride, samples, experts, k,
+                                               hist, me, count0, tiles, l_aux);
+    PM_LAUNCH_CHECK("planmoe_route_topk");
+    return 0;
+}

@@ -1,0 +1,55 @@
+// Row access helpers shared by the kernels that move token rows to and from capacity slots.
+#pragma once
+#include "common.hpp"
+
+namespace pm {
+
+template <int DT, bool VECTOR>
+struct RowIO {
+    using E = Elem<DT>;
+    static constexpr int U = VECTOR ? E::VEC : 1;      // elements per lane access
+    __device__ static __forceinline__ void load(const void *row, int unit, float *f)
+    {
+        if constexpr (VECTOR) E::unpack(reinterpret_cast<const uint4 *>(row)[unit], f);
+        else f[0] = E::load(row, unit);
+    }
+    __device__ static __forceinline__ void store(void *row, int unit, const float *f)
+    {
+        if constexpr (VECTOR) reinterpret_cast<uint4 *>(row)[unit] = E::pack(f);
+        else E::store(row, unit, f[0]);
+    }
+    __device__ static __forceinline__ void store_zero(void *row, int unit)
+    {
+        if constexpr (VECTOR) reinterpret_cast<uint4 *>(row)[unit] = make_uint4(0, 0, 0, 0);
+        else E::store(row, unit, 0.f);
+    }
+};
+
+__device__ __forceinline__ int   rl_i(int v, int lane)   { return __builtin_amdgcn_readlane(v, lane); }
+__device__ __forceinline__ float rl_f(float v, int lane) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane)); }
+
+// Lane j (< nplanes) of the calling wave fetches plane j0+j of token t: its slot row
+// (-1 when the pair is not live) and its gate.
+__device__ __forceinline__ void fetch_planes(const float *gates, const int32_t *indices,
+                                             const int32_t *locations, int64_t stride, int t,
+                                             int j0, int nplanes, int experts, int capacity,
+                                             int &slot, float &gate)
+{
+    slot = -1; gate = 1.f;
+    const int lane = lane_id();
+    if (lane < nplanes) {
+        const int64_t o = (int64_t)(j0 + lane) * stride + t;
+        const int e = indices[o], l = locations[o];
+        if (e >= 0 && e < experts && l >= 0 && l < capacity) slot = e * capacity + l;
+        if (gates) gate = gates[o];
+    }
+}
+
+// occupancy flags of the experts*capacity slots (1 = some live pair addresses the slot)
+void launch_slot_flags(uint32_t *flags, const int32_t *indices, const int32_t *locations,
+                       int64_t stride, int top_k, int samples, int experts, int capacity,
+                       hipStream_t st);
+int check_planes(const char *who, const int32_t *indices, const int32_t *locations,
+                 int64_t stride, int top_k, int samples);
+
+} // namespace pm

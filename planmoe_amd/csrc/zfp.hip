@@ -1,0 +1,404 @@
+// zfp fixed-rate float codec (stream-compatible with stock zfp 0.5.5), 1-D and 2-D.
+//
+// Takes the place of zfp_compress / zfp_decompress with the CUDA execution policy as called
+// by ZfpCompressor (custom/compressor/zfpc.cpp:31-51, 66-84).  One thread owns one block
+// (4 or 4x4 values): block-floating-point cast, lifting transform, negabinary reorder and the
+// embedded bit-plane coder all run in registers; a block's bits leave the thread as NW
+// 32-bit words (2-D rate 8: exactly one 16-byte store).  Loads are 16 bytes per lane per
+// row, consecutive lanes taking consecutive blocks along the fastest axis.
+#include "common.hpp"
+#include <cmath>
+
+namespace pm {
+
+template <int NW>
+struct BitWriter {
+    uint32_t w[NW];
+    uint64_t acc;
+    int fill, wi;
+    __device__ __forceinline__ void init()
+    {
+#pragma unroll
+        for (int i = 0; i < NW; ++i) w[i] = 0u;
+        acc = 0; fill = 0; wi = 0;
+    }
+    __device__ __forceinline__ void flush_word()
+    {
+        const uint32_t x = (uint32_t)acc;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) if (i == wi) w[i] = x;
+        ++wi; acc >>= 32; fill -= 32;
+    }
+    // append the low n (<= 32) bits of v; bits of v above n must be zero
+    __device__ __forceinline__ void put(uint32_t v, int n)
+    {
+        acc |= (uint64_t)v << fill;
+        fill += n;
+        if (fill >= 32) flush_word();
+    }
+    __device__ __forceinline__ void finish() { if (fill > 0) flush_word(); }
+};
+
+template <int NW>
+struct BitReader {
+    uint32_t w[NW];
+    uint64_t acc;
+    int avail, wi;
+    __device__ __forceinline__ void init()
+    {
+        acc = w[0];
+        avail = 32; wi = 1;
+        if constexpr (NW > 1) { acc |= (uint64_t)w[1] << 32; avail = 64; wi = 2; }
+    }
+    __device__ __forceinline__ void skip(int n)
+    {
+        acc >>= n; avail -= n;
+        if (avail <= 32 && wi < NW) {
+            uint32_t x = 0;
+#pragma unroll
+            for (int i = 0; i < NW; ++i) if (i == wi) x = w[i];
+            acc |= (uint64_t)x << avail;
+            avail += 32; ++wi;
+        }
+    }
+    __device__ __forceinline__ uint32_t get(int n)   // n <= 31
+    {
+        const uint32_t v = (uint32_t)acc & ((1u << n) - 1u);
+        skip(n);
+        return v;
+    }
+};
+
+__device__ __forceinline__ void fwd_lift(int32_t &x, int32_t &y, int32_t &z, int32_t &w)
+{
+    x += w; x >>= 1; w -= x;
+    z += y; z >>= 1; y -= z;
+    x += z; x >>= 1; z -= x;
+    w += y; w >>= 1; y -= w;
+    w += y >> 1; y -= w >> 1;
+}
+
+__device__ __forceinline__ void inv_lift(int32_t &x, int32_t &y, int32_t &z, int32_t &w)
+{
+    y += w >> 1; w -= y >> 1;
+    y += w; w = (int32_t)((uint32_t)w << 1); w -= y;
+    z += x; x = (int32_t)((uint32_t)x << 1); x -= z;
+    y += z; z = (int32_t)((uint32_t)z << 1); z -= y;
+    w += x; x = (int32_t)((uint32_t)x << 1); x -= w;
+}
+
+__device__ __forceinline__ uint32_t to_negabinary(int32_t v) { return ((uint32_t)v + 0xaaaaaaaau) ^ 0xaaaaaaaau; }
+__device__ __forceinline__ int32_t from_negabinary(uint32_t v) { return (int32_t)((v ^ 0xaaaaaaaau) - 0xaaaaaaaau); }
+
+// sequency order of the 4x4 coefficients (index into the i + 4j block layout)
+__device__ constexpr int perm2(int i)
+{
+    constexpr int P[16] = {0, 1, 4, 5, 2, 8, 6, 9, 3, 12, 10, 7, 13, 11, 14, 15};
+    return P[i];
+}
+
+// N = values per block (4 or 16).  f is consumed; the block's maxbits = 32*NW bits land in bw.
+template <int N, int NW>
+__device__ __forceinline__ void encode_block(const float *f, BitWriter<NW> &bw)
+{
+    bw.init();
+    float m = 0.f;
+#pragma unroll
+    for (int i = 0; i < N; ++i) m = fmaxf(m, fabsf(f[i]));
+    if (!(m > 0.f)) return;                       // all-zero block: '0' flag and zero padding
+    // frexp exponent clamped at 1 - 127, i.e. exponent field - 126 (a denormal maximum reads 0)
+    const int field = (int)((__float_as_uint(m) >> 23) & 0xffu);
+    const int emax = field - 126;
+    bw.put(2u * (uint32_t)(emax + 127) + 1u, 9);
+
+    // block-floating-point cast: q = (int32)(f * 2^(30 - emax)), x86 conversion on overflow
+    const int se = 30 - emax;
+    const float s = se > 127 ? INFINITY : __uint_as_float((uint32_t)(se + 127) << 23);
+    int32_t q[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const float v = f[i] * s;
+        q[i] = (v >= 2147483648.0f || v < -2147483648.0f || v != v) ? (int32_t)0x80000000 : (int32_t)v;
+    }
+    uint32_t u[N];
+    if constexpr (N == 4) {
+        fwd_lift(q[0], q[1], q[2], q[3]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) u[i] = to_negabinary(q[i]);
+    } else {
+#pragma unroll
+        for (int y = 0; y < 4; ++y) fwd_lift(q[4 * y], q[4 * y + 1], q[4 * y + 2], q[4 * y + 3]);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) fwd_lift(q[x], q[x + 4], q[x + 8], q[x + 12]);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) u[i] = to_negabinary(q[perm2(i)]);
+    }
+
+    // embedded coding: bit planes from the top, group-tested, until the budget is spent
+    int bits = 32 * NW - 9;
+    int nsig = 0;
+    for (int k = 31; k >= 0 && bits > 0; --k) {
+        uint32_t x = 0;
+#pragma unroll
+        for (int i = 0; i < N; ++i) x |= ((u[i] >> k) & 1u) << i;
+        const int mm = min(nsig, bits);
+        bits -= mm;
+        bw.put(x & ((1u << mm) - 1u), mm);
+        x >>= mm;
+        while (nsig < N && bits > 0) {
+            --bits;
+            bw.put(x != 0u ? 1u : 0u, 1);
+            if (x == 0u) break;
+            // zeros up to the next one bit, then the one (implicit when it is the last value)
+            const int z = __builtin_ctz(x);
+            const int r = N - 1 - nsig;
+            const int cnt = min(z + 1, r);
+            const int emit = min(cnt, bits);
+            const uint32_t pat = (z < r ? (1u << z) : 0u) & ((1u << emit) - 1u);
+            bw.put(pat, emit);
+            bits -= emit;
+            x >>= z; x >>= 1;
+            nsig += z + 1;
+        }
+    }
+    bw.finish();
+}
+
+template <int N, int NW>
+__device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f)
+{
+    br.init();
+    if (!br.get(1)) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) f[i] = 0.f;
+        return;
+    }
+    const int emax = (int)br.get(8) - 127;
+    uint32_t u[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) u[i] = 0u;
+    int bits = 32 * NW - 9;
+    int nsig = 0;
+    for (int k = 31; k >= 0 && bits > 0; --k) {
+        const int mm = min(nsig, bits);
+        bits -= mm;
+        uint32_t x = br.get(mm);
+        while (nsig < N && bits > 0) {
+            --bits;
+            if (!br.get(1)) break;
+            const int lim = min(N - 1 - nsig, bits);
+            const uint32_t win = (uint32_t)br.acc & ((1u << lim) - 1u);
+            if (win != 0u) {
+                const int z = __builtin_ctz(win);
+                br.skip(z + 1); bits -= z + 1; nsig += z;
+            } else {
+                br.skip(lim); bits -= lim; nsig += lim;
+            }
+            x |= 1u << nsig;
+            ++nsig;
+        }
+#pragma unroll
+        for (int i = 0; i < N; ++i) u[i] |= ((x >> i) & 1u) << k;
+    }
+    int32_t q[N];
+    if constexpr (N == 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) q[i] = from_negabinary(u[i]);
+        inv_lift(q[0], q[1], q[2], q[3]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) q[perm2(i)] = from_negabinary(u[i]);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) inv_lift(q[x], q[x + 4], q[x + 8], q[x + 12]);
+#pragma unroll
+        for (int y = 0; y < 4; ++y) inv_lift(q[4 * y], q[4 * y + 1], q[4 * y + 2], q[4 * y + 3]);
+    }
+    const float s = ldexpf(1.0f, emax - 30);
+#pragma unroll
+    for (int i = 0; i < N; ++i) f[i] = (float)q[i] * s;
+}
+
+template <int NW>
+__device__ __forceinline__ void store_words(uint32_t *dst, const uint32_t *w)
+{
+    if constexpr (NW == 1) dst[0] = w[0];
+    else if constexpr (NW == 2) *reinterpret_cast<uint2 *>(dst) = make_uint2(w[0], w[1]);
+    else {
+#pragma unroll
+        for (int i = 0; i < NW / 4; ++i)
+            reinterpret_cast<uint4 *>(dst)[i] = make_uint4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
+    }
+}
+
+template <int NW>
+__device__ __forceinline__ void load_words(const uint32_t *src, uint32_t *w)
+{
+    if constexpr (NW == 1) w[0] = src[0];
+    else if constexpr (NW == 2) { const uint2 v = *reinterpret_cast<const uint2 *>(src); w[0] = v.x; w[1] = v.y; }
+    else {
+#pragma unroll
+        for (int i = 0; i < NW / 4; ++i) {
+            const uint4 v = reinterpret_cast<const uint4 *>(src)[i];
+            w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
+        }
+    }
+}
+
+template <int NW>
+__global__ __launch_bounds__(256) void zfp_encode1_kernel(const float *__restrict__ field, int64_t blocks,
+                                                          uint32_t *__restrict__ out)
+{
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    const float4 v = reinterpret_cast<const float4 *>(field)[b];
+    const float f[4] = {v.x, v.y, v.z, v.w};
+    BitWriter<NW> bw;
+    encode_block<4, NW>(f, bw);
+    store_words<NW>(out + b * NW, bw.w);
+    // an odd count of 32-bit words leaves half of the last 64-bit stream word as padding
+    if (b == blocks - 1 && ((blocks * NW) & 1)) out[blocks * NW] = 0u;
+}
+
+template <int NW>
+__global__ __launch_bounds__(256) void zfp_decode1_kernel(const uint32_t *__restrict__ in, int64_t blocks,
+                                                          float *__restrict__ field)
+{
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    BitReader<NW> br;
+    load_words<NW>(in + b * NW, br.w);
+    float f[4];
+    decode_block<4, NW>(br, f);
+    reinterpret_cast<float4 *>(field)[b] = make_float4(f[0], f[1], f[2], f[3]);
+}
+
+template <int NW>
+__global__ __launch_bounds__(256) void zfp_encode2_kernel(const float *__restrict__ field, int64_t nx,
+                                                          int64_t nbx, int64_t blocks,
+                                                          uint32_t *__restrict__ out)
+{
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    const int64_t by = b / nbx, bx = b - by * nbx;
+    const float *p = field + 4 * by * nx + 4 * bx;
+    float f[16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float4 v = *reinterpret_cast<const float4 *>(p + j * nx);
+        f[4 * j] = v.x; f[4 * j + 1] = v.y; f[4 * j + 2] = v.z; f[4 * j + 3] = v.w;
+    }
+    BitWriter<NW> bw;
+    encode_block<16, NW>(f, bw);
+    store_words<NW>(out + b * NW, bw.w);
+}
+
+template <int NW>
+__global__ __launch_bounds__(256) void zfp_decode2_kernel(const uint32_t *__restrict__ in, int64_t nx,
+                                                          int64_t nbx, int64_t blocks,
+                                                          float *__restrict__ field)
+{
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    BitReader<NW> br;
+    load_words<NW>(in + b * NW, br.w);
+    float f[16];
+    decode_block<16, NW>(br, f);
+    const int64_t by = b / nbx, bx = b - by * nbx;
+    float *p = field + 4 * by * nx + 4 * bx;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<float4 *>(p + j * nx) = make_float4(f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]);
+}
+
+static int zfp_maxbits(int dims, double rate)
+{
+    const int n = dims == 1 ? 4 : 16;
+    int bits = (int)std::floor(n * rate + 0.5);
+    if (bits < 9) bits = 9;
+    return bits;
+}
+
+static int zfp_check(const char *who, int dims, int64_t nx, int64_t ny, double rate, int &nw,
+                     int64_t &blocks)
+{
+    PM_REQUIRE(dims == 1 || dims == 2, "%s: dims must be 1 or 2 (got %d)", who, dims);
+    PM_REQUIRE(nx >= 0 && ny >= 0, "%s: negative extent", who);
+    PM_REQUIRE(nx % 4 == 0 && ny % 4 == 0, "%s: zfp fails. (every extent must be a multiple of 4, got nx=%lld ny=%lld)",
+               who, (long long)nx, (long long)ny);
+    PM_REQUIRE(rate > 0, "%s: rate must be > 0", who);
+    const int maxbits = zfp_maxbits(dims, rate);
+    PM_REQUIRE(maxbits % 32 == 0 && (maxbits / 32 == 1 || maxbits / 32 == 2 || maxbits / 32 == 4 || maxbits / 32 == 8),
+               "%s: rate %.3f gives %d bits per block; supported block sizes are 32, 64, 128 and 256 bits",
+               who, rate, maxbits);
+    nw = maxbits / 32;
+    blocks = dims == 1 ? (nx * ny) / 4 : (nx / 4) * (ny / 4);
+    PM_REQUIRE((blocks + 255) / 256 < (1ll << 31), "%s: field too large", who);
+    return 0;
+}
+
+} // namespace pm
+
+using namespace pm;
+
+extern "C" size_t planmoe_zfp_max_bytes(int dims, int64_t nx, int64_t ny, double rate)
+{
+    if ((dims != 1 && dims != 2) || nx < 0 || ny < 0 || !(rate > 0)) return 0;
+    const uint64_t blocks = dims == 1 ? (uint64_t)(nx * ny + 3) / 4 : (uint64_t)((nx + 3) / 4) * (uint64_t)((ny + 3) / 4);
+    const uint64_t bits = 148u + blocks * (uint64_t)zfp_maxbits(dims, rate);   // header allowance
+    return (size_t)(((bits + 63u) / 64u) * 8u);
+}
+
+extern "C" size_t planmoe_zfp_stream_bytes(int dims, int64_t nx, int64_t ny, double rate)
+{
+    if ((dims != 1 && dims != 2) || nx < 0 || ny < 0 || !(rate > 0)) return 0;
+    const uint64_t blocks = dims == 1 ? (uint64_t)(nx * ny) / 4 : (uint64_t)(nx / 4) * (uint64_t)(ny / 4);
+    const uint64_t bits = blocks * (uint64_t)zfp_maxbits(dims, rate);
+    return (size_t)(((bits + 63u) / 64u) * 8u);
+}
+
+#define PM_NW_SWITCH(nw, NW, ...)                              \
+    switch (nw) {                                              \
+    case 1: { constexpr int NW = 1; __VA_ARGS__; break; }      \
+    case 2: { constexpr int NW = 2; __VA_ARGS__; break; }      \
+    case 4: { constexpr int NW = 4; __VA_ARGS__; break; }      \
+    default: { constexpr int NW = 8; __VA_ARGS__; break; }     \
+    }
+
+extern "C" int planmoe_zfp_compress(const float *field, int dims, int64_t nx, int64_t ny, double rate,
+                                    void *stream_out, size_t stream_capacity, void *stream)
+{
+    int nw; int64_t blocks;
+    if (zfp_check("planmoe_zfp_compress", dims, nx, ny, rate, nw, blocks)) return 1;
+    if (blocks == 0) return 0;
+    PM_REQUIRE(field && stream_out, "planmoe_zfp_compress: NULL argument");
+    PM_REQUIRE(aligned16(field) && aligned16(stream_out), "planmoe_zfp_compress: buffers must be 16-byte aligned");
+    const size_t need = planmoe_zfp_stream_bytes(dims, nx, ny, rate);
+    PM_REQUIRE(stream_capacity >= need, "planmoe_zfp_compress: stream buffer too small (%zu < %zu)",
+               stream_capacity, need);
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned grid = (unsigned)((blocks + 255) / 256);
+    PM_NW_SWITCH(nw, NW, {
+        if (dims == 1) zfp_encode1_kernel<NW><<<grid, 256, 0, st>>>(field, blocks, (uint32_t *)stream_out);
+        else zfp_encode2_kernel<NW><<<grid, 256, 0, st>>>(field, nx, nx / 4, blocks, (uint32_t *)stream_out);
+    });
+    PM_LAUNCH_CHECK("planmoe_zfp_compress");
+    return 0;
+}
+
+extern "C" int planmoe_zfp_decompress(const void *stream_in, int dims, int64_t nx, int64_t ny, double rate,
+                                      float *field, void *stream)
+{
+    int nw; int64_t blocks;
+    if (zfp_check("planmoe_zfp_decompress", dims, nx, ny, rate, nw, blocks)) return 1;
+    if (blocks == 0) return 0;
+    PM_REQUIRE(field && stream_in, "planmoe_zfp_decompress: NULL argument");
+    PM_REQUIRE(aligned16(field) && aligned16(stream_in), "planmoe_zfp_decompress: buffers must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned grid = (unsigned)((blocks + 255) / 256);
+    PM_NW_SWITCH(nw, NW, {
+        if (dims == 1) zfp_decode1_kernel<NW><<<grid, 256, 0, st>>>((const uint32_t *)stream_in, blocks, field);
+        else zfp_decode2_kernel<NW><<<grid, 256, 0, st>>>((const uint32_t *)stream_in, nx, nx / 4, blocks, field);
+    });
+    PM_LAUNCH_CHECK("planmoe_zfp_decompress");
+    return 0;
+}

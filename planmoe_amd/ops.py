@@ -1,0 +1,266 @@
+"""Tensor-level wrappers of the libplanmoe_hip C ABI.
+
+torch is used for what it is good at here -- device memory and the current HIP stream; all
+arithmetic happens in the HIP kernels.  Every function enqueues on
+``torch.cuda.current_stream()`` of the tensors' device and returns without synchronising.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import PlanMoEError, check, lib
+
+F32, BF16, F16 = 0, 1, 2
+_DT = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+
+
+def _dt(t, who):
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise PlanMoEError("%s: unsupported dtype %s (float32, bfloat16 or float16)" % (who, t.dtype))
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _need_gpu(t, who):
+    if not t.is_cuda:
+        raise PlanMoEError("%s: tensors must live on the GPU (this build has no CPU path)" % who)
+
+
+def _contig(t, who):
+    if not t.is_contiguous():
+        raise PlanMoEError("%s: tensor must be contiguous" % who)
+    return t
+
+
+def _ws(nbytes, device):
+    return torch.empty((max(int(nbytes), 16),), dtype=torch.uint8, device=device)
+
+
+def planes(tensors, dtype):
+    """Pack a list of k 1-D tensors as k planes of one buffer.
+
+    Returns (base tensor, plane stride in elements).  When the tensors already are equally
+    spaced views of one allocation (as route_topk returns them) no copy is made."""
+    k = len(tensors)
+    n = tensors[0].numel()
+    ok = all(t.dtype == dtype and t.dim() == 1 and t.numel() == n and t.is_contiguous() for t in tensors)
+    if ok:
+        if k == 1:
+            return tensors[0], max(n, 1)
+        es = tensors[0].element_size()
+        d = tensors[1].data_ptr() - tensors[0].data_ptr()
+        if d >= n * es and d % es == 0 and all(
+                tensors[j].data_ptr() - tensors[0].data_ptr() == j * d for j in range(k)) and \
+                tensors[0].untyped_storage().data_ptr() == tensors[-1].untyped_storage().data_ptr():
+            return tensors[0], d // es
+    stacked = torch.stack([t.reshape(-1).to(dtype) for t in tensors]).contiguous()
+    return stacked, max(n, 1)
+
+
+# ------------------------------------------------------------------------------ routing
+def capacity(samples, experts, top_k, capacity_factor=1.0, alignment=1):
+    out = ctypes.c_int(0)
+    check(lib.planmoe_capacity(samples, experts, top_k, float(capacity_factor), int(alignment),
+                               ctypes.byref(out)))
+    return out.value
+
+
+def cumsum_sub_one(mask):
+    """int32 [T, E] -> int32 [T, E]: cumsum over dim 0, minus one."""
+    _need_gpu(mask, "cumsum_sub_one")
+    x = mask.to(torch.int32).contiguous()
+    T, E = x.shape
+    out = torch.empty_like(x)
+    nbytes = lib.planmoe_cumsum_workspace_bytes(T, E)
+    ws = _ws(nbytes, x.device)
+    check(lib.planmoe_cumsum_sub_one(_ptr(x), _ptr(out), T, E, _ptr(ws), ws.numel(), _stream(x)))
+    return out
+
+
+def route_topk(inp, top_k, is_logits=False, logit_bias=None, normalize_gate=True,
+               want_scores=False, want_l_aux=True, want_counts=False):
+    """Top-k routing of scores (or logits) [T, E].
+
+    Returns dict(indices [k,T] int32, locations [k,T] int32, gates [k,T] inp.dtype,
+    scores [T,E] | None, l_aux 0-dim fp32 | None, counts [k,E] int32 | None)."""
+    _need_gpu(inp, "route_topk")
+    inp = _contig(inp, "route_topk")
+    if inp.dim() != 2:
+        raise PlanMoEError("route_topk: scores must be [samples, experts]")
+    T, E = inp.shape
+    k = min(int(top_k), E)
+    dev = inp.device
+    idx = torch.empty((k, T), dtype=torch.int32, device=dev)
+    loc = torch.empty((k, T), dtype=torch.int32, device=dev)
+    gates = torch.empty((k, T), dtype=inp.dtype, device=dev)
+    scores = torch.empty_like(inp) if want_scores else None
+    l_aux = torch.zeros((), dtype=torch.float32, device=dev) if want_l_aux else None
+    counts = torch.empty((k, E), dtype=torch.int32, device=dev) if want_counts else None
+    bias = None
+    if logit_bias is not None:
+        bias = logit_bias.to(device=dev, dtype=torch.float32).contiguous()
+    ws = _ws(lib.planmoe_route_workspace_bytes(T, E, k), dev)
+    check(lib.planmoe_route_topk(_ptr(inp), _dt(inp, "route_topk"), int(bool(is_logits)), _ptr(bias),
+                                 T, E, k, int(bool(normalize_gate)), _ptr(idx), _ptr(loc), _ptr(gates),
+                                 max(T, 1), _ptr(scores), _ptr(l_aux), _ptr(counts), _ptr(ws),
+                                 ws.numel(), _stream(inp)))
+    return dict(indices=idx, locations=loc, gates=gates, scores=scores, l_aux=l_aux, counts=counts)
+
+
+def gate_logits(x, wg, out_dtype=None):
+    """logits[T, E] = x[T, M] @ wg[E, M]^T with fp32 accumulation."""
+    _need_gpu(x, "gate_logits")
+    x = _contig(x, "gate_logits")
+    wg = _contig(wg, "gate_logits")
+    if x.dtype != wg.dtype:
+        raise PlanMoEError("gate_logits: x and wg must share a dtype")
+    out_dtype = out_dtype or x.dtype
+    T, M = x.shape
+    E = wg.shape[0]
+    out = torch.empty((T, E), dtype=out_dtype, device=x.device)
+    check(lib.planmoe_gate_logits(_ptr(x), _ptr(wg), _dt(x, "gate_logits"), _ptr(out), _DT[out_dtype],
+                                  T, M, E, _stream(x)))
+    return out
+
+
+# ------------------------------------------------------------------------------ dispatch / combine
+def _plane_args(indices, locations, gates, who):
+    idx, s1 = planes(indices, torch.int32)
+    loc, s2 = planes(locations, torch.int32)
+    if s1 != s2:
+        loc = torch.stack(list(locations)).contiguous()
+        idx = torch.stack(list(indices)).contiguous()
+        s1 = s2 = max(indices[0].numel(), 1)
+    g = None
+    if gates is not None:
+        g, s3 = planes(gates, torch.float32)
+        if s3 != s1:
+            # bring all three to one stride
+            idx = torch.stack(list(indices)).contiguous()
+            loc = torch.stack(list(locations)).contiguous()
+            g = torch.stack([t.to(torch.float32) for t in gates]).contiguous()
+            s1 = max(indices[0].numel(), 1)
+    return idx, loc, g, s1
+
+
+def dispatch_fwd(x, indices, locations, gates, experts, capacity_):
+    """[T, M] -> [experts*capacity, M]; gates=None is the all-ones helper."""
+    _need_gpu(x, "dispatch_fwd")
+    x = _contig(x, "dispatch_fwd")
+    T, M = x.shape
+    idx, loc, g, stride = _plane_args(indices, locations, gates, "dispatch_fwd")
+    out = torch.empty((experts * capacity_, M), dtype=x.dtype, device=x.device)
+    ws = _ws(lib.planmoe_dispatch_workspace_bytes(experts, capacity_), x.device)
+    check(lib.planmoe_dispatch_fwd(_ptr(x), _dt(x, "dispatch_fwd"), _ptr(g), _ptr(idx), _ptr(loc),
+                                   stride, len(indices), T, M, experts, capacity_, _ptr(out),
+                                   _ptr(ws), ws.numel(), _stream(x)))
+    return out
+
+
+def combine_fwd(dispatched, indices, locations, gates, samples, capacity_):
+    """[experts*capacity, M] -> [T, M]."""
+    _need_gpu(dispatched, "combine_fwd")
+    d = _contig(dispatched, "combine_fwd")
+    M = d.shape[-1]
+    idx, loc, g, stride = _plane_args(indices, locations, gates, "combine_fwd")
+    out = torch.empty((samples, M), dtype=d.dtype, device=d.device)
+    check(lib.planmoe_combine_fwd(_ptr(d), _dt(d, "combine_fwd"), _ptr(g), _ptr(idx), _ptr(loc), stride,
+                                  len(indices), samples, M, capacity_, _ptr(out), _stream(d)))
+    return out
+
+
+def bwd_gate(x, dispatched, indices, locations, capacity_):
+    """grad_gates[k, T] (fp32) = <dispatched[slot], x[t]>."""
+    _need_gpu(x, "bwd_gate")
+    x = _contig(x, "bwd_gate")
+    d = _contig(dispatched, "bwd_gate")
+    if x.dtype != d.dtype:
+        raise PlanMoEError("bwd_gate: x and dispatched must share a dtype")
+    T, M = x.shape
+    idx, loc, _, stride = _plane_args(indices, locations, None, "bwd_gate")
+    k = len(indices)
+    out = torch.empty((k, stride), dtype=torch.float32, device=x.device)
+    check(lib.planmoe_bwd_gate(_ptr(x), _ptr(d), _dt(x, "bwd_gate"), _ptr(idx), _ptr(loc), stride, k, T,
+                               M, capacity_, _ptr(out), _stream(x)))
+    return out[:, :T]
+
+
+# ------------------------------------------------------------------------------ "int8" codec
+def int8_compress(x):
+    """x [..., M] -> codes uint8 [..., M], bias [..., 1], scale [..., 1] (x's dtype)."""
+    _need_gpu(x, "int8_compress")
+    x = _contig(x, "int8_compress")
+    M = x.shape[-1]
+    rows = x.numel() // M if M else 0
+    codes = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    bias = torch.empty(x.shape[:-1] + (1,), dtype=x.dtype, device=x.device)
+    scale = torch.empty_like(bias)
+    check(lib.planmoe_int8_compress(_ptr(x), _dt(x, "int8_compress"), rows, M, _ptr(codes), _ptr(bias),
+                                    _ptr(scale), _stream(x)))
+    return codes, bias, scale
+
+
+def int8_decompress(codes, bias, scale):
+    _need_gpu(codes, "int8_decompress")
+    codes = _contig(codes, "int8_decompress")
+    M = codes.shape[-1]
+    rows = codes.numel() // M if M else 0
+    out = torch.empty(codes.shape, dtype=bias.dtype, device=codes.device)
+    check(lib.planmoe_int8_decompress(_ptr(codes), _ptr(bias.contiguous()), _ptr(scale.contiguous()),
+                                      _dt(bias, "int8_decompress"), rows, M, _ptr(out), _stream(codes)))
+    return out
+
+
+def dispatch_int8(x, indices, locations, gates, experts, capacity_):
+    """fast_encode followed by the int8 compressor, in one pass.
+    Returns codes [experts*capacity, M] uint8, bias, scale [experts*capacity, 1]."""
+    _need_gpu(x, "dispatch_int8")
+    x = _contig(x, "dispatch_int8")
+    T, M = x.shape
+    idx, loc, g, stride = _plane_args(indices, locations, gates, "dispatch_int8")
+    R = experts * capacity_
+    codes = torch.empty((R, M), dtype=torch.uint8, device=x.device)
+    bias = torch.empty((R, 1), dtype=x.dtype, device=x.device)
+    scale = torch.empty_like(bias)
+    ws = _ws(lib.planmoe_dispatch_workspace_bytes(experts, capacity_), x.device)
+    check(lib.planmoe_dispatch_int8(_ptr(x), _dt(x, "dispatch_int8"), _ptr(g), _ptr(idx), _ptr(loc),
+                                    stride, len(indices), T, M, experts, capacity_, _ptr(codes),
+                                    _ptr(bias), _ptr(scale), _ptr(ws), ws.numel(), _stream(x)))
+    return codes, bias, scale
+
+
+# ------------------------------------------------------------------------------ zfp codec
+def zfp_stream_bytes(dims, nx, ny, rate=8.0):
+    return int(lib.planmoe_zfp_stream_bytes(dims, nx, ny, float(rate)))
+
+
+def zfp_max_bytes(dims, nx, ny, rate=8.0):
+    return int(lib.planmoe_zfp_max_bytes(dims, nx, ny, float(rate)))
+
+
+def zfp_compress(field, nx, ny, dims=2, rate=8.0, out=None):
+    """field: fp32 storage holding ny rows of nx values.  Returns a uint8 tensor of
+    zfp_max_bytes (what the reference allocates) whose first zfp_stream_bytes are the stream."""
+    _need_gpu(field, "zfp_compress")
+    field = _contig(field, "zfp_compress")
+    if out is None:
+        out = torch.zeros((zfp_max_bytes(dims, nx, ny, rate),), dtype=torch.uint8, device=field.device)
+    check(lib.planmoe_zfp_compress(_ptr(field), dims, nx, ny, float(rate), _ptr(out), out.numel(),
+                                   _stream(field)))
+    return out
+
+
+def zfp_decompress(stream, nx, ny, dims=2, rate=8.0):
+    _need_gpu(stream, "zfp_decompress")
+    out = torch.empty((ny, nx), dtype=torch.float32, device=stream.device)
+    check(lib.planmoe_zfp_decompress(_ptr(stream), dims, nx, ny, float(rate), _ptr(out), _stream(stream)))
+    return out
