@@ -223,3 +223,16 @@ def zfp_decompress(stream, ny, nx, dims=2, rate=8.0):
     if rc != 0:
         raise ValueError("zfp fails.")
     return out
+
+
+def zfp_encode_block(block, dims=2, rate=8.0):
+    """One block through the block coder: float32 input -> float path, int32 input -> integer
+    path (the library's zfp_encode_block_float_N / zfp_encode_block_int32_N).  64-byte buffer."""
+    out = np.zeros((64,), np.uint8)
+    if block.dtype == np.int32:
+        lib().orc_zfp_encode_block_int32(_p(_c(block, np.int32)), ctypes.c_int(dims),
+                                         ctypes.c_double(rate), _p(out))
+    else:
+        lib().orc_zfp_encode_block_float(_p(_c(block, np.float32)), ctypes.c_int(dims),
+                                         ctypes.c_double(rate), _p(out))
+    return out

@@ -279,7 +279,10 @@ ORC_API void orc_int8_compress_f32(const float *x, int64_t rows, int row_len, ui
     for (int64_t r = 0; r < rows; ++r) {
         const float *p = x + r * row_len;
         float mn = p[0], mx = p[0];
-        for (int j = 1; j < row_len; ++j) { if (p[j] < mn) mn = p[j]; if (p[j] > mx) mx = p[j]; }
+        for (int j = 1; j < row_len; ++j) {
+            if (p[j] < mn || p[j] != p[j]) mn = p[j];   /* torch.min / max keep a NaN */
+            if (p[j] > mx || p[j] != p[j]) mx = p[j];
+        }
         float sc = mx - mn;
         bias[r] = mn; scale[r] = sc;
         for (int j = 0; j < row_len; ++j) {
@@ -299,8 +302,8 @@ ORC_API void orc_int8_compress_bf16(const uint16_t *x, int64_t rows, int row_len
         float mn = bf16_to_f32(p[0]), mx = mn;
         for (int j = 1; j < row_len; ++j) {
             float v = bf16_to_f32(p[j]);
-            if (v < mn) mn = v;
-            if (v > mx) mx = v;
+            if (v < mn || v != v) mn = v;
+            if (v > mx || v != v) mx = v;
         }
         float sc = rbf(mx - mn);
         bias[r] = f32_to_bf16(mn); scale[r] = f32_to_bf16(sc);
@@ -394,6 +397,7 @@ static void inv_lift(int32_t *p, int s)
 static const uint8_t PERM1[4] = {0, 1, 2, 3};
 static const uint8_t PERM2[16] = {0, 1, 4, 5, 2, 8, 6, 9, 3, 12, 10, 7, 13, 11, 14, 15};
 
+
 static int zfp_maxbits(int dims, double rate)
 {
     int n = dims == 1 ? 4 : 16;
@@ -402,29 +406,14 @@ static int zfp_maxbits(int dims, double rate)
     return bits;
 }
 
-static void zfp_encode_block(bitw_t *w, const float *f, int dims, int maxbits)
+/* integer block: lifting transform, negabinary reorder, embedded coding of at most `budget`
+ * bits with precision `prec` (zfp's encode_block for Int = int32) */
+static void zfp_encode_iblock(bitw_t *w, const int32_t *iblock, int dims, int budget, int prec)
 {
     const int n = dims == 1 ? 4 : 16;
     const uint8_t *perm = dims == 1 ? PERM1 : PERM2;
-    const uint64_t start = w->bitpos;
-    float m = 0.f;
-    for (int i = 0; i < n; ++i) { float a = fabsf(f[i]); if (a > m) m = a; }
-    int emax = -127;
-    if (m > 0.f) { int e; frexpf(m, &e); emax = e > -126 ? e : -126; }
-    int prec = emax + 1074 + 2 * (dims + 1);
-    if (prec > 64) prec = 64;
-    if (prec < 0) prec = 0;
-    uint32_t e = prec ? (uint32_t)(emax + 127) : 0u;
-    if (!e) { w->bitpos = start + (uint64_t)maxbits; return; }   /* '0' flag + zero padding */
-    put_bits(w, 2u * e + 1u, 9);
-
     int32_t q[16];
-    float s = ldexpf(1.0f, 30 - emax);
-    for (int i = 0; i < n; ++i) {
-        float v = f[i] * s;
-        /* out-of-range products take the x86 conversion result (INT_MIN) */
-        q[i] = (v >= 2147483648.0f || v < -2147483648.0f || v != v) ? INT32_MIN : (int32_t)v;
-    }
+    for (int i = 0; i < n; ++i) q[i] = iblock[i];
     if (dims == 1) fwd_lift(q, 1);
     else {
         for (int y = 0; y < 4; ++y) fwd_lift(q + 4 * y, 1);
@@ -434,7 +423,7 @@ static void zfp_encode_block(bitw_t *w, const float *f, int dims, int maxbits)
     for (int i = 0; i < n; ++i)
         u[i] = ((uint32_t)q[perm[i]] + 0xaaaaaaaau) ^ 0xaaaaaaaau;
 
-    int bits = maxbits - 9;
+    int bits = budget;
     int kmin = prec >= 32 ? 0 : 32 - prec;
     int nsig = 0;
     for (int k = 31; bits > 0 && k >= kmin; --k) {
@@ -455,7 +444,46 @@ static void zfp_encode_block(bitw_t *w, const float *f, int dims, int maxbits)
             x >>= 1; nsig++;
         }
     }
+}
+
+static void zfp_encode_block(bitw_t *w, const float *f, int dims, int maxbits)
+{
+    const int n = dims == 1 ? 4 : 16;
+    const uint64_t start = w->bitpos;
+    float m = 0.f;
+    for (int i = 0; i < n; ++i) { float a = fabsf(f[i]); if (a > m) m = a; }
+    int emax = -127;
+    if (m > 0.f) { int e; frexpf(m, &e); emax = e > -126 ? e : -126; }
+    int prec = emax + 1074 + 2 * (dims + 1);
+    if (prec > 64) prec = 64;
+    if (prec < 0) prec = 0;
+    uint32_t e = prec ? (uint32_t)(emax + 127) : 0u;
+    if (!e) { w->bitpos = start + (uint64_t)maxbits; return; }   /* '0' flag + zero padding */
+    put_bits(w, 2u * e + 1u, 9);
+
+    int32_t q[16];
+    float s = ldexpf(1.0f, 30 - emax);
+    for (int i = 0; i < n; ++i) {
+        float v = f[i] * s;
+        /* out-of-range products take the x86 conversion result (INT_MIN) */
+        q[i] = (v >= 2147483648.0f || v < -2147483648.0f || v != v) ? INT32_MIN : (int32_t)v;
+    }
+    zfp_encode_iblock(w, q, dims, maxbits - 9, prec);
     w->bitpos = start + (uint64_t)maxbits;
+}
+
+/* single-block entry points mirroring zfp_encode_block_float_{1,2} and
+ * zfp_encode_block_int32_{1,2} of the library (fixed rate; out zero-initialised, >= 64 bytes).
+ * The integer variant has the whole maxbits as budget and full precision. */
+ORC_API void orc_zfp_encode_block_float(const float *block, int dims, double rate, uint8_t *out)
+{
+    bitw_t w = {out, 0};
+    zfp_encode_block(&w, block, dims, zfp_maxbits(dims, rate));
+}
+ORC_API void orc_zfp_encode_block_int32(const int32_t *block, int dims, double rate, uint8_t *out)
+{
+    bitw_t w = {out, 0};
+    zfp_encode_iblock(&w, block, dims, zfp_maxbits(dims, rate), 32);
 }
 
 static void zfp_decode_block(const uint8_t *base, uint64_t start, float *f, int dims, int maxbits)

@@ -1,0 +1,161 @@
+"""Routing and dispatch/combine API -- mirror of the reference's impls/fast_dispatch.py.
+
+Same names, arguments, defaults and return structure; the work is done by libplanmoe_hip
+(one launch for all k choices instead of one JIT kernel launch per choice)."""
+import torch
+
+from . import losses, ops
+from ._lib import PlanMoEError
+from .gating import fast_cumsum_sub_one  # noqa: F401  (re-exported like the reference)
+
+
+class GatingEncoder(torch.autograd.Function):
+    """fast_dispatch.py:16-46: forward = dispatch; backward = combine (+ gate gradient when
+    real gates were passed)."""
+
+    @staticmethod
+    def forward(ctx, config, reshaped_input, *gates_):
+        ctx.reshaped_input = reshaped_input
+        ctx.config = config
+        ctx.gates = list(gates_) if gates_ else None
+        return ops.dispatch_fwd(reshaped_input, config.indices_, config.locations_, ctx.gates,
+                                config.num_global_experts, config.capacity)
+
+    @staticmethod
+    def backward(ctx, dispatched_input):
+        cfg = ctx.config
+        dispatched_input = dispatched_input.contiguous()
+        grad_data = ops.combine_fwd(dispatched_input, cfg.indices_, cfg.locations_, ctx.gates,
+                                    cfg.sample_size, cfg.capacity)
+        grad_gates = []
+        if ctx.gates is not None:
+            gg = ops.bwd_gate(ctx.reshaped_input, dispatched_input, cfg.indices_, cfg.locations_,
+                              cfg.capacity)
+            grad_gates = [gg[j] for j in range(len(cfg.indices_))]
+        return (None, grad_data, *grad_gates)
+
+
+class GatingDecoder(torch.autograd.Function):
+    """fast_dispatch.py:49-79: forward = combine; backward = dispatch of the gated gradient
+    (+ gate gradient when real gates were passed)."""
+
+    @staticmethod
+    def forward(ctx, config, expert_output, *gates_):
+        ctx.expert_output = expert_output
+        ctx.config = config
+        ctx.gates = list(gates_) if gates_ else None
+        return ops.combine_fwd(expert_output, config.indices_, config.locations_, ctx.gates,
+                               config.sample_size, config.capacity)
+
+    @staticmethod
+    def backward(ctx, combined_output):
+        cfg = ctx.config
+        combined_output = combined_output.contiguous()
+        grad_expert_output = ops.dispatch_fwd(combined_output, cfg.indices_, cfg.locations_, ctx.gates,
+                                              cfg.num_global_experts, cfg.capacity)
+        grad_gates = []
+        if ctx.gates is not None:
+            gg = ops.bwd_gate(combined_output, ctx.expert_output, cfg.indices_, cfg.locations_,
+                              cfg.capacity)
+            grad_gates = [gg[j] for j in range(len(cfg.indices_))]
+        return (None, grad_expert_output, *grad_gates)
+
+
+class TutelMoeFastDispatcher:
+    """fast_dispatch.py:82-131.  The compute dtype is fp32 for every input dtype but fp16
+    on CUDA in the reference (:91-93); here the kernels read and write the input dtype directly
+    and do the same fp32 arithmetic in registers, which gives the same bits without the two
+    full-tensor casts."""
+
+    def __init__(self, num_global_experts, capacity, model_dim, dispatch_dtype):
+        self.num_global_experts = int(num_global_experts)
+        self.capacity = int(capacity)
+        self.model_dim = int(model_dim)
+        self.dtype = torch.float32
+        self.original_dtype = dispatch_dtype
+        self.aligned_dim = model_dim
+        self.is_cuda = None
+
+    def update(self, indices_, locations_, gates_, capacity=None, is_postscore=True):
+        self.indices_ = [x.to(torch.int32).view(-1) for x in indices_]
+        self.locations_ = [x.to(torch.int32) for x in locations_]
+        self.gates_ = [x.to(self.dtype) for x in gates_]
+        self.is_postscore = is_postscore
+        self.sample_size, self.capacity = int(self.indices_[0].size(0)), int(capacity) or self.capacity
+        if not self.indices_[0].is_cuda:
+            raise PlanMoEError("fast_dispatcher: routing tensors must live on the GPU "
+                               "(this build has no CPU kernels)")
+        self.is_cuda = True
+
+    def encode(self, data):
+        data = data.to(self.original_dtype).contiguous()
+        if self.is_postscore:
+            return GatingEncoder.apply(self, data)
+        return GatingEncoder.apply(self, data, *self.gates_)
+
+    def decode(self, data):
+        data = data.to(self.original_dtype).contiguous()
+        if self.is_postscore:
+            return GatingDecoder.apply(self, data, *self.gates_)
+        return GatingDecoder.apply(self, data)
+
+
+fast_dispatcher = TutelMoeFastDispatcher
+
+
+def extract_critical(scores, top_k, loss_fn=losses.gshard_loss, capacity_factor=1.0,
+                     batch_prioritized_routing=False, normalize_gate=True, group=None, alignment=1):
+    """fast_dispatch.py:140-195.  Returns ((E, indices_s, locations_s, gates_s, capacity), l_loss).
+
+    Not carried over yet: batch_prioritized_routing=True (raises) and gradients flowing from
+    the returned gates back into `scores`."""
+    if batch_prioritized_routing:
+        raise NotImplementedError("extract_critical: batch_prioritized_routing is not built yet")
+    if not scores.is_cuda:
+        raise PlanMoEError("extract_critical: scores must live on the GPU (no CPU path in this build)")
+    num_global_experts = int(scores.size(1))
+    top_k = min(top_k, num_global_experts)
+    want_kernel_loss = loss_fn is losses.gshard_loss
+    r = ops.route_topk(scores.detach().contiguous(), top_k, is_logits=False,
+                       normalize_gate=normalize_gate, want_l_aux=want_kernel_loss)
+    indices_s = [r["indices"][j] for j in range(top_k)]
+    locations_s = [r["locations"][j] for j in range(top_k)]
+    gates_s = [r["gates"][j] for j in range(top_k)]
+
+    if loss_fn is None:
+        l_loss = None
+    elif want_kernel_loss:
+        l_loss = r["l_aux"].to(scores.dtype)
+    else:
+        topk_indices = torch.stack(indices_s, dim=1).to(torch.int64)
+        l_loss = loss_fn(scores, topk_indices)
+
+    samples = int(scores.size(0))
+    if capacity_factor > 0:
+        capacity = ops.capacity(samples, num_global_experts, top_k, capacity_factor, alignment)
+    else:
+        # data-dependent capacity (fast_dispatch.py:183-186); world size 1, so no all-reduce
+        capacity = int(torch.max(r["locations"])) + 1
+        if capacity_factor < 0:
+            per_expert = (samples + num_global_experts - 1) // num_global_experts
+            capacity = min(capacity, top_k * int(-capacity_factor * per_expert))
+        remainder = capacity % alignment
+        if remainder > 0:
+            capacity = capacity + alignment - remainder
+    return (num_global_experts, indices_s, locations_s, gates_s, capacity), l_loss
+
+
+def fast_encode(data, critial_data, is_postscore=True):
+    # fast_dispatch.py:197-201
+    num_global_experts = critial_data[0]
+    dispatcher = TutelMoeFastDispatcher(num_global_experts, 0, data.size(-1), data.dtype)
+    dispatcher.update(*critial_data[1:], is_postscore=is_postscore)
+    return dispatcher.encode(data).view(num_global_experts, -1, data.size(-1))
+
+
+def fast_decode(data, critial_data, is_postscore=True):
+    # fast_dispatch.py:203-207
+    num_global_experts = critial_data[0]
+    dispatcher = TutelMoeFastDispatcher(num_global_experts, 0, data.size(-1), data.dtype)
+    dispatcher.update(*critial_data[1:], is_postscore=is_postscore)
+    return dispatcher.decode(data.reshape(-1, data.size(-1))).view(-1, data.size(-1))

@@ -195,13 +195,17 @@ def bwd_gate(x, dispatched, indices, locations, capacity_):
 
 
 # ------------------------------------------------------------------------------ "int8" codec
-def int8_compress(x):
-    """x [..., M] -> codes uint8 [..., M], bias [..., 1], scale [..., 1] (x's dtype)."""
+def int8_compress(x, codes_out=None):
+    """x [..., M] -> codes uint8 [..., M], bias [..., 1], scale [..., 1] (x's dtype).
+    codes_out: optional contiguous uint8 storage of x.numel() bytes to write the codes into."""
     _need_gpu(x, "int8_compress")
     x = _contig(x, "int8_compress")
     M = x.shape[-1]
     rows = x.numel() // M if M else 0
-    codes = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    if codes_out is None:
+        codes = torch.empty(x.shape, dtype=torch.uint8, device=x.device)
+    else:
+        codes = codes_out.view(torch.uint8).reshape(-1)[:x.numel()].view(x.shape)
     bias = torch.empty(x.shape[:-1] + (1,), dtype=x.dtype, device=x.device)
     scale = torch.empty_like(bias)
     check(lib.planmoe_int8_compress(_ptr(x), _dt(x, "int8_compress"), rows, M, _ptr(codes), _ptr(bias),

@@ -1,0 +1,150 @@
+"""GPU parity: gate-logits GEMM (MFMA), the fused forward chain of config 2 and the
+moe_layer mirror end to end."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import bf16_bits, np_raw, raw, to_np, zipf_bias
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("T,M,E,dtype", [(100, 512, 8, torch.bfloat16), (1000, 4096, 8, torch.bfloat16), (777, 2048, 64, torch.bfloat16),
+                                         (100, 2048, 2, torch.float32), (50, 100, 5, torch.float32), (50, 1000, 20, torch.float32),
+                                         (31, 136, 17, torch.bfloat16), (16, 4100, 8, torch.bfloat16), (10, 64, 100, torch.float32)])
+def test_gate_logits(T, M, E, dtype):
+    """fp32-accumulated logits against the oracle's fp64 dot products: rtol 1e-5 of the row scale
+    (products of bf16 values are exact in fp32, only the summation order differs)."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(T, M, generator=g).to(dtype)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).to(dtype)
+    out = ops.gate_logits(x.to(DEV), wg.to(DEV), torch.float32).cpu().numpy()
+    ref = oracle.gate_logits(to_np(x), to_np(wg))
+    mag = oracle.gate_logits(to_np(x.abs()), to_np(wg.abs()))
+    assert (np.abs(out - ref) <= 1e-5 * np.abs(ref) + 1e-6 * mag).all()
+
+
+def test_gate_logits_fp16_and_rounded_output():
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(64, 1024, generator=g).half()
+    wg = (torch.randn(33, 1024, generator=g) / 32).half()
+    out = ops.gate_logits(x.to(DEV), wg.to(DEV), torch.float32).cpu()
+    assert torch.allclose(out.double(), x.double() @ wg.double().t(), rtol=1e-5, atol=1e-5)
+    xb, wb = x.bfloat16(), wg.bfloat16()
+    o32 = ops.gate_logits(xb.to(DEV), wb.to(DEV), torch.float32)
+    o16 = ops.gate_logits(xb.to(DEV), wb.to(DEV), torch.bfloat16)
+    assert torch.equal(o16, o32.bfloat16())
+
+
+def _forward_chain(T, M, E, k, cf, seed, bias=None):
+    """gate GEMM -> softmax/top-k/slots -> dispatch+int8, every stage checked against the
+    oracle evaluated on the bits the previous HIP stage produced."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, M, generator=g).bfloat16()
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16()
+    xd, wd = x.to(DEV), wg.to(DEV)
+    logits = ops.gate_logits(xd, wd, torch.float32)
+    ref = oracle.gate_logits(bf16_bits(x), bf16_bits(wg))
+    assert np.abs(logits.cpu().numpy() - ref).max() <= 1e-5 * np.abs(ref).max()
+    r = ops.route_topk(logits, k, is_logits=True, logit_bias=bias, want_scores=True, want_counts=True)
+    scores = r["scores"].cpu()
+    lg = logits.cpu() if bias is None else logits.cpu() + bias
+    assert torch.allclose(scores, torch.softmax(lg, 1), rtol=1e-5, atol=1e-9)
+    idx, loc, gates, counts = oracle.route_topk(scores.numpy(), k)
+    assert np.array_equal(r["indices"].cpu().numpy(), idx) and np.array_equal(r["locations"].cpu().numpy(), loc)
+    assert np.array_equal(raw(r["gates"]), np_raw(gates)) and np.array_equal(r["counts"].cpu().numpy(), counts)
+    C = ops.capacity(T, E, k, cf, 4)
+    codes, b, s = ops.dispatch_int8(xd, list(r["indices"]), list(r["locations"]), None, E, C)
+    return x, idx, loc, gates, counts, C, codes, b, s
+
+
+def test_config2_forward_chain_full_size():
+    """16384 x 4096 bf16, 8 experts, top-2, cf 1.25: codes / bias / scale of the whole
+    [8, 5120, 4096] buffer against the oracle, then the int8 round trip back to tokens."""
+    from planmoe_amd import ops
+    T, M, E, k = 16384, 4096, 8, 2
+    x, idx, loc, gates, counts, C, codes, b, s = _forward_chain(T, M, E, k, 1.25, seed=0)
+    assert C == 5120
+    d = torch.from_numpy(oracle.encode(x.float().numpy(), list(idx), list(loc), None, E, C)).bfloat16()
+    rc, rb, rs = oracle.int8_compress(bf16_bits(d))
+    assert np.array_equal(codes.cpu().numpy(), rc)
+    assert np.array_equal(raw(b), np_raw(rb)) and np.array_equal(raw(s), np_raw(rs))
+    dec = ops.int8_decompress(codes, b, s)
+    assert np.array_equal(raw(dec), np_raw(oracle.int8_decompress(rc, rb, rs)))
+    # decode(int8 round trip) stays within the codec's error of x * sum(kept gates)
+    i = [torch.from_numpy(a).to(DEV) for a in idx]; l = [torch.from_numpy(a).to(DEV) for a in loc]
+    gt = [torch.from_numpy(a).to(DEV) for a in gates]
+    y = ops.combine_fwd(dec, i, l, gt, T, C).float().cpu()
+    w = torch.from_numpy(((loc < C) * gates).sum(0))
+    assert (y - x.float() * w[:, None]).abs().max() < 0.06
+
+
+def test_config3_forward_chain_full_size_zipf():
+    T, M, E = 32768, 2048, 64
+    x, idx, loc, gates, counts, C, codes, b, s = _forward_chain(T, M, E, 1, 1.0, seed=0, bias=zipf_bias(E))
+    assert C == 512
+    kept = int((loc[0] < C).sum())
+    assert kept == int(np.minimum(counts[0], C).sum()) and kept < T * 3 // 4
+    # slots past an expert's fill are empty rows: codes 0, scale 0
+    fill = np.minimum(counts[0], C)
+    occupied = (np.arange(C)[None, :] < fill[:, None]).reshape(-1)
+    sc = s.float().view(-1).cpu().numpy()
+    assert (sc[~occupied] == 0).all() and (codes.view(E * C, M)[torch.from_numpy(~occupied).to(DEV)] == 0).all()
+    # occupied rows hold their token's codes
+    rows = np.nonzero(loc[0] < C)[0][::97]
+    rc, rb, rs = oracle.int8_compress(bf16_bits(x[torch.from_numpy(rows)] + 0.0))
+    slot = idx[0][rows].astype(np.int64) * C + loc[0][rows]
+    assert np.array_equal(codes[torch.from_numpy(slot).to(DEV)].cpu().numpy(), rc)
+
+
+def test_moe_layer_forward_matches_the_oracle_composition():
+    """moe_layer with identity experts: out == decode(codec(encode(x))) assembled from the oracle."""
+    import planmoe_amd
+
+    class Identity(torch.nn.Module):
+        def update(self, ctx):
+            self.dummy = torch.nn.Parameter(torch.zeros(1, dtype=torch.bfloat16))
+
+        def forward(self, x, ctx):
+            return x
+
+    T, M, E, k = 512, 256, 4, 2
+    for compress in ("no", "int8"):
+        layer = planmoe_amd.moe_layer({'type': 'top', 'k': k, 'capacity_factor': 1.0, 'fp32_gate': True}, M,
+                                      experts={'type': 'custom', 'module': Identity(), 'count_per_node': E},
+                                      seeds=(1, 2, 3), compress_name=compress).to(DEV).eval()
+        x = torch.randn(2, T // 2, M, generator=torch.Generator().manual_seed(0)).bfloat16()
+        with torch.no_grad():
+            y = layer(x.to(DEV))
+        assert y.shape == x.shape and y.dtype == torch.bfloat16
+        from planmoe_amd import ops
+        wg = layer.gates[0].wg.weight.detach().to(torch.bfloat16)
+        logits = ops.gate_logits(x.view(T, M).to(DEV), wg.contiguous(), torch.float32)
+        r = ops.route_topk(logits, k, is_logits=True, want_scores=True)
+        idx, loc, gates, _ = oracle.route_topk(r["scores"].cpu().numpy(), k)
+        C = oracle.capacity(T, E, k, 1.0, 4)
+        d = torch.from_numpy(oracle.encode(x.view(T, M).float().numpy(), list(idx), list(loc), None, E, C)).bfloat16()
+        for _ in range(2):                                     # the pipeline applies the codec twice
+            if compress == "int8":
+                rc, rb, rs = oracle.int8_compress(bf16_bits(d))
+                d = torch.from_numpy(oracle.int8_decompress(rc, rb, rs).view(np.int16)).view(torch.bfloat16)
+        want = torch.from_numpy(oracle.decode(d.float().numpy(), list(idx), list(loc), list(gates), T, C)).bfloat16()
+        assert np.array_equal(raw(y.view(T, M)), raw(want))
+        assert abs(float(y.l_aux) - oracle.gshard_loss(r["scores"].cpu().numpy(), idx[0])) < 1e-4
+
+
+def test_moe_layer_trains_with_builtin_ffn():
+    import planmoe_amd
+    layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True}, 64,
+                                  experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 128},
+                                  seeds=(1, 2, 3), compress_name='no').to(DEV)
+    x = torch.randn(8, 32, 64, device=DEV, requires_grad=True)
+    y = layer(x)
+    (y.float().pow(2).mean() + y.l_aux).backward()
+    assert x.grad is not None and torch.isfinite(x.grad).all()
+    assert layer.experts.batched_fc1_w.grad is not None

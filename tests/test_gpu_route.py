@@ -1,0 +1,140 @@
+"""GPU parity: routing (top-k, capacity slots, gates, GShard loss) and the capacity cumsum,
+bit-exact against the CPU oracle through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from conftest import case
+from helpers import bf16_bits, np_raw, raw, random_scores, tie_free_scores, to_np, zipf_bias
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _check(scores, k, normalize=True):
+    from planmoe_amd import ops
+    r = ops.route_topk(scores.to(DEV), k, normalize_gate=normalize, want_counts=True)
+    s_np = to_np(scores)
+    idx, loc, gates, counts = oracle.route_topk(s_np, k, normalize)
+    assert np.array_equal(r["indices"].cpu().numpy(), idx)
+    assert np.array_equal(r["locations"].cpu().numpy(), loc)
+    assert np.array_equal(raw(r["gates"]), np_raw(gates))
+    assert np.array_equal(r["counts"].cpu().numpy(), counts)
+    want = oracle.gshard_loss(s_np, idx[0])
+    tol = 1e-2 if scores.dtype == torch.bfloat16 else 1e-5      # fp32 rtol 1e-5, bf16 rtol 1e-2
+    assert abs(float(r["l_aux"]) - want) <= tol * abs(want)
+    return r
+
+
+@pytest.mark.parametrize("name,k,norm", [("route_t2_e2", 2, True), ("route_t2_e8", 2, True),
+                                         ("route_t1_e64", 1, True), ("route_t3_e16_nonorm", 3, False)])
+def test_golden_fixtures(torch_golden, name, k, norm):
+    from planmoe_amd import ops
+    c = case(torch_golden, name)
+    r = ops.route_topk(torch.from_numpy(c["scores"]).to(DEV), k, normalize_gate=norm, want_counts=True)
+    assert np.array_equal(r["indices"].cpu().numpy(), c["indices"])
+    assert np.array_equal(r["locations"].cpu().numpy(), c["locations"])
+    assert np.array_equal(raw(r["gates"]), np_raw(c["gates"]))
+    assert np.array_equal(r["counts"].cpu().numpy(), c["counts"])
+    assert abs(float(r["l_aux"]) - float(c["l_aux"][0])) <= 1e-5 * abs(float(c["l_aux"][0]))
+
+
+@pytest.mark.parametrize("T,E,k", [(1, 1, 1), (7, 2, 2), (255, 8, 2), (256, 8, 2), (257, 8, 2), (1000, 64, 1),
+                                   (5000, 100, 3), (3000, 16, 16), (4097, 3, 2), (2000, 300, 2)])
+def test_against_oracle(T, E, k):
+    _check(tie_free_scores(T, E, k, seed=T + E), k)
+
+
+def test_without_gate_normalisation():
+    _check(tie_free_scores(700, 8, 2, seed=3), 2, normalize=False)
+
+
+def test_bf16_scores():
+    # bf16 scores tie almost surely; oracle and kernel share the lower-index rule
+    _check(random_scores(3000, 8, seed=4, dtype=torch.bfloat16), 2)
+
+
+def test_tied_scores_pick_lower_index_like_the_oracle():
+    s = torch.full((300, 8), 0.125)
+    s[::3, 5] = 0.25
+    _check(s, 2)
+
+
+def test_config1_full_size():
+    # 8192 tokens, 2 experts, top-2: every expert receives every token, nothing is dropped
+    r = _check(tie_free_scores(8192, 2, 2, seed=0), 2)
+    from planmoe_amd import ops
+    assert ops.capacity(8192, 2, 2, 1.0, 4) == 8192
+    assert int(r["locations"].max()) == 8191
+    assert r["counts"].sum(0).tolist() == [8192, 8192]
+
+
+def test_config2_full_size():
+    _check(tie_free_scores(16384, 8, 2, seed=0), 2)
+
+
+def test_config3_full_size_zipf_overflow():
+    from planmoe_amd import ops
+    T, E = 32768, 64
+    r = _check(tie_free_scores(T, E, 1, seed=0, bias=zipf_bias(E)), 1)
+    C = ops.capacity(T, E, 1, 1.0, 4)
+    assert C == 512
+    counts = r["counts"][0].cpu().numpy()
+    dropped = int((r["locations"][0] >= C).sum())
+    assert dropped == int(np.maximum(counts - C, 0).sum()) and dropped > T // 4
+
+
+def test_config5_full_size():
+    _check(tie_free_scores(65536, 16, 2, seed=0), 2)
+
+
+def test_logits_input_matches_scores_input():
+    """With input_is_logits the kernel's own softmax feeds the same routing: feed the scores it
+    reports back through the oracle, and compare them with an fp32 softmax within rtol 1e-5."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(8)
+    logits = torch.randn(5000, 8, generator=g) * 2
+    bias = zipf_bias(8)
+    r = ops.route_topk(logits.to(DEV), 2, is_logits=True, logit_bias=bias, want_scores=True, want_counts=True)
+    scores = r["scores"].cpu()
+    assert torch.allclose(scores, torch.softmax(logits + bias, 1), rtol=1e-5, atol=1e-8)
+    idx, loc, gates, counts = oracle.route_topk(scores.numpy(), 2)
+    assert np.array_equal(r["indices"].cpu().numpy(), idx)
+    assert np.array_equal(r["locations"].cpu().numpy(), loc)
+    assert np.array_equal(raw(r["gates"]), np_raw(gates))
+
+
+def test_empty_batch():
+    from planmoe_amd import ops
+    r = ops.route_topk(torch.zeros(0, 8, device=DEV), 2, want_counts=True)
+    assert r["indices"].shape == (2, 0) and int(r["counts"].sum()) == 0
+
+
+@pytest.mark.parametrize("T,E", [(1, 1), (5, 3), (1000, 8), (1024, 2), (4097, 64), (777, 130), (32768, 64)])
+def test_cumsum_sub_one(T, E):
+    import planmoe_amd
+    g = torch.Generator().manual_seed(T)
+    m = (torch.rand(T, E, generator=g) < 0.3).to(torch.int64)
+    out = planmoe_amd.fast_cumsum_sub_one(m.to(DEV))
+    assert out.dtype == torch.int32
+    assert np.array_equal(out.cpu().numpy(), oracle.cumsum_sub_one(m.numpy()))
+
+
+def test_extract_critical_structure():
+    import planmoe_amd
+    scores = tie_free_scores(1000, 8, 2, seed=12)
+    (E, idxs, locs, gates, C), l_aux = planmoe_amd.extract_critical(scores.to(DEV), 2, capacity_factor=1.25, alignment=4)
+    assert E == 8 and C == oracle.capacity(1000, 8, 2, 1.25, 4) and len(idxs) == len(locs) == len(gates) == 2
+    idx, loc, g, _ = oracle.route_topk(scores.numpy(), 2)
+    for j in range(2):
+        assert idxs[j].dtype == torch.int32 and locs[j].dtype == torch.int32 and gates[j].dtype == torch.float32
+        assert np.array_equal(idxs[j].cpu().numpy(), idx[j]) and np.array_equal(locs[j].cpu().numpy(), loc[j])
+        assert np.array_equal(raw(gates[j]), np_raw(g[j]))
+    assert abs(float(l_aux) - oracle.gshard_loss(scores.numpy(), idx[0])) < 1e-5
+    # data-dependent capacity (capacity_factor = 0): max location + 1, aligned
+    (_, _, _, _, C0), _ = planmoe_amd.extract_critical(scores.to(DEV), 2, capacity_factor=0, alignment=4)
+    assert C0 == (int(loc.max()) + 1 + 3) // 4 * 4
+    # custom loss callables see (scores, top-k ids [T, k])
+    (_, _, _, _, _), l2 = planmoe_amd.extract_critical(scores.to(DEV), 2, loss_fn=lambda s, ids: ids.float().mean())
+    assert abs(float(l2) - float(np.stack(list(idx), 1).mean())) < 1e-5
