@@ -36,12 +36,21 @@ inline bool dtype_ok(int dt) { return dt == PLANMOE_F32 || dt == PLANMOE_BF16 ||
 // ---------------------------------------------------------------- scalar conversions
 __device__ __forceinline__ float bf16_to_f32(uint32_t bits) { return __uint_as_float(bits << 16); }
 
-// round-to-nearest-even, NaN kept quiet: the rounding torch applies after each bf16 op
+// round-to-nearest-even float -> bf16 (the rounding torch applies after each bf16 op), done by
+// the gfx950 conversion instruction
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float  f32x2_t  __attribute__((ext_vector_type(2)));
+
 __device__ __forceinline__ uint32_t f32_to_bf16(float f)
 {
-    uint32_t u = __float_as_uint(f);
-    uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-    return ((u & 0x7fffffffu) > 0x7f800000u) ? ((u >> 16) | 0x40u) : r;
+    const __bf16 h = (__bf16)f;
+    return (uint32_t)__builtin_bit_cast(uint16_t, h);
+}
+// two values at once: lo in bits 0..15, hi in bits 16..31
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi)
+{
+    const f32x2_t p = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2_t));
 }
 
 __device__ __forceinline__ float f16_to_f32(uint32_t bits)
@@ -87,10 +96,8 @@ template <> struct Elem<PLANMOE_BF16> {
     }
     __device__ static __forceinline__ uint4 pack(const float *f)
     {
-        return make_uint4(f32_to_bf16(f[0]) | (f32_to_bf16(f[1]) << 16),
-                          f32_to_bf16(f[2]) | (f32_to_bf16(f[3]) << 16),
-                          f32_to_bf16(f[4]) | (f32_to_bf16(f[5]) << 16),
-                          f32_to_bf16(f[6]) | (f32_to_bf16(f[7]) << 16));
+        return make_uint4(f32x2_to_bf16x2(f[0], f[1]), f32x2_to_bf16x2(f[2], f[3]),
+                          f32x2_to_bf16x2(f[4], f[5]), f32x2_to_bf16x2(f[6], f[7]));
     }
     __device__ static __forceinline__ float load(const void *p, int64_t i) { return bf16_to_f32(((const uint16_t *)p)[i]); }
     __device__ static __forceinline__ void store(void *p, int64_t i, float v) { ((uint16_t *)p)[i] = (uint16_t)f32_to_bf16(v); }

@@ -73,15 +73,14 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
         mn = wave_allreduce(mn, [](float a, float b) { return nan_min(a, b); });
         mx = wave_allreduce(mx, [](float a, float b) { return nan_max(a, b); });
     };
-    auto encode = [&](const uint4 &raw, float g, float mn, float scale, uint32_t *w) {
+    auto encode = [&](const uint4 &raw, float g, const RowQuant<DT> &rq, uint32_t *w) {
         float f[V];
         E::unpack(raw, f);
 #pragma unroll
         for (int i = 0; i < V; ++i) f[i] = E::round(0.f + g * f[i]);
 #pragma unroll
         for (int i = 0; i < V / 4; ++i)
-            w[i] = quantise<DT>(f[4 * i], mn, scale) | (quantise<DT>(f[4 * i + 1], mn, scale) << 8) |
-                   (quantise<DT>(f[4 * i + 2], mn, scale) << 16) | (quantise<DT>(f[4 * i + 3], mn, scale) << 24);
+            w[i] = rq(f[4 * i]) | (rq(f[4 * i + 1]) << 8) | (rq(f[4 * i + 2]) << 16) | (rq(f[4 * i + 3]) << 24);
     };
     auto put = [&](int s, int u, const uint32_t *w) {
         uint8_t *row = codes + (int64_t)s * model_dim;
@@ -101,9 +100,10 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
             reduce(1.f, mn, mx);
             const float scale = E::round(mx - mn);
             if (lane < np && slot >= 0) { E::store(bias_out, slot, mn); E::store(scale_out, slot, scale); }
+            const RowQuant<DT> rq(mn, scale);
             auto emit = [&](int u, const uint4 &raw) {
                 uint32_t w[2];
-                encode(raw, 1.f, mn, scale, w);
+                encode(raw, 1.f, rq, w);
                 for (int j = 0; j < np; ++j) {
                     const int s = rl_i(slot, j);
                     if (s >= 0) put(s, u, w);
@@ -124,9 +124,10 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
                 reduce(g, mn, mx);
                 const float scale = E::round(mx - mn);
                 if (lane == 0) { E::store(bias_out, s, mn); E::store(scale_out, s, scale); }
+                const RowQuant<DT> rq(mn, scale);
                 auto emit = [&](int u, const uint4 &raw) {
                     uint32_t w[2];
-                    encode(raw, g, mn, scale, w);
+                    encode(raw, g, rq, w);
                     put(s, u, w);
                 };
                 if constexpr (CACHE > 0) {

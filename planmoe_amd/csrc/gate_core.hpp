@@ -37,8 +37,17 @@ template <> struct Mma<PLANMOE_F32> {
     }
 };
 
+template <int NT, int TPW>
+struct GateFrag {
+    uint4 a[TPW][4];
+    uint4 b[NT][4];
+};
+
 // Partial logits of tokens [t0, t0 + 16*TPW) against experts [0, 16*NT): wave w accumulates
-// the K steps w, w+4, ... and leaves its tiles in part[w][token][expert].
+// the K steps w, w+4, ... (a step is 16 vectors = 256 bytes of every row) and leaves its
+// tiles in part[w][token][expert].  Rows past the end of x / wg are clamped to the last valid
+// row: their products land in tile entries nobody reads.  Loads of the next step are issued
+// before the MFMAs of the current one.
 // Requires model_dim % VEC == 0 and 16-byte aligned x / wg.  Call with all 256 threads.
 template <int DT, int NT, int TPW>
 __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
@@ -50,21 +59,16 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
     const int w = threadIdx.x >> 6, l = lane_id();
     const int m = l & 15, g = l >> 4;
     const int nv = model_dim / V;                    // 16-byte vectors per row
-    const int steps = (nv + 15) / 16;
-    const int64_t row_vecs = nv;
+    const int full = nv / 16, rem = nv % 16;
 
-    const uint4 *arow[TPW];
-    const uint4 *brow[NT];
+    const uint4 *ap[TPW];
+    const uint4 *bp[NT];
 #pragma unroll
-    for (int tp = 0; tp < TPW; ++tp) {
-        const int t = t0 + tp * 16 + m;
-        arow[tp] = t < samples ? reinterpret_cast<const uint4 *>(x) + (int64_t)t * row_vecs : nullptr;
-    }
+    for (int tp = 0; tp < TPW; ++tp)
+        ap[tp] = reinterpret_cast<const uint4 *>(x) + (int64_t)min(t0 + tp * 16 + m, samples - 1) * nv + g * 4;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-        const int e = nt * 16 + m;
-        brow[nt] = e < experts ? reinterpret_cast<const uint4 *>(wg) + (int64_t)e * row_vecs : nullptr;
-    }
+    for (int nt = 0; nt < NT; ++nt)
+        bp[nt] = reinterpret_cast<const uint4 *>(wg) + (int64_t)min(nt * 16 + m, experts - 1) * nv + g * 4;
 
     f32x4 acc[TPW][NT];
 #pragma unroll
@@ -72,24 +76,61 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[tp][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-    for (int step = w; step < steps; step += 4) {
-        const int v0 = step * 16 + g * 4;
-        uint4 a[TPW][4], b[NT][4];
+    auto load = [&](GateFrag<NT, TPW> &f, int step) {
+        const int o = step * 16;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const bool in = v0 + s < nv;
+        for (int tp = 0; tp < TPW; ++tp)
 #pragma unroll
-            for (int tp = 0; tp < TPW; ++tp) a[tp][s] = (in && arow[tp]) ? arow[tp][v0 + s] : zero;
+            for (int s = 0; s < 4; ++s) f.a[tp][s] = ap[tp][o + s];
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) b[nt][s] = (in && brow[nt]) ? brow[nt][v0 + s] : zero;
-        }
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) f.b[nt][s] = bp[nt][o + s];
+    };
+    auto mma = [&](const GateFrag<NT, TPW> &f) {
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
             for (int tp = 0; tp < TPW; ++tp)
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) Mma<DT>::run(a[tp][s], b[nt][s], acc[tp][nt]);
+                for (int nt = 0; nt < NT; ++nt) Mma<DT>::run(f.a[tp][s], f.b[nt][s], acc[tp][nt]);
+    };
+
+    GateFrag<NT, TPW> f0, f1;
+    int step = w;
+    if (step < full) load(f0, step);
+    while (step < full) {
+        const bool more1 = step + 4 < full;
+        if (more1) load(f1, step + 4);
+        mma(f0);
+        if (!more1) break;
+        const bool more2 = step + 8 < full;
+        if (more2) load(f0, step + 8);
+        mma(f1);
+        step += 8;
+        if (!more2) break;
+    }
+
+    if (rem && (full & 3) == w) {
+        // last, partial step: vectors past the row end are read from a clamped index and zeroed
+        GateFrag<NT, TPW> f;
+        const int o = full * 16;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const bool in = g * 4 + s < rem;
+            const int off = in ? o + s : o - g * 4;   // out of range: re-read vector `o` of the row, then zero it
+#pragma unroll
+            for (int tp = 0; tp < TPW; ++tp) {
+                uint4 v = ap[tp][off];
+                f.a[tp][s] = in ? v : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                uint4 v = bp[nt][off];
+                f.b[nt][s] = in ? v : make_uint4(0, 0, 0, 0);
+            }
+        }
+        mma(f);
     }
 
 #pragma unroll

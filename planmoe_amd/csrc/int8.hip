@@ -56,14 +56,14 @@ __global__ __launch_bounds__(256) void int8_compress_vec_kernel(
     if (lane == 0) { E::store(bias_out, r, mn); E::store(scale_out, r, scale); }
 
     uint8_t *dst = codes + r * row_len;
+    const RowQuant<DT> rq(mn, scale);
     auto emit = [&](int u, const uint4 &raw) {
         float f[V];
         E::unpack(raw, f);
         uint32_t w[V / 4];
 #pragma unroll
         for (int i = 0; i < V / 4; ++i)
-            w[i] = quantise<DT>(f[4 * i], mn, scale) | (quantise<DT>(f[4 * i + 1], mn, scale) << 8) |
-                   (quantise<DT>(f[4 * i + 2], mn, scale) << 16) | (quantise<DT>(f[4 * i + 3], mn, scale) << 24);
+            w[i] = rq(f[4 * i]) | (rq(f[4 * i + 1]) << 8) | (rq(f[4 * i + 2]) << 16) | (rq(f[4 * i + 3]) << 24);
         if constexpr (V == 8) reinterpret_cast<uint2 *>(dst)[u] = make_uint2(w[0], w[1]);
         else reinterpret_cast<uint32_t *>(dst)[u] = w[0];
     };
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256) void int8_decompress_vec_kernel(
     const int lane = lane_id();
     const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (r >= rows) return;
-    const float bias = E::load(bias_in, r), scale = E::load(scale_in, r);
+    const RowDequant<DT> dq(E::load(bias_in, r), E::load(scale_in, r));
     const int units = row_len / V;
     const uint8_t *src = codes + r * row_len;
     uint4 *dst = reinterpret_cast<uint4 *>((char *)out + r * row_len * (int64_t)sizeof(typename E::store_t));
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(256) void int8_decompress_vec_kernel(
         else { w[0] = reinterpret_cast<const uint32_t *>(src)[u]; w[1] = 0; }
         float f[V];
 #pragma unroll
-        for (int i = 0; i < V; ++i) f[i] = dequantise<DT>((w[i / 4] >> (8 * (i % 4))) & 0xffu, bias, scale);
+        for (int i = 0; i < V; ++i) f[i] = dq((w[i / 4] >> (8 * (i % 4))) & 0xffu);
         dst[u] = E::pack(f);
     }
 }

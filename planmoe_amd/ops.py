@@ -242,6 +242,80 @@ def dispatch_int8(x, indices, locations, gates, experts, capacity_):
     return codes, bias, scale
 
 
+# ------------------------------------------------------------------------------ fused forward chain
+_forward_ws = {}
+
+
+def _forward_workspace(T, E, k, device):
+    """Per-device workspace of the fused chain, grown on demand and initialised once (its
+    completion counter must start at zero; every call leaves it at zero)."""
+    need = lib.planmoe_forward_workspace_bytes(T, E, k)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    ws = _forward_ws.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty((max(need, 1 << 20),), dtype=torch.uint8, device=device)
+        check(lib.planmoe_forward_workspace_init(_ptr(ws), ws.numel(), _stream(ws)))
+        _forward_ws[key] = ws
+    return ws
+
+
+def _forward_common(x, wg, top_k, fp32_gate, logit_bias, want_logits, want_scores, want_l_aux, want_counts):
+    _need_gpu(x, "forward")
+    x = _contig(x, "forward")
+    wg = _contig(wg, "forward")
+    if x.dtype != wg.dtype:
+        raise PlanMoEError("forward: x and wg must share a dtype")
+    T, M = x.shape
+    E = wg.shape[0]
+    k = min(int(top_k), E)
+    dev = x.device
+    sdt = torch.float32 if (fp32_gate or x.dtype == torch.float32) else x.dtype
+    out = dict(
+        indices=torch.empty((k, T), dtype=torch.int32, device=dev),
+        locations=torch.empty((k, T), dtype=torch.int32, device=dev),
+        gates=torch.empty((k, T), dtype=sdt, device=dev),
+        logits=torch.empty((T, E), dtype=sdt, device=dev) if want_logits else None,
+        scores=torch.empty((T, E), dtype=sdt, device=dev) if want_scores else None,
+        l_aux=torch.zeros((), dtype=torch.float32, device=dev) if want_l_aux else None,
+        counts=torch.empty((k, E), dtype=torch.int32, device=dev) if want_counts else None)
+    bias = None
+    if logit_bias is not None:
+        bias = logit_bias.to(device=dev, dtype=torch.float32).contiguous()
+    return x, wg, T, M, E, k, bias, out, _forward_workspace(T, E, k, dev)
+
+
+def gate_route(x, wg, top_k, fp32_gate=True, logit_bias=None, normalize_gate=True, want_logits=False,
+               want_scores=False, want_l_aux=True, want_counts=False):
+    """Gate GEMM + softmax + top-k routing in two launches (experts <= 64)."""
+    x, wg, T, M, E, k, bias, out, ws = _forward_common(x, wg, top_k, fp32_gate, logit_bias, want_logits,
+                                                       want_scores, want_l_aux, want_counts)
+    check(lib.planmoe_gate_route(_ptr(x), _ptr(wg), _dt(x, "gate_route"), int(bool(fp32_gate)), _ptr(bias),
+                                 T, M, E, k, int(bool(normalize_gate)), _ptr(out["indices"]),
+                                 _ptr(out["locations"]), _ptr(out["gates"]), max(T, 1), _ptr(out["logits"]),
+                                 _ptr(out["scores"]), _ptr(out["l_aux"]), _ptr(out["counts"]), _ptr(ws),
+                                 ws.numel(), _stream(x)))
+    return out
+
+
+def forward_int8(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
+                 want_logits=False, want_scores=False, want_l_aux=True, want_counts=False):
+    """Gate GEMM + routing + dispatch + int8 compress in two launches.  Adds codes
+    [E*capacity, M] uint8 and bias / scale [E*capacity, 1] to gate_route's outputs."""
+    x, wg, T, M, E, k, bias, out, ws = _forward_common(x, wg, top_k, fp32_gate, logit_bias, want_logits,
+                                                       want_scores, want_l_aux, want_counts)
+    R = E * capacity_
+    out["codes"] = torch.empty((R, M), dtype=torch.uint8, device=x.device)
+    out["bias"] = torch.empty((R, 1), dtype=x.dtype, device=x.device)
+    out["scale"] = torch.empty((R, 1), dtype=x.dtype, device=x.device)
+    check(lib.planmoe_forward_int8(_ptr(x), _ptr(wg), _dt(x, "forward_int8"), int(bool(fp32_gate)), _ptr(bias),
+                                   T, M, E, k, int(bool(normalize_gate)), capacity_, _ptr(out["indices"]),
+                                   _ptr(out["locations"]), _ptr(out["gates"]), max(T, 1), _ptr(out["logits"]),
+                                   _ptr(out["scores"]), _ptr(out["l_aux"]), _ptr(out["counts"]),
+                                   _ptr(out["codes"]), _ptr(out["bias"]), _ptr(out["scale"]), _ptr(ws),
+                                   ws.numel(), _stream(x)))
+    return out
+
+
 # ------------------------------------------------------------------------------ zfp codec
 def zfp_stream_bytes(dims, nx, ny, rate=8.0):
     return int(lib.planmoe_zfp_stream_bytes(dims, nx, ny, float(rate)))

@@ -148,3 +148,51 @@ def test_moe_layer_trains_with_builtin_ffn():
     (y.float().pow(2).mean() + y.l_aux).backward()
     assert x.grad is not None and torch.isfinite(x.grad).all()
     assert layer.experts.batched_fc1_w.grad is not None
+
+
+@pytest.mark.parametrize("T,M,E,k,cf,dtype,fp32_gate,use_bias", [
+    (1000, 512, 8, 2, 1.25, torch.bfloat16, True, False), (33, 256, 4, 2, 1.0, torch.bfloat16, True, False),
+    (4096, 1024, 64, 1, 1.0, torch.bfloat16, True, True), (500, 2048, 2, 2, 1.0, torch.float32, True, False),
+    (700, 264, 16, 3, 0.5, torch.bfloat16, False, False), (257, 128, 33, 4, 1.0, torch.float16, True, False),
+    (31, 64, 5, 5, 2.0, torch.float32, False, True)])
+def test_fused_forward_matches_unfused_and_oracle(T, M, E, k, cf, dtype, fp32_gate, use_bias):
+    """planmoe_forward_int8 / planmoe_gate_route against the stage-by-stage entry points and the
+    oracle (routing evaluated on the scores the kernel reports)."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(T + E)
+    x = torch.randn(T, M, generator=g).to(dtype).to(DEV)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).to(dtype).to(DEV)
+    bias = zipf_bias(E) if use_bias else None
+    C = ops.capacity(T, E, k, cf, 4)
+    sdt = torch.float32 if (fp32_gate or dtype == torch.float32) else dtype
+    for rep in range(2):                    # twice: the workspace counter must come back to zero
+        out = ops.forward_int8(x, wg, k, C, fp32_gate=fp32_gate, logit_bias=bias, want_logits=True,
+                               want_scores=True, want_counts=True)
+        assert torch.equal(out["logits"], ops.gate_logits(x, wg, sdt))
+        scores = out["scores"]
+        assert scores.dtype == sdt and out["gates"].dtype == sdt
+        lg = out["logits"].float().cpu() + (bias if use_bias else 0)
+        if sdt != torch.float32:
+            lg = lg.to(sdt).float()
+        assert torch.allclose(scores.float().cpu(), torch.softmax(lg, 1), rtol=1e-5 if sdt == torch.float32 else 1e-2, atol=1e-8)
+        if sdt == torch.float16:
+            r = ops.route_topk(scores, k, want_counts=True)     # the oracle has no fp16 mode
+            idx, loc, gates, counts = (r["indices"].cpu().numpy(), r["locations"].cpu().numpy(), None, r["counts"].cpu().numpy())
+            assert torch.equal(out["gates"], r["gates"])
+        else:
+            idx, loc, gates, counts = oracle.route_topk(to_np(scores), k)
+            assert np.array_equal(raw(out["gates"]), np_raw(gates))
+        assert np.array_equal(out["indices"].cpu().numpy(), idx)
+        assert np.array_equal(out["locations"].cpu().numpy(), loc)
+        assert np.array_equal(out["counts"].cpu().numpy(), counts)
+        if sdt != torch.float16:
+            want = oracle.gshard_loss(to_np(scores), idx[0])
+            assert abs(float(out["l_aux"]) - want) <= (1e-5 if sdt == torch.float32 else 1e-2) * abs(want)
+        c2, b2, s2 = ops.dispatch_int8(x, list(out["indices"]), list(out["locations"]), None, E, C)
+        assert torch.equal(out["codes"], c2)
+        assert np.array_equal(raw(out["bias"]), raw(b2)) and np.array_equal(raw(out["scale"]), raw(s2))
+        r2 = ops.gate_route(x, wg, k, fp32_gate=fp32_gate, logit_bias=bias, want_counts=True)
+        for name in ("indices", "locations", "counts"):
+            assert torch.equal(r2[name], out[name])
+        assert np.array_equal(raw(r2["gates"]), raw(out["gates"]))
+        assert abs(float(r2["l_aux"]) - float(out["l_aux"])) == 0
