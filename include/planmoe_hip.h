@@ -153,7 +153,7 @@ int planmoe_dispatch_int8(const void *x, int dtype, const float *gates, const in
                           void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------- fused forward chain
- * The layer's forward path up to the all-to-all send buffer in two launches: gate GEMM +
+ * The layer's forward path up to the all-to-all send buffer in three launches: gate GEMM +
  * routing (gates/top.py:20-26, moe_layer.py:230-256, fast_dispatch.py:140-195), then
  * fast_encode + Int8Compressor::compress (fast_dispatch.py:197-201, int8.cpp:7-44).
  * Limits: experts <= 64, model_dim a multiple of 8 (bf16/fp16) or 4 (fp32), the all-ones gate
@@ -163,12 +163,8 @@ int planmoe_dispatch_int8(const void *x, int dtype, const float *gates, const in
  * scores and gates are fp32 (top.py:21-23); otherwise they are rounded to `dtype`.
  * gates, logits_out, scores_out are in that score dtype; logits_out / scores_out / l_aux /
  * expert_counts / logit_bias may be NULL.  Other arguments as in planmoe_route_topk.
- *
- * The workspace carries one counter that must be zero before the first call and is left zero
- * by every call: run planmoe_forward_workspace_init once after allocating it.  Calls sharing a
- * workspace must not overlap. */
+ * Limits in addition: top_k <= 16.  Calls sharing a workspace must not overlap. */
 size_t planmoe_forward_workspace_bytes(int samples, int experts, int top_k);
-int planmoe_forward_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
 
 /* gate GEMM + routing only (the outputs of planmoe_gate_logits + planmoe_route_topk) */
 int planmoe_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
@@ -186,6 +182,16 @@ int planmoe_forward_int8(const void *x, const void *wg, int dtype, int fp32_gate
                          void *gates, int64_t plane_stride, void *logits_out, void *scores_out,
                          float *l_aux, int32_t *expert_counts, uint8_t *codes, void *bias, void *scale,
                          void *workspace, size_t workspace_bytes, void *stream);
+
+/* Runs only the last launch of planmoe_forward_int8 (slot finalisation + dispatch + int8
+ * compress) again, from the state a preceding planmoe_forward_int8 call with the same shapes
+ * left in `workspace`.  Same outputs; meant for profiling that launch on its own.  It has no
+ * counterpart in the reference. */
+int planmoe_forward_int8_redispatch(const void *x, int dtype, int samples, int model_dim,
+                                    int experts, int top_k, int capacity, const int32_t *indices,
+                                    int32_t *locations, int64_t plane_stride, uint8_t *codes,
+                                    void *bias, void *scale, void *workspace, size_t workspace_bytes,
+                                    void *stream);
 
 /* ---------------------------------------------------------------- zfp fixed-rate codec
  * Replaces ZfpCompressor::compress / ::decompress (custom/compressor/zfpc.cpp:23-86), i.e.

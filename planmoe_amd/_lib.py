@@ -44,7 +44,6 @@ SIGNATURES = {
                                       c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                       c_void_p, c_size_t, c_void_p]),
     "planmoe_forward_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
-    "planmoe_forward_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),
     "planmoe_gate_route": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
                                    c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
                                    c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
@@ -52,6 +51,9 @@ SIGNATURES = {
                                      c_int, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_size_t, c_void_p]),
+    "planmoe_forward_int8_redispatch": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p,
+                                                c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                                                c_size_t, c_void_p]),
     "planmoe_zfp_max_bytes": (c_size_t, [c_int, c_int64, c_int64, c_double]),
     "planmoe_zfp_stream_bytes": (c_size_t, [c_int, c_int64, c_int64, c_double]),
     "planmoe_zfp_compress": (c_int, [c_void_p, c_int, c_int64, c_int64, c_double, c_void_p, c_size_t,

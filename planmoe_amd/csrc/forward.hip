@@ -1,11 +1,12 @@
-// The forward chain in two launches:
+// The forward chain in three launches:
 //
 //   gate_route_kernel     x is read once: gate-logits GEMM on the matrix cores, then, for the
 //                         work-group's 32 tokens, softmax, k-fold arg-max, gates, the rank of
 //                         every token among the group's tokens with the same choice, and the
-//                         group's expert histogram.  The last work-group to finish turns the
-//                         histograms into slot offsets (choice plane after choice plane) and
-//                         computes the GShard loss.
+//                         group's expert histogram.
+//   group_offsets_kernel  exclusive prefix of the histograms over groups, choice plane after
+//                         choice plane (all first choices of an expert precede its second
+//                         choices), expert totals and the GShard loss.  Tiny.
 //   dispatch_int8_routed  slot = rank in group + group offset; token rows go to uint8 codes in
 //                         their slots (x read a second time, normally from cache), slots past an
 //                         expert's fill are zero rows.  Or route_offsets_kernel when only the
@@ -14,36 +15,39 @@
 // This replaces gates/top.py:20-26 + moe_layer.py:230-256 + fast_dispatch.py:140-195 +
 // fast_encode (fast_dispatch.py:197-201) + Int8Compressor::compress (int8.cpp:7-44).
 //
-// Workspace (int32 words): [0] finished-group counter (zero before the first use, restored to
-// zero by every call), [1..15] unused, totals[E], hist[groups][k][E], me[groups][E] (fp32).
+// Workspace (32-bit words): totals[E], loss_part[64], hist[groups][k][E], offs[groups][k][E],
+// me[groups][E] (fp32), rank[k][samples] (rank of a token inside its group).
 #include "gate_core.hpp"
 #include "rows.hpp"
 #include "int8_core.hpp"
 
 namespace pm {
 
-constexpr int FWD_TPW = 2;
-constexpr int FWD_GROUP = 16 * FWD_TPW;      // tokens per work-group
-constexpr int FWD_HEADER = 16;               // int32 words before totals
+// tokens per work-group of the gate kernel (16 per MFMA row tile): more tokens per group re-use
+// every gate-weight fragment more often; the register budget allows 4 tiles up to 16 experts
+__host__ __device__ inline int fwd_group_tokens(int experts) { return experts <= 16 ? 64 : 32; }
+constexpr int FWD_LOSS_PARTS = 64;
 
 struct FwdWs {
-    int32_t *counter, *totals, *hist;
-    float *me;
+    int32_t *totals, *hist, *offs, *rank;
+    float *loss_part, *me;
 };
 __host__ __device__ inline FwdWs fwd_ws(void *ws, int groups, int k, int experts)
 {
     FwdWs w;
-    w.counter = (int32_t *)ws;
-    w.totals = w.counter + FWD_HEADER;
-    w.hist = w.totals + experts;
-    w.me = (float *)(w.hist + (size_t)groups * k * experts);
+    w.totals = (int32_t *)ws;
+    w.loss_part = (float *)(w.totals + experts);
+    w.hist = (int32_t *)(w.loss_part + FWD_LOSS_PARTS);
+    w.offs = w.hist + (size_t)groups * k * experts;
+    w.me = (float *)(w.offs + (size_t)groups * k * experts);
+    w.rank = (int32_t *)(w.me + (size_t)groups * experts);
     return w;
 }
 
 __device__ __forceinline__ uint64_t lanes_below() { return ((uint64_t)1 << lane_id()) - 1; }
 
 // SDT: dtype of logits / scores / gates (F32 when fp32_gate, else the input dtype)
-template <int DT, int SDT, int NT>
+template <int DT, int SDT, int NT, int TPW>
 __global__ __launch_bounds__(256) void gate_route_kernel(
     const void *__restrict__ x, const void *__restrict__ wg, const float *__restrict__ logit_bias,
     int samples, int model_dim, int experts, int k, int normalize_gate,
@@ -53,21 +57,20 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
 {
     using S = Elem<SDT>;
     constexpr int CAP = 16 * NT;
-    __shared__ float part[4][FWD_GROUP][CAP + 1];
+    constexpr int GROUP = 16 * TPW;
+    __shared__ float part[4][GROUP][CAP + 1];
     __shared__ int32_t s_hist[CAP];
-    __shared__ int32_t s_scan[256];
-    __shared__ int s_last;
 
     const int tid = threadIdx.x, lane = lane_id();
     const int groups = gridDim.x;
     const FwdWs ws = fwd_ws(workspace, groups, k, experts);
-    const int t0 = blockIdx.x * FWD_GROUP;
-    gate_tile_partials<DT, NT, FWD_TPW>(x, wg, t0, samples, model_dim, experts, part);
+    const int t0 = blockIdx.x * GROUP;
+    gate_tile_partials<DT, NT, TPW>(x, wg, t0, samples, model_dim, experts, part);
     __syncthreads();
 
     if (tid < WAVE) {                                  // wave 0: one lane per token of the group
         const int t = t0 + tid;
-        const bool valid = tid < FWD_GROUP && t < samples;
+        const bool valid = tid < GROUP && t < samples;
         float s[CAP];
         if (valid) {
             float mx = -INFINITY;
@@ -131,7 +134,7 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
                 if (lane == leader) s_hist[le] = __popcll(m);
                 todo &= ~m;
             }
-            if (valid) locations[(int64_t)j * stride + t] = rank;
+            if (valid) ws.rank[(int64_t)j * samples + t] = rank;
             __builtin_amdgcn_wave_barrier();
             if (lane < experts) ws.hist[((int64_t)blockIdx.x * k + j) * experts + lane] = s_hist[lane];
         }
@@ -146,85 +149,144 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
         }
     }
 
-    // ---- the last group to arrive scans the histograms of all groups
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const int ticket = atomicAdd(ws.counter, 1);
-        s_last = (ticket == groups - 1);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
+}
 
-    int lanes_e = 1; while (lanes_e < experts) lanes_e <<= 1;      // experts <= 64
-    const int chunks = 256 / lanes_e;
-    const int e = tid % lanes_e, ch = tid / lanes_e;
-    const bool live = e < experts;
-    const int per = (groups + chunks - 1) / chunks;
-    const int g0 = min(ch * per, groups), g1 = min(g0 + per, groups);
-    int32_t carry = 0, count0 = 0;
-    for (int j = 0; j < k; ++j) {
-        int32_t sum = 0;
-        if (live)
-            for (int g = g0; g < g1; ++g) sum += ws.hist[((int64_t)g * k + j) * experts + e];
-        s_scan[tid] = sum;
-        __syncthreads();
-        int32_t before = 0, total = 0;
-        for (int c = 0; c < chunks; ++c) {
-            const int32_t v = s_scan[c * lanes_e + e];
-            before += (c < ch) ? v : 0;
-            total += v;
-        }
-        if (live) {
-            int32_t run = carry + before;
-            for (int g = g0; g < g1; ++g) {
-                const int64_t o = ((int64_t)g * k + j) * experts + e;
-                const int32_t v = ws.hist[o];
-                ws.hist[o] = run;
-                run += v;
+// One block per set of experts (all k planes of an expert stay together): 16 column lanes
+// (plane, expert) x 16 row lanes over the groups.  offs[g][j][e] = slots of expert e taken
+// before group g of plane j = all of planes < j + groups < g of plane j.
+constexpr int GO_COLS = 16, GO_ROWS = 16, GO_BATCH = 16, GO_KEEP = 32;
+
+__global__ __launch_bounds__(256) void group_offsets_kernel(
+    const int32_t *__restrict__ hist, int32_t *__restrict__ offs, const float *__restrict__ me,
+    int groups, int k, int experts, int experts_per_block, int samples,
+    int32_t *__restrict__ totals, int32_t *__restrict__ counts_out, float *__restrict__ loss_part,
+    int want_loss)
+{
+    __shared__ int32_t s_sum[GO_ROWS][GO_COLS];
+    __shared__ int32_t s_tot[GO_COLS];
+    __shared__ float s_me[GO_ROWS][GO_COLS];
+    const int cl = threadIdx.x % GO_COLS, rl = threadIdx.x / GO_COLS;
+    const int e0 = blockIdx.x * experts_per_block;
+    const int ne = min(experts_per_block, experts - e0);
+    // column cl = plane j, expert e0 + el, planes outermost so that plane 0 comes first
+    const int j = cl / experts_per_block, el = cl - j * experts_per_block;
+    const bool live = j < k && el < ne;
+    const int e = e0 + el;
+    const int per = (groups + GO_ROWS - 1) / GO_ROWS;
+    const int g0 = min(rl * per, groups), g1 = min(g0 + per, groups);
+
+    int32_t sum = 0;
+    float mes = 0.f;
+    int32_t keep[GO_KEEP];                               // this thread's rows, when they fit
+    const bool kept = per <= GO_KEEP;
+    if (live) {
+        if (kept) {
+#pragma unroll
+            for (int i = 0; i < GO_KEEP; ++i)
+                keep[i] = (g0 + i < g1) ? hist[((int64_t)(g0 + i) * k + j) * experts + e] : 0;
+#pragma unroll
+            for (int i = 0; i < GO_KEEP; ++i) sum += keep[i];
+        } else {
+            for (int g = g0; g < g1; g += GO_BATCH) {
+                int32_t v[GO_BATCH];
+#pragma unroll
+                for (int i = 0; i < GO_BATCH; ++i)
+                    v[i] = (g + i < g1) ? hist[((int64_t)(g + i) * k + j) * experts + e] : 0;
+#pragma unroll
+                for (int i = 0; i < GO_BATCH; ++i) sum += v[i];
             }
-            if (ch == 0 && counts_out) counts_out[j * experts + e] = total;
         }
-        if (j == 0) count0 = total;
-        carry += total;
-        __syncthreads();
+        if (want_loss && j == 0) {
+            for (int g = g0; g < g1; g += GO_BATCH) {
+                float v[GO_BATCH];
+#pragma unroll
+                for (int i = 0; i < GO_BATCH; ++i) v[i] = (g + i < g1) ? me[(int64_t)(g + i) * experts + e] : 0.f;
+#pragma unroll
+                for (int i = 0; i < GO_BATCH; ++i) mes += v[i];
+            }
+        }
     }
-    if (live && ch == 0) ws.totals[e] = carry;
-    if (l_aux) {
-        // l_aux = sum_e(me[e] * ce[e]) / T with ce[e] = count0[e] * (E / T)
-        float mes = 0.f;
-        if (live)
-            for (int g = g0; g < g1; ++g) mes += ws.me[(int64_t)g * experts + e];
-        float *f_scan = reinterpret_cast<float *>(s_scan);
-        f_scan[tid] = mes;
-        __syncthreads();
-        if (tid < WAVE) {
+    s_sum[rl][cl] = sum;
+    s_me[rl][cl] = mes;
+    __syncthreads();
+    int32_t before = 0, total = 0;
+#pragma unroll
+    for (int r = 0; r < GO_ROWS; ++r) {
+        const int32_t v = s_sum[r][cl];
+        before += (r < rl) ? v : 0;
+        total += v;
+    }
+    if (rl == 0) s_tot[cl] = total;
+    __syncthreads();
+    int32_t base = 0;                                   // slots taken by the planes before j
+    for (int p = 0; p < j; ++p) base += s_tot[p * experts_per_block + el];
+    if (live) {
+        int32_t run = base + before;
+        if (kept) {
+#pragma unroll
+            for (int i = 0; i < GO_KEEP; ++i) {
+                if (g0 + i < g1) offs[((int64_t)(g0 + i) * k + j) * experts + e] = run;
+                run += keep[i];
+            }
+        } else {
+            for (int g = g0; g < g1; g += GO_BATCH) {
+                int32_t v[GO_BATCH];
+#pragma unroll
+                for (int i = 0; i < GO_BATCH; ++i)
+                    v[i] = (g + i < g1) ? hist[((int64_t)(g + i) * k + j) * experts + e] : 0;
+#pragma unroll
+                for (int i = 0; i < GO_BATCH; ++i) {
+                    if (g + i < g1) offs[((int64_t)(g + i) * k + j) * experts + e] = run;
+                    run += v[i];
+                }
+            }
+        }
+        if (rl == 0) {
+            if (counts_out) counts_out[j * experts + e] = total;
+            if (j == k - 1) totals[e] = base + total;
+        }
+    }
+    if (want_loss) {
+        // this block's share of sum_e(me[e] * ce[e]) / T, ce[e] = count0[e] * (E / T)
+        if (threadIdx.x < WAVE) {
             float acc = 0.f;
-            if (tid < experts) {
-                float me = 0.f;
-                for (int c = 0; c < chunks; ++c) me += f_scan[c * lanes_e + tid];
-                // count0 of expert `tid` lives in thread (ch 0, e = tid) == this thread
-                acc = me * ((float)count0 * ((float)experts / (float)samples));
+            if (threadIdx.x < ne) {
+                float m = 0.f;
+#pragma unroll
+                for (int r = 0; r < GO_ROWS; ++r) m += s_me[r][threadIdx.x];
+                acc = m * ((float)s_tot[threadIdx.x] * ((float)experts / (float)samples));
             }
             acc = wave_sum(acc);
-            if (tid == 0) *l_aux = acc / (float)samples;
+            if (threadIdx.x == 0) loss_part[blockIdx.x] = acc;
         }
     }
-    if (tid == 0) *ws.counter = 0;                     // ready for the next call
+}
+
+// l_aux = (sum of the per-block shares) / T, written by one thread of the launch
+__device__ __forceinline__ void finish_loss(const float *loss_part, int loss_parts, int samples, float *l_aux)
+{
+    if (l_aux && blockIdx.x == 0 && threadIdx.x == 0) {
+        float a = 0.f;
+        for (int b = 0; b < loss_parts; ++b) a += loss_part[b];
+        *l_aux = a / (float)samples;
+    }
 }
 
 // locations += offset of the token's group (routing only, no dispatch)
 __global__ __launch_bounds__(256) void route_offsets_kernel(const int32_t *__restrict__ indices,
                                                             int32_t *__restrict__ locations,
                                                             int64_t stride, int samples, int experts,
-                                                            int k, const int32_t *__restrict__ hist)
+                                                            int k, const int32_t *__restrict__ hist,
+                                                            const int32_t *__restrict__ rank, int group_tokens,
+                                                            const float *__restrict__ loss_part,
+                                                            int loss_parts, float *__restrict__ l_aux)
 {
+    finish_loss(loss_part, loss_parts, samples, l_aux);
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= samples * k) return;
     const int j = i / samples, t = i - j * samples;
     const int64_t o = (int64_t)j * stride + t;
-    locations[o] += hist[((int64_t)(t / FWD_GROUP) * k + j) * experts + indices[o]];
+    locations[o] = rank[i] + hist[((int64_t)(t / group_tokens) * k + j) * experts + indices[o]];
 }
 
 // Dispatch + int8 with the slot offsets still to be added (see dispatch_int8_kernel for the
@@ -234,12 +296,15 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     const void *__restrict__ x, const int32_t *__restrict__ indices, int32_t *__restrict__ locations,
     int64_t stride, int top_k, int samples, int model_dim, int experts, int capacity,
     uint8_t *__restrict__ codes, void *__restrict__ bias_out, void *__restrict__ scale_out,
-    const int32_t *__restrict__ hist, const int32_t *__restrict__ totals, int token_blocks)
+    const int32_t *__restrict__ hist, const int32_t *__restrict__ totals, const int32_t *__restrict__ rank,
+    int group_tokens, int token_blocks, const float *__restrict__ loss_part, int loss_parts,
+    float *__restrict__ l_aux)
 {
     using E = Elem<DT>;
     constexpr int V = E::VEC;
     const int wave = threadIdx.x >> 6, lane = lane_id();
     const int units = model_dim / V;
+    finish_loss(loss_part, loss_parts, samples, l_aux);
 
     if ((int)blockIdx.x >= token_blocks) {
         const int slots = experts * capacity;
@@ -257,8 +322,10 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
         return;
     }
 
-    const int t = blockIdx.x * 4 + wave;
-    if (t >= samples) return;
+    // tokens are walked from the last to the first: the rows the gate kernel read most recently
+    // are the likeliest to still sit in cache
+    const int t = samples - 1 - (int)(blockIdx.x * 4 + wave);
+    if (t < 0) return;
     const uint4 *src = reinterpret_cast<const uint4 *>((const char *)x + (int64_t)t * model_dim * (int64_t)sizeof(typename E::store_t));
     uint4 cache[CACHE > 0 ? CACHE : 1];
     if constexpr (CACHE > 0) {
@@ -274,38 +341,29 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     if (lane < top_k) {
         const int64_t o = (int64_t)lane * stride + t;
         const int e = indices[o];
-        const int l = locations[o] + hist[((int64_t)(t / FWD_GROUP) * top_k + lane) * experts + e];
+        const int l = rank[(int64_t)lane * samples + t] + hist[((int64_t)(t / group_tokens) * top_k + lane) * experts + e];
         locations[o] = l;
         if (l < capacity) slot = e * capacity + l;
     }
     if (__ballot(slot >= 0) == 0) return;
 
-    float mn = INFINITY, mx = -INFINITY;
-    auto visit = [&](const uint4 &raw) {
-        float f[V];
-        E::unpack(raw, f);
-#pragma unroll
-        for (int i = 0; i < V; ++i) { const float d = 0.f + f[i]; mn = nan_min(mn, d); mx = nan_max(mx, d); }
-    };
+    RowStats<DT, true> stats;
+    stats.init();
     if constexpr (CACHE > 0) {
 #pragma unroll
-        for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) visit(cache[c]);
+        for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) stats.add(cache[c]);
     } else {
-        for (int u = lane; u < units; u += WAVE) visit(src[u]);
+        for (int u = lane; u < units; u += WAVE) stats.add(src[u]);
     }
-    mn = wave_allreduce(mn, [](float a, float b) { return nan_min(a, b); });
-    mx = wave_allreduce(mx, [](float a, float b) { return nan_max(a, b); });
+    float mn, mx;
+    stats.finish(mn, mx);
     const float scale = E::round(mx - mn);
     if (slot >= 0) { E::store(bias_out, slot, mn); E::store(scale_out, slot, scale); }
-    const RowQuant<DT> rq(mn, scale);
+    const RowEncoder<DT> enc(mn, scale);
 
     auto emit = [&](int u, const uint4 &raw) {
-        float f[V];
-        E::unpack(raw, f);
         uint32_t w[2];
-#pragma unroll
-        for (int i = 0; i < V / 4; ++i)
-            w[i] = rq(0.f + f[4 * i]) | (rq(0.f + f[4 * i + 1]) << 8) | (rq(0.f + f[4 * i + 2]) << 16) | (rq(0.f + f[4 * i + 3]) << 24);
+        enc.encode(raw, w);
         for (int j = 0; j < top_k; ++j) {
             const int s = rl_i(slot, j);
             if (s < 0) continue;
@@ -328,12 +386,12 @@ static void launch_gate_route(int experts, int groups, hipStream_t st, const voi
                               int32_t *indices, int32_t *locations, void *gates, int64_t stride,
                               void *logits_out, void *scores_out, float *l_aux, int32_t *counts, void *ws)
 {
-#define PM_GR(NT)                                                                                   \
-    gate_route_kernel<DT, SDT, NT><<<groups, 256, 0, st>>>(x, wg, bias, samples, model_dim, experts, \
+#define PM_GR(NT, TPW)                                                                                   \
+    gate_route_kernel<DT, SDT, NT, TPW><<<groups, 256, 0, st>>>(x, wg, bias, samples, model_dim, experts, \
         k, normalize, indices, locations, gates, stride, logits_out, scores_out, l_aux, counts, ws)
-    if (experts <= 16) PM_GR(1);
-    else if (experts <= 32) PM_GR(2);
-    else PM_GR(4);
+    if (experts <= 16) PM_GR(1, 4);          // TPW must equal fwd_group_tokens(experts) / 16
+    else if (experts <= 32) PM_GR(2, 2);
+    else PM_GR(4, 2);
 #undef PM_GR
 }
 
@@ -341,12 +399,14 @@ template <int DT>
 static void launch_dispatch_routed(int per_lane, unsigned grid, hipStream_t st, const void *x,
                                    const int32_t *indices, int32_t *locations, int64_t stride, int top_k,
                                    int samples, int model_dim, int experts, int capacity, uint8_t *codes,
-                                   void *bias, void *scale, const int32_t *hist, const int32_t *totals,
-                                   int token_blocks)
+                                   void *bias, void *scale, const int32_t *offs, const int32_t *totals,
+                                   const int32_t *rank, int group_tokens, int token_blocks,
+                                   const float *loss_part, int loss_parts, float *l_aux)
 {
 #define PM_DR(CACHE)                                                                                 \
     dispatch_int8_routed_kernel<DT, CACHE><<<grid, 256, 0, st>>>(x, indices, locations, stride, top_k, \
-        samples, model_dim, experts, capacity, codes, bias, scale, hist, totals, token_blocks)
+        samples, model_dim, experts, capacity, codes, bias, scale, offs, totals, rank, group_tokens,  \
+        token_blocks, loss_part, loss_parts, l_aux)
     if (per_lane <= 2) PM_DR(2);
     else if (per_lane <= 4) PM_DR(4);
     else if (per_lane <= 8) PM_DR(8);
@@ -362,7 +422,7 @@ static int fused_check(const char *who, const void *x, const void *wg, int dtype
     PM_REQUIRE(samples >= 1 && model_dim >= 1 && experts >= 1 && top_k >= 1, "%s: bad shape", who);
     PM_REQUIRE(experts <= 64, "%s: the fused path supports up to 64 experts (got %d); use "
                "planmoe_gate_logits + planmoe_route_topk", who, experts);
-    PM_REQUIRE(top_k <= 64, "%s: top_k must be <= 64", who);
+    PM_REQUIRE((top_k < experts ? top_k : experts) <= GO_COLS, "%s: the fused path supports top_k <= %d", who, GO_COLS);
     const int vec = dtype == PLANMOE_F32 ? 4 : 8;
     PM_REQUIRE(model_dim % vec == 0 && aligned16(x) && aligned16(wg),
                "%s: model_dim must be a multiple of %d and x / wg 16-byte aligned", who, vec);
@@ -371,33 +431,26 @@ static int fused_check(const char *who, const void *x, const void *wg, int dtype
     return 0;
 }
 
-} // namespace pm
+struct FwdPlan {
+    int k, groups, group_tokens, experts_per_block, blocks;
+    FwdWs ws;
+};
 
-using namespace pm;
-
-extern "C" size_t planmoe_forward_workspace_bytes(int samples, int experts, int top_k)
-{
-    if (samples <= 0 || experts <= 0 || top_k <= 0) return 256;
-    const size_t k = (size_t)(top_k < experts ? top_k : experts);
-    const size_t groups = ((size_t)samples + FWD_GROUP - 1) / FWD_GROUP;
-    return round_up((FWD_HEADER + (size_t)experts + groups * k * experts + groups * experts) * 4, 256);
-}
-
-extern "C" int planmoe_forward_workspace_init(void *workspace, size_t workspace_bytes, void *stream)
-{
-    PM_REQUIRE(workspace && workspace_bytes >= 256, "planmoe_forward_workspace_init: workspace too small");
-    fill_u32((uint32_t *)workspace, FWD_HEADER, 0u, (hipStream_t)stream);
-    PM_LAUNCH_CHECK("planmoe_forward_workspace_init");
-    return 0;
-}
-
-static int run_gate_route(const char *who, const void *x, const void *wg, int dtype, int fp32_gate,
-                          const float *logit_bias, int samples, int model_dim, int experts, int k,
+// launches gate_route_kernel and group_offsets_kernel
+static int run_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
+                          const float *logit_bias, int samples, int model_dim, int experts, int top_k,
                           int normalize_gate, int32_t *indices, int32_t *locations, void *gates,
                           int64_t stride, void *logits_out, void *scores_out, float *l_aux,
-                          int32_t *counts, void *workspace, hipStream_t st)
+                          int32_t *counts, void *workspace, hipStream_t st, FwdPlan &plan)
 {
-    const int groups = (samples + FWD_GROUP - 1) / FWD_GROUP;
+    plan.k = top_k < experts ? top_k : experts;
+    plan.group_tokens = fwd_group_tokens(experts);
+    plan.groups = (samples + plan.group_tokens - 1) / plan.group_tokens;
+    plan.experts_per_block = GO_COLS / plan.k;
+    if (plan.experts_per_block > experts) plan.experts_per_block = experts;
+    plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
+    plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts);
+    const int k = plan.k, groups = plan.groups;
     if (fp32_gate || dtype == PLANMOE_F32) {
         PM_DTYPE_SWITCH(dtype, DT, (launch_gate_route<DT, PLANMOE_F32>(
             experts, groups, st, x, wg, logit_bias, samples, model_dim, k, normalize_gate, indices,
@@ -411,8 +464,42 @@ static int run_gate_route(const char *who, const void *x, const void *wg, int dt
             model_dim, k, normalize_gate, indices, locations, gates, stride, logits_out, scores_out,
             l_aux, counts, workspace);
     }
-    (void)who;
+    group_offsets_kernel<<<plan.blocks, 256, 0, st>>>(plan.ws.hist, plan.ws.offs, plan.ws.me, groups, k,
+                                                      experts, plan.experts_per_block, samples,
+                                                      plan.ws.totals, counts, plan.ws.loss_part,
+                                                      l_aux != nullptr);
     return 0;
+}
+
+static int run_dispatch_routed(const void *x, int dtype, int samples, int model_dim, int experts,
+                               int capacity, const int32_t *indices, int32_t *locations, int64_t stride,
+                               float *l_aux, uint8_t *codes, void *bias, void *scale, const FwdPlan &plan,
+                               hipStream_t st)
+{
+    const int slots = experts * capacity;
+    const int token_blocks = (samples + 3) / 4;
+    const int fill_blocks = min((slots + 3) / 4, 2048);
+    const int vec = dtype == PLANMOE_F32 ? 4 : 8;
+    const int per_lane = (model_dim / vec + WAVE - 1) / WAVE;
+    PM_DTYPE_SWITCH(dtype, DT,
+        launch_dispatch_routed<DT>(per_lane, (unsigned)(token_blocks + fill_blocks), st, x, indices, locations,
+                                   stride, plan.k, samples, model_dim, experts, capacity, codes, bias,
+                                   scale, plan.ws.offs, plan.ws.totals, plan.ws.rank, plan.group_tokens, token_blocks,
+                                   plan.ws.loss_part, plan.blocks, l_aux));
+    return 0;
+}
+
+} // namespace pm
+
+using namespace pm;
+
+extern "C" size_t planmoe_forward_workspace_bytes(int samples, int experts, int top_k)
+{
+    if (samples <= 0 || experts <= 0 || top_k <= 0) return 256;
+    const size_t k = (size_t)(top_k < experts ? top_k : experts);
+    const size_t groups = ((size_t)samples + 31) / 32;      // upper bound over the group sizes
+    return round_up(((size_t)experts + FWD_LOSS_PARTS + 2 * groups * k * experts + groups * experts +
+                     k * (size_t)samples) * 4, 256);
 }
 
 extern "C" int planmoe_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
@@ -427,15 +514,14 @@ extern "C" int planmoe_gate_route(const void *x, const void *wg, int dtype, int 
     PM_REQUIRE(indices && locations && gates, "planmoe_gate_route: NULL output");
     PM_REQUIRE(workspace && workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
                "planmoe_gate_route: workspace too small");
-    const int k = top_k < experts ? top_k : experts;
     hipStream_t st = (hipStream_t)stream;
-    if (run_gate_route("planmoe_gate_route", x, wg, dtype, fp32_gate, logit_bias, samples, model_dim,
-                       experts, k, normalize_gate, indices, locations, gates, plane_stride, logits_out,
-                       scores_out, l_aux, expert_counts, workspace, st)) return 1;
-    const int groups = (samples + FWD_GROUP - 1) / FWD_GROUP;
-    const FwdWs ws = fwd_ws(workspace, groups, k, experts);
-    route_offsets_kernel<<<(samples * k + 255) / 256, 256, 0, st>>>(indices, locations, plane_stride,
-                                                                   samples, experts, k, ws.hist);
+    FwdPlan plan;
+    if (run_gate_route(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
+                       normalize_gate, indices, locations, gates, plane_stride, logits_out, scores_out,
+                       l_aux, expert_counts, workspace, st, plan)) return 1;
+    route_offsets_kernel<<<(samples * plan.k + 255) / 256, 256, 0, st>>>(
+        indices, locations, plane_stride, samples, experts, plan.k, plan.ws.offs, plan.ws.rank,
+        plan.group_tokens, plan.ws.loss_part, plan.blocks, l_aux);
     PM_LAUNCH_CHECK("planmoe_gate_route");
     return 0;
 }
@@ -455,22 +541,43 @@ extern "C" int planmoe_forward_int8(const void *x, const void *wg, int dtype, in
     PM_REQUIRE((uintptr_t)codes % 8 == 0, "planmoe_forward_int8: codes must be 8-byte aligned");
     PM_REQUIRE(workspace && workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
                "planmoe_forward_int8: workspace too small");
-    const int k = top_k < experts ? top_k : experts;
     hipStream_t st = (hipStream_t)stream;
-    if (run_gate_route("planmoe_forward_int8", x, wg, dtype, fp32_gate, logit_bias, samples, model_dim,
-                       experts, k, normalize_gate, indices, locations, gates, plane_stride, logits_out,
-                       scores_out, l_aux, expert_counts, workspace, st)) return 1;
-    const int groups = (samples + FWD_GROUP - 1) / FWD_GROUP;
-    const FwdWs ws = fwd_ws(workspace, groups, k, experts);
-    const int slots = experts * capacity;
-    const int token_blocks = (samples + 3) / 4;
-    const int fill_blocks = min((slots + 3) / 4, 2048);
-    const int vec = dtype == PLANMOE_F32 ? 4 : 8;
-    const int per_lane = (model_dim / vec + WAVE - 1) / WAVE;
-    PM_DTYPE_SWITCH(dtype, DT,
-        launch_dispatch_routed<DT>(per_lane, (unsigned)(token_blocks + fill_blocks), st, x, indices, locations,
-                                   plane_stride, k, samples, model_dim, experts, capacity, codes, bias,
-                                   scale, ws.hist, ws.totals, token_blocks));
+    FwdPlan plan;
+    if (run_gate_route(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
+                       normalize_gate, indices, locations, gates, plane_stride, logits_out, scores_out,
+                       l_aux, expert_counts, workspace, st, plan)) return 1;
+    if (run_dispatch_routed(x, dtype, samples, model_dim, experts, capacity, indices, locations,
+                            plane_stride, l_aux, codes, bias, scale, plan, st)) return 1;
     PM_LAUNCH_CHECK("planmoe_forward_int8");
+    return 0;
+}
+
+extern "C" int planmoe_forward_int8_redispatch(const void *x, int dtype, int samples, int model_dim,
+                                               int experts, int top_k, int capacity,
+                                               const int32_t *indices, int32_t *locations,
+                                               int64_t plane_stride, uint8_t *codes, void *bias,
+                                               void *scale, void *workspace, size_t workspace_bytes,
+                                               void *stream)
+{
+    PM_REQUIRE(dtype_ok(dtype) && samples >= 1 && experts >= 1 && experts <= 64 && top_k >= 1 && capacity >= 0,
+               "planmoe_forward_int8_redispatch: bad arguments");
+    PM_REQUIRE(x && indices && locations && codes && bias && scale && workspace,
+               "planmoe_forward_int8_redispatch: NULL argument");
+    PM_REQUIRE(workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
+               "planmoe_forward_int8_redispatch: workspace too small");
+    const int vec = dtype == PLANMOE_F32 ? 4 : 8;
+    PM_REQUIRE(model_dim % vec == 0 && aligned16(x) && (uintptr_t)codes % 8 == 0,
+               "planmoe_forward_int8_redispatch: bad alignment");
+    FwdPlan plan;
+    plan.k = top_k < experts ? top_k : experts;
+    plan.group_tokens = fwd_group_tokens(experts);
+    plan.groups = (samples + plan.group_tokens - 1) / plan.group_tokens;
+    plan.experts_per_block = GO_COLS / plan.k;
+    if (plan.experts_per_block > experts) plan.experts_per_block = experts;
+    plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
+    plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts);
+    if (run_dispatch_routed(x, dtype, samples, model_dim, experts, capacity, indices, locations,
+                            plane_stride, nullptr, codes, bias, scale, plan, (hipStream_t)stream)) return 1;
+    PM_LAUNCH_CHECK("planmoe_forward_int8_redispatch");
     return 0;
 }

@@ -95,15 +95,23 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
         if (__ballot(slot >= 0) == 0) continue;
 
         if (!gates) {
-            // one code row shared by all live choices
+            // one code row shared by all live choices; 0 + 1 * x needs no rounding
+            RowStats<DT, true> stats;
+            stats.init();
+            if constexpr (CACHE > 0) {
+#pragma unroll
+                for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) stats.add(cache[c]);
+            } else {
+                for (int u = lane; u < units; u += WAVE) stats.add(src[u]);
+            }
             float mn, mx;
-            reduce(1.f, mn, mx);
+            stats.finish(mn, mx);
             const float scale = E::round(mx - mn);
             if (lane < np && slot >= 0) { E::store(bias_out, slot, mn); E::store(scale_out, slot, scale); }
-            const RowQuant<DT> rq(mn, scale);
+            const RowEncoder<DT> enc(mn, scale);
             auto emit = [&](int u, const uint4 &raw) {
                 uint32_t w[2];
-                encode(raw, 1.f, rq, w);
+                enc.encode(raw, w);
                 for (int j = 0; j < np; ++j) {
                     const int s = rl_i(slot, j);
                     if (s >= 0) put(s, u, w);

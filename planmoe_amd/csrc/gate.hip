@@ -62,7 +62,7 @@ static void launch_gate_logits(const void *x, const void *wg, void *logits, int 
 #define PM_GATE(NT, TPW)                                                                     \
     gate_logits_kernel<DT, NT, TPW><<<(samples + 16 * TPW - 1) / (16 * TPW), 256, 0, st>>>(  \
         x, wg, logits, out_dt, samples, model_dim, experts)
-    if (experts <= 16) PM_GATE(1, 2);
+    if (experts <= 16) PM_GATE(1, 4);
     else if (experts <= 32) PM_GATE(2, 2);
     else PM_GATE(4, 2);
 #undef PM_GATE

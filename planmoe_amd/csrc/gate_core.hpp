@@ -63,12 +63,16 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
 
     const uint4 *ap[TPW];
     const uint4 *bp[NT];
+    bool bv[NT];                                     // lane holds a real gate-weight row
 #pragma unroll
     for (int tp = 0; tp < TPW; ++tp)
         ap[tp] = reinterpret_cast<const uint4 *>(x) + (int64_t)min(t0 + tp * 16 + m, samples - 1) * nv + g * 4;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
+    {
+        bv[nt] = nt * 16 + m < experts;
         bp[nt] = reinterpret_cast<const uint4 *>(wg) + (int64_t)min(nt * 16 + m, experts - 1) * nv + g * 4;
+    }
 
     f32x4 acc[TPW][NT];
 #pragma unroll
@@ -83,9 +87,14 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
 #pragma unroll
             for (int s = 0; s < 4; ++s) f.a[tp][s] = ap[tp][o + s];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
+        for (int nt = 0; nt < NT; ++nt) {
+            // lanes past the last expert skip the load: whatever their registers hold only
+            // reaches tile columns nobody reads
+            if (bv[nt]) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) f.b[nt][s] = bp[nt][o + s];
+                for (int s = 0; s < 4; ++s) f.b[nt][s] = bp[nt][o + s];
+            }
+        }
     };
     auto mma = [&](const GateFrag<NT, TPW> &f) {
 #pragma unroll

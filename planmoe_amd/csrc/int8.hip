@@ -25,7 +25,8 @@ __global__ __launch_bounds__(256) void int8_compress_vec_kernel(
     const uint4 *src = reinterpret_cast<const uint4 *>((const char *)x + r * row_len * (int64_t)sizeof(typename E::store_t));
 
     uint4 cache[CACHE > 0 ? CACHE : 1];
-    float mn = INFINITY, mx = -INFINITY;
+    RowStats<DT, false> stats;
+    stats.init();
     if constexpr (CACHE > 0) {
 #pragma unroll
         for (int c = 0; c < CACHE; ++c) {
@@ -33,37 +34,21 @@ __global__ __launch_bounds__(256) void int8_compress_vec_kernel(
             if (u < units) cache[c] = src[u];
         }
 #pragma unroll
-        for (int c = 0; c < CACHE; ++c) {
-            const int u = c * WAVE + lane;
-            if (u < units) {
-                float f[V];
-                E::unpack(cache[c], f);
-#pragma unroll
-                for (int i = 0; i < V; ++i) { mn = nan_min(mn, f[i]); mx = nan_max(mx, f[i]); }
-            }
-        }
+        for (int c = 0; c < CACHE; ++c)
+            if (c * WAVE + lane < units) stats.add(cache[c]);
     } else {
-        for (int u = lane; u < units; u += WAVE) {
-            float f[V];
-            E::unpack(src[u], f);
-#pragma unroll
-            for (int i = 0; i < V; ++i) { mn = nan_min(mn, f[i]); mx = nan_max(mx, f[i]); }
-        }
+        for (int u = lane; u < units; u += WAVE) stats.add(src[u]);
     }
-    mn = wave_allreduce(mn, [](float a, float b) { return nan_min(a, b); });
-    mx = wave_allreduce(mx, [](float a, float b) { return nan_max(a, b); });
+    float mn, mx;
+    stats.finish(mn, mx);
     const float scale = E::round(mx - mn);
     if (lane == 0) { E::store(bias_out, r, mn); E::store(scale_out, r, scale); }
 
     uint8_t *dst = codes + r * row_len;
-    const RowQuant<DT> rq(mn, scale);
+    const RowEncoder<DT> enc(mn, scale);
     auto emit = [&](int u, const uint4 &raw) {
-        float f[V];
-        E::unpack(raw, f);
-        uint32_t w[V / 4];
-#pragma unroll
-        for (int i = 0; i < V / 4; ++i)
-            w[i] = rq(f[4 * i]) | (rq(f[4 * i + 1]) << 8) | (rq(f[4 * i + 2]) << 16) | (rq(f[4 * i + 3]) << 24);
+        uint32_t w[2];
+        enc.encode(raw, w);
         if constexpr (V == 8) reinterpret_cast<uint2 *>(dst)[u] = make_uint2(w[0], w[1]);
         else reinterpret_cast<uint32_t *>(dst)[u] = w[0];
     };

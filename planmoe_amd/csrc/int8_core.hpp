@@ -84,4 +84,118 @@ struct RowDequant {
     }
 };
 
+// ---------------------------------------------------------------- row-level building blocks
+// RowStats<DT, CANON>: running min / max of a row, NaN-propagating like torch.min / torch.max.
+// CANON: the row as the dispatcher would store it (0 + x, so -0 reads as +0).  RowEncoder<DT>: one 16-byte vector of
+// the row -> VEC codes packed four per 32-bit word.
+template <int DT, bool CANON>
+struct RowStats {
+    using E = Elem<DT>;
+    float mn, mx;
+    __device__ __forceinline__ void init() { mn = INFINITY; mx = -INFINITY; }
+    __device__ __forceinline__ void add(const uint4 &raw)
+    {
+        float f[E::VEC];
+        E::unpack(raw, f);
+#pragma unroll
+        for (int i = 0; i < E::VEC; ++i) { const float d = CANON ? 0.f + f[i] : f[i]; mn = nan_min(mn, d); mx = nan_max(mx, d); }
+    }
+    // reduce over the wavefront
+    __device__ __forceinline__ void finish(float &lo, float &hi) const
+    {
+        lo = wave_allreduce(mn, [](float a, float b) { return nan_min(a, b); });
+        hi = wave_allreduce(mx, [](float a, float b) { return nan_max(a, b); });
+    }
+};
+
+template <int DT>
+struct RowEncoder {
+    using E = Elem<DT>;
+    RowQuant<DT> rq;
+    __device__ __forceinline__ RowEncoder(float bias, float scale) : rq(bias, scale) {}
+    __device__ __forceinline__ void encode(const uint4 &raw, uint32_t *w) const
+    {
+        float f[E::VEC];
+        E::unpack(raw, f);
+#pragma unroll
+        for (int i = 0; i < E::VEC / 4; ++i)
+            w[i] = rq(0.f + f[4 * i]) | (rq(0.f + f[4 * i + 1]) << 8) | (rq(0.f + f[4 * i + 2]) << 16) | (rq(0.f + f[4 * i + 3]) << 24);
+    }
+};
+
+// bf16: two elements per 32-bit word all the way.  Min / max run on 16-bit order-preserving
+// keys (sign-magnitude -> two's complement) with packed integer min / max; NaNs are found by a
+// packed unsigned max of the magnitudes.
+typedef short          s16x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+
+template <bool CANON>
+struct RowStats<PLANMOE_BF16, CANON> {
+    s16x2_t mn, mx;
+    u16x2_t mag;
+    __device__ __forceinline__ void init()
+    {
+        mn = s16x2_t{(short)0x7fff, (short)0x7fff};
+        mx = s16x2_t{(short)0x8000, (short)0x8000};
+        mag = u16x2_t{0, 0};
+    }
+    __device__ __forceinline__ void add_word(uint32_t w)
+    {
+        const s16x2_t v = __builtin_bit_cast(s16x2_t, w);
+        const s16x2_t key = v ^ ((v >> 15) & (short)0x7fff);
+        mn = __builtin_elementwise_min(mn, key);
+        mx = __builtin_elementwise_max(mx, key);
+        mag = __builtin_elementwise_max(mag, __builtin_bit_cast(u16x2_t, w & 0x7fff7fffu));
+    }
+    __device__ __forceinline__ void add(const uint4 &raw)
+    {
+        add_word(raw.x); add_word(raw.y); add_word(raw.z); add_word(raw.w);
+    }
+    __device__ static __forceinline__ float key_to_f32(int key)
+    {
+        uint32_t bits = (uint32_t)(key ^ ((key >> 15) & 0x7fff)) & 0xffffu;
+        if (CANON && bits == 0x8000u) bits = 0u;         // 0 + (-0) = +0
+        return bf16_to_f32(bits);
+    }
+    __device__ __forceinline__ void finish(float &lo, float &hi) const
+    {
+        int a = min((int)mn.x, (int)mn.y), b = max((int)mx.x, (int)mx.y);
+        int n = max((int)mag.x, (int)mag.y);
+        a = wave_allreduce(a, [](int p, int q) { return min(p, q); });
+        b = wave_allreduce(b, [](int p, int q) { return max(p, q); });
+        n = wave_allreduce(n, [](int p, int q) { return max(p, q); });
+        lo = key_to_f32(a);
+        hi = key_to_f32(b);
+        if (n > 0x7f80) { lo = __uint_as_float(0x7fc00000u); hi = lo; }
+    }
+};
+
+template <>
+struct RowEncoder<PLANMOE_BF16> {
+    RowQuant<PLANMOE_BF16> rq;
+    __device__ __forceinline__ RowEncoder(float bias, float scale) : rq(bias, scale) {}
+    // two bf16 in w -> code0 | code1 << 8
+    __device__ __forceinline__ uint32_t pair(uint32_t w) const
+    {
+        const float f0 = __uint_as_float(w << 16), f1 = __uint_as_float(w & 0xffff0000u);
+        if (!rq.fast) return rq(0.f + f0) | (rq(0.f + f1) << 8);
+        uint32_t pk = f32x2_to_bf16x2(f0 - rq.bias, f1 - rq.bias);
+        const float d0 = __uint_as_float(pk << 16), d1 = __uint_as_float(pk & 0xffff0000u);
+        float t0 = d0 * rq.inv, t1 = d1 * rq.inv;
+        t0 = fmaf(fmaf(-t0, rq.scale, d0), rq.inv, t0);
+        t1 = fmaf(fmaf(-t1, rq.scale, d1), rq.inv, t1);
+        pk = f32x2_to_bf16x2(t0, t1);
+        const float q0 = __uint_as_float(pk << 16), q1 = __uint_as_float(pk & 0xffff0000u);
+        pk = f32x2_to_bf16x2(q0 * 255.0f, q1 * 255.0f);
+        const float m0 = __uint_as_float(pk << 16), m1 = __uint_as_float(pk & 0xffff0000u);
+        // truncation; the conversion saturates NaN (0/0 rows) and negatives to 0, m <= 255
+        return __float2uint_rz(m0) | (__float2uint_rz(m1) << 8);
+    }
+    __device__ __forceinline__ void encode(const uint4 &raw, uint32_t *w) const
+    {
+        w[0] = pair(raw.x) | (pair(raw.y) << 16);
+        w[1] = pair(raw.z) | (pair(raw.w) << 16);
+    }
+};
+
 } // namespace pm

@@ -247,14 +247,12 @@ _forward_ws = {}
 
 
 def _forward_workspace(T, E, k, device):
-    """Per-device workspace of the fused chain, grown on demand and initialised once (its
-    completion counter must start at zero; every call leaves it at zero)."""
+    """Per-device workspace of the fused chain, grown on demand."""
     need = lib.planmoe_forward_workspace_bytes(T, E, k)
     key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
     ws = _forward_ws.get(key)
     if ws is None or ws.numel() < need:
         ws = torch.empty((max(need, 1 << 20),), dtype=torch.uint8, device=device)
-        check(lib.planmoe_forward_workspace_init(_ptr(ws), ws.numel(), _stream(ws)))
         _forward_ws[key] = ws
     return ws
 
@@ -314,6 +312,36 @@ def forward_int8(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, norma
                                    _ptr(out["codes"]), _ptr(out["bias"]), _ptr(out["scale"]), _ptr(ws),
                                    ws.numel(), _stream(x)))
     return out
+
+
+class ForwardInt8Plan:
+    """forward_int8 with every output and the workspace allocated once: `run()` is a single
+    C-ABI call that enqueues the three launches (for serving loops that reuse their buffers)."""
+
+    def __init__(self, x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
+                 want_l_aux=True, want_counts=False):
+        x, wg, T, M, E, k, bias, out, ws = _forward_common(x, wg, top_k, fp32_gate, logit_bias, False,
+                                                           False, want_l_aux, want_counts)
+        R = E * capacity_
+        out["codes"] = torch.empty((R, M), dtype=torch.uint8, device=x.device)
+        out["bias"] = torch.empty((R, 1), dtype=x.dtype, device=x.device)
+        out["scale"] = torch.empty((R, 1), dtype=x.dtype, device=x.device)
+        self.out, self.x, self.wg, self._bias, self._ws = out, x, wg, bias, ws
+        self._args = [_ptr(x), _ptr(wg), _dt(x, "forward_int8"), int(bool(fp32_gate)), _ptr(bias), T, M, E, k,
+                      int(bool(normalize_gate)), capacity_, _ptr(out["indices"]), _ptr(out["locations"]),
+                      _ptr(out["gates"]), max(T, 1), None, None, _ptr(out["l_aux"]), _ptr(out["counts"]),
+                      _ptr(out["codes"]), _ptr(out["bias"]), _ptr(out["scale"]), _ptr(ws), ws.numel()]
+
+    def run(self):
+        check(lib.planmoe_forward_int8(*self._args, _stream(self.x)))
+        return self.out
+
+    def redispatch(self):
+        """Only the last launch again (dispatch + int8 from the routing state of the last run)."""
+        a = self._args
+        check(lib.planmoe_forward_int8_redispatch(a[0], a[2], a[5], a[6], a[7], a[8], a[10], a[11], a[12], a[14],
+                                                  a[19], a[20], a[21], a[22], a[23], _stream(self.x)))
+        return self.out
 
 
 # ------------------------------------------------------------------------------ zfp codec
