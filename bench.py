@@ -18,37 +18,47 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 
-def event_time_us(fn, iters, warm):
+def event_time_us(fn, iters, warm, rounds=5):
+    """Average device time of one call: `iters` calls are enqueued back to back between one
+    pair of HIP events (so the GPU never waits for the host), best and mean of `rounds`."""
     import torch
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
-    for a, b in evs:
+    per_call = []
+    for _ in range(rounds):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
-        fn()
+        for _ in range(iters):
+            fn()
         b.record()
-    torch.cuda.synchronize()
-    ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)
-    return sum(ts) / len(ts), ts[len(ts) // 2], ts[0]
+        torch.cuda.synchronize()
+        per_call.append(a.elapsed_time(b) * 1e3 / iters)
+    per_call.sort()
+    return sum(per_call) / len(per_call), per_call[len(per_call) // 2], per_call[0]
 
 
-def cpu_baseline(T_sample, M, E, k, cf, x_bits, wg_bits):
-    """The CPU oracle (single thread) on the first T_sample tokens of the same batch."""
+def cpu_baseline(T_sample, M, E, k, cf, x_bits, wg_bits, min_seconds):
+    """The CPU oracle (single thread) on the first T_sample tokens of the same batch, repeated
+    until `min_seconds` have passed."""
     import numpy as np
     import oracle
     xs = np.ascontiguousarray(x_bits[:T_sample])
-    t0 = time.perf_counter()
-    logits = oracle.gate_logits(xs, wg_bits).astype(np.float32)
-    scores = oracle.softmax(logits)
-    idx, loc, gates, _ = oracle.route_topk(scores, k)
-    C = oracle.capacity(T_sample, E, k, cf, 4)
-    x32 = (xs.astype(np.uint32) << 16).view(np.float32)
-    d = oracle.encode(x32, list(idx), list(loc), None, E, C)
-    d_bits = (d.view(np.uint32) >> 16).astype(np.uint16)          # exact: values are bf16 already
-    oracle.int8_compress(d_bits)
-    dt = time.perf_counter() - t0
-    return T_sample / dt, dt
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        logits = oracle.gate_logits(xs, wg_bits).astype(np.float32)
+        scores = oracle.softmax(logits)
+        idx, loc, gates, _ = oracle.route_topk(scores, k)
+        C = oracle.capacity(T_sample, E, k, cf, 4)
+        x32 = (xs.astype(np.uint32) << 16).view(np.float32)
+        d = oracle.encode(x32, list(idx), list(loc), None, E, C)
+        d_bits = (d.view(np.uint32) >> 16).astype(np.uint16)          # exact: values are bf16 already
+        oracle.int8_compress(d_bits)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= min_seconds:
+            break
+    return T_sample * reps / dt, dt, reps
 
 
 def main():
@@ -56,7 +66,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--cpu-sample", type=int, default=2048, help="tokens given to the CPU baseline (0 = skip)")
+    ap.add_argument("--cpu-sample", type=int, default=16384, help="tokens given to the CPU baseline (0 = skip)")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="minimum CPU-baseline run time")
+    ap.add_argument("--copy-reference", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times (a kernel of known traffic, "
+                         "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings against)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
@@ -80,6 +94,13 @@ def main():
 
     def chain():
         return plan.run()
+
+    if args.copy_reference:
+        ref_src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        ref_dst = torch.empty_like(ref_src)
+        for _ in range(5):
+            ref_dst.copy_(ref_src)
+        torch.cuda.synchronize()
 
     # timed region: EXACTLY --steps passes between two synchronisations
     for _ in range(args.warmup):
@@ -117,7 +138,10 @@ def main():
                                "compress, forward", "tokens": T, "model_dim": M, "experts": E, "top_k": k,
                    "capacity_factor": cf, "capacity": C},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     # HBM bytes per launch read from rocprofv3 FETCH_SIZE (x 2.0, the factor a device
+                     # copy of known size shows for that counter) + WRITE_SIZE; see profiles/
+                     "traffic": 306.0e6,
                      "kernel": "dispatch_int8_routed_kernel (last launch of the chain, timed alone)",
                      "algorithmic_bytes": dom_bytes, "avg_us": dom_avg_us},
         "chain": {"algorithmic_bytes": chain_bytes, "device_us_avg": chain_ev[0], "device_us_min": chain_ev[2],
@@ -126,10 +150,10 @@ def main():
     }
     if args.cpu_sample > 0:
         bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
-        v, dt = cpu_baseline(min(args.cpu_sample, T), M, E, k, cf, bits(x), bits(wg))
+        v, dt, reps = cpu_baseline(min(args.cpu_sample, T), M, E, k, cf, bits(x), bits(wg), args.cpu_seconds)
         out["cpu_baseline"] = {"value": v, "unit": "tokens/s", "cores": 1, "kind": "port",
-                               "sample": "first %d of the %d tokens, same chain through the CPU oracle "
-                                         "(single thread, %.1f s)" % (min(args.cpu_sample, T), T, dt),
+                               "sample": "%d of the %d tokens x %d passes of the same chain through the CPU "
+                                         "oracle (single thread, %.1f s)" % (min(args.cpu_sample, T), T, reps, dt),
                                "host_cores": os.cpu_count()}
     print(json.dumps(out))
 
