@@ -16,7 +16,8 @@
 // fast_encode (fast_dispatch.py:197-201) + Int8Compressor::compress (int8.cpp:7-44).
 //
 // Workspace (32-bit words): totals[E], loss_part[64], hist[groups][k][E], offs[groups][k][E],
-// me[groups][E] (fp32), rank[k][samples] (rank of a token inside its group).
+// me[groups][E] (fp32), rank[k][samples] (rank of a token inside its group), row_min[samples],
+// row_max[samples] (fp32; bf16 inputs only: the gate kernel scans the rows it streams anyway).
 #include "gate_core.hpp"
 #include "rows.hpp"
 #include "int8_core.hpp"
@@ -30,9 +31,9 @@ constexpr int FWD_LOSS_PARTS = 64;
 
 struct FwdWs {
     int32_t *totals, *hist, *offs, *rank;
-    float *loss_part, *me;
+    float *loss_part, *me, *row_min, *row_max;
 };
-__host__ __device__ inline FwdWs fwd_ws(void *ws, int groups, int k, int experts)
+__host__ __device__ inline FwdWs fwd_ws(void *ws, int groups, int k, int experts, int samples)
 {
     FwdWs w;
     w.totals = (int32_t *)ws;
@@ -41,13 +42,16 @@ __host__ __device__ inline FwdWs fwd_ws(void *ws, int groups, int k, int experts
     w.offs = w.hist + (size_t)groups * k * experts;
     w.me = (float *)(w.offs + (size_t)groups * k * experts);
     w.rank = (int32_t *)(w.me + (size_t)groups * experts);
+    w.row_min = (float *)(w.rank + (size_t)k * samples);
+    w.row_max = w.row_min + samples;
     return w;
 }
 
 __device__ __forceinline__ uint64_t lanes_below() { return ((uint64_t)1 << lane_id()) - 1; }
 
 // SDT: dtype of logits / scores / gates (F32 when fp32_gate, else the input dtype)
-template <int DT, int SDT, int NT, int TPW>
+// CAP: compile-time bound of the expert count held in registers by the routing epilogue
+template <int DT, int SDT, int NT, int TPW, int CAP>
 __global__ __launch_bounds__(256) void gate_route_kernel(
     const void *__restrict__ x, const void *__restrict__ wg, const float *__restrict__ logit_bias,
     int samples, int model_dim, int experts, int k, int normalize_gate,
@@ -56,22 +60,36 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
     float *__restrict__ l_aux, int32_t *__restrict__ counts_out, void *__restrict__ workspace)
 {
     using S = Elem<SDT>;
-    constexpr int CAP = 16 * NT;
     constexpr int GROUP = 16 * TPW;
-    __shared__ float part[4][GROUP][CAP + 1];
+    __shared__ float part[4][GROUP][16 * NT + 1];
     __shared__ int32_t s_hist[CAP];
 
     const int tid = threadIdx.x, lane = lane_id();
     const int groups = gridDim.x;
-    const FwdWs ws = fwd_ws(workspace, groups, k, experts);
+    const FwdWs ws = fwd_ws(workspace, groups, k, experts, samples);
     const int t0 = blockIdx.x * GROUP;
-    gate_tile_partials<DT, NT, TPW>(x, wg, t0, samples, model_dim, experts, part);
+    constexpr bool STATS = DT == PLANMOE_BF16;
+    __shared__ int32_t pstat[4][GROUP][3];
+    gate_tile_partials<DT, NT, TPW, 4, STATS>(x, wg, t0, samples, model_dim, experts, part, pstat);
     __syncthreads();
 
     if (tid < WAVE) {                                  // wave 0: one lane per token of the group
         const int t = t0 + tid;
         const bool valid = tid < GROUP && t < samples;
         float s[CAP];
+        if constexpr (STATS) {
+            if (valid) {
+                // row min / max for the int8 codec of the dispatch launch
+                int a = pstat[0][tid][0], b = pstat[0][tid][1], n = pstat[0][tid][2];
+#pragma unroll
+                for (int w = 1; w < 4; ++w) {
+                    a = min(a, pstat[w][tid][0]); b = max(b, pstat[w][tid][1]); n = max(n, pstat[w][tid][2]);
+                }
+                float lo, hi;
+                RowStats<PLANMOE_BF16, true>::decode(a, b, n, lo, hi);
+                ws.row_min[t] = lo; ws.row_max[t] = hi;
+            }
+        }
         if (valid) {
             float mx = -INFINITY;
 #pragma unroll
@@ -89,10 +107,11 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
             float sum = 0.f;
 #pragma unroll
             for (int e = 0; e < CAP; ++e) if (e < experts) { s[e] = expf(s[e] - mx); sum += s[e]; }
+            const float inv = 1.0f / sum;                 // scores are tolerance-level quantities
 #pragma unroll
             for (int e = 0; e < CAP; ++e) {
                 if (e < experts) {
-                    s[e] = S::round(s[e] / sum);
+                    s[e] = S::round(s[e] * inv);
                     if (scores_out) S::store(scores_out, (int64_t)t * experts + e, s[e]);
                 }
             }
@@ -108,6 +127,8 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
         }
         float denom = 0.f;
         uint64_t taken = 0;
+        constexpr int KREG = 4;                          // raw gates of the first planes stay in registers
+        float gv[KREG] = {0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < k; ++j) {
             int best = -1; float bv = -INFINITY;
             if (valid) {
@@ -118,7 +139,9 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
                 }
                 taken |= (uint64_t)1 << best;
                 indices[(int64_t)j * stride + t] = best;
-                S::store(gates, (int64_t)j * stride + t, bv);
+#pragma unroll
+                for (int q = 0; q < KREG; ++q) if (q == j) gv[q] = bv;
+                if (j >= KREG || !(k > 1 && normalize_gate)) S::store(gates, (int64_t)j * stride + t, bv);
                 denom = (j == 0) ? bv : S::round(denom + bv);
             }
             __builtin_amdgcn_wave_barrier();
@@ -142,7 +165,10 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
             const float eps = SDT == PLANMOE_F32 ? 1.1920928955078125e-07f
                             : SDT == PLANMOE_BF16 ? 0.0078125f : 0.0009765625f;
             const float d = fmaxf(denom, eps);
-            for (int j = 0; j < k; ++j) {
+#pragma unroll
+            for (int j = 0; j < KREG; ++j)
+                if (j < k) S::store(gates, (int64_t)j * stride + t, gv[j] / d);
+            for (int j = KREG; j < k; ++j) {
                 const float g = S::load(gates, (int64_t)j * stride + t);
                 S::store(gates, (int64_t)j * stride + t, g / d);
             }
@@ -298,7 +324,7 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     uint8_t *__restrict__ codes, void *__restrict__ bias_out, void *__restrict__ scale_out,
     const int32_t *__restrict__ hist, const int32_t *__restrict__ totals, const int32_t *__restrict__ rank,
     int group_tokens, int token_blocks, const float *__restrict__ loss_part, int loss_parts,
-    float *__restrict__ l_aux)
+    float *__restrict__ l_aux, const float *__restrict__ row_min, const float *__restrict__ row_max)
 {
     using E = Elem<DT>;
     constexpr int V = E::VEC;
@@ -347,16 +373,20 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     }
     if (__ballot(slot >= 0) == 0) return;
 
-    RowStats<DT, true> stats;
-    stats.init();
-    if constexpr (CACHE > 0) {
-#pragma unroll
-        for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) stats.add(cache[c]);
-    } else {
-        for (int u = lane; u < units; u += WAVE) stats.add(src[u]);
-    }
     float mn, mx;
-    stats.finish(mn, mx);
+    if (row_min) {                                      // the gate kernel already scanned the row
+        mn = row_min[t]; mx = row_max[t];
+    } else {
+        RowStats<DT, true> stats;
+        stats.init();
+        if constexpr (CACHE > 0) {
+#pragma unroll
+            for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) stats.add(cache[c]);
+        } else {
+            for (int u = lane; u < units; u += WAVE) stats.add(src[u]);
+        }
+        stats.finish(mn, mx);
+    }
     const float scale = E::round(mx - mn);
     if (slot >= 0) { E::store(bias_out, slot, mn); E::store(scale_out, slot, scale); }
     const RowEncoder<DT> enc(mn, scale);
@@ -386,12 +416,13 @@ static void launch_gate_route(int experts, int groups, hipStream_t st, const voi
                               int32_t *indices, int32_t *locations, void *gates, int64_t stride,
                               void *logits_out, void *scores_out, float *l_aux, int32_t *counts, void *ws)
 {
-#define PM_GR(NT, TPW)                                                                                   \
-    gate_route_kernel<DT, SDT, NT, TPW><<<groups, 256, 0, st>>>(x, wg, bias, samples, model_dim, experts, \
+#define PM_GR(NT, TPW, CAP)                                                                                   \
+    gate_route_kernel<DT, SDT, NT, TPW, CAP><<<groups, 256, 0, st>>>(x, wg, bias, samples, model_dim, experts, \
         k, normalize, indices, locations, gates, stride, logits_out, scores_out, l_aux, counts, ws)
-    if (experts <= 16) PM_GR(1, 4);          // TPW must equal fwd_group_tokens(experts) / 16
-    else if (experts <= 32) PM_GR(2, 2);
-    else PM_GR(4, 2);
+    if (experts <= 8) PM_GR(1, 4, 8);        // TPW must equal fwd_group_tokens(experts) / 16
+    else if (experts <= 16) PM_GR(1, 4, 16);
+    else if (experts <= 32) PM_GR(2, 2, 32);
+    else PM_GR(4, 2, 64);
 #undef PM_GR
 }
 
@@ -401,12 +432,13 @@ static void launch_dispatch_routed(int per_lane, unsigned grid, hipStream_t st, 
                                    int samples, int model_dim, int experts, int capacity, uint8_t *codes,
                                    void *bias, void *scale, const int32_t *offs, const int32_t *totals,
                                    const int32_t *rank, int group_tokens, int token_blocks,
-                                   const float *loss_part, int loss_parts, float *l_aux)
+                                   const float *loss_part, int loss_parts, float *l_aux,
+                                   const float *row_min, const float *row_max)
 {
 #define PM_DR(CACHE)                                                                                 \
     dispatch_int8_routed_kernel<DT, CACHE><<<grid, 256, 0, st>>>(x, indices, locations, stride, top_k, \
         samples, model_dim, experts, capacity, codes, bias, scale, offs, totals, rank, group_tokens,  \
-        token_blocks, loss_part, loss_parts, l_aux)
+        token_blocks, loss_part, loss_parts, l_aux, row_min, row_max)
     if (per_lane <= 2) PM_DR(2);
     else if (per_lane <= 4) PM_DR(4);
     else if (per_lane <= 8) PM_DR(8);
@@ -449,7 +481,7 @@ static int run_gate_route(const void *x, const void *wg, int dtype, int fp32_gat
     plan.experts_per_block = GO_COLS / plan.k;
     if (plan.experts_per_block > experts) plan.experts_per_block = experts;
     plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
-    plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts);
+    plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts, samples);
     const int k = plan.k, groups = plan.groups;
     if (fp32_gate || dtype == PLANMOE_F32) {
         PM_DTYPE_SWITCH(dtype, DT, (launch_gate_route<DT, PLANMOE_F32>(
@@ -485,7 +517,9 @@ static int run_dispatch_routed(const void *x, int dtype, int samples, int model_
         launch_dispatch_routed<DT>(per_lane, (unsigned)(token_blocks + fill_blocks), st, x, indices, locations,
                                    stride, plan.k, samples, model_dim, experts, capacity, codes, bias,
                                    scale, plan.ws.offs, plan.ws.totals, plan.ws.rank, plan.group_tokens, token_blocks,
-                                   plan.ws.loss_part, plan.blocks, l_aux));
+                                   plan.ws.loss_part, plan.blocks, l_aux,
+                                   dtype == PLANMOE_BF16 ? plan.ws.row_min : nullptr,
+                                   dtype == PLANMOE_BF16 ? plan.ws.row_max : nullptr));
     return 0;
 }
 
@@ -499,7 +533,7 @@ extern "C" size_t planmoe_forward_workspace_bytes(int samples, int experts, int 
     const size_t k = (size_t)(top_k < experts ? top_k : experts);
     const size_t groups = ((size_t)samples + 31) / 32;      // upper bound over the group sizes
     return round_up(((size_t)experts + FWD_LOSS_PARTS + 2 * groups * k * experts + groups * experts +
-                     k * (size_t)samples) * 4, 256);
+                     (k + 2) * (size_t)samples) * 4, 256);
 }
 
 extern "C" int planmoe_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
@@ -575,7 +609,7 @@ extern "C" int planmoe_forward_int8_redispatch(const void *x, int dtype, int sam
     plan.experts_per_block = GO_COLS / plan.k;
     if (plan.experts_per_block > experts) plan.experts_per_block = experts;
     plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
-    plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts);
+    plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts, samples);
     if (run_dispatch_routed(x, dtype, samples, model_dim, experts, capacity, indices, locations,
                             plane_stride, nullptr, codes, bias, scale, plan, (hipStream_t)stream)) return 1;
     PM_LAUNCH_CHECK("planmoe_forward_int8_redispatch");

@@ -10,20 +10,22 @@
 
 namespace pm {
 
-template <int DT, int NT, int TPW>
-__global__ __launch_bounds__(256) void gate_logits_kernel(
+template <int DT, int NT, int TPW, int NW>
+__global__ __launch_bounds__(64 * NW) void gate_logits_kernel(
     const void *__restrict__ x, const void *__restrict__ wg, void *__restrict__ logits, int out_dt,
     int samples, int model_dim, int experts)
 {
-    __shared__ float part[4][16 * TPW][16 * NT + 1];
+    __shared__ float part[NW][16 * TPW][16 * NT + 1];
     const int t0 = blockIdx.x * 16 * TPW;
-    gate_tile_partials<DT, NT, TPW>(x, wg, t0, samples, model_dim, experts, part);
+    gate_tile_partials<DT, NT, TPW, NW>(x, wg, t0, samples, model_dim, experts, part);
     __syncthreads();
-    for (int i = threadIdx.x; i < 16 * TPW * experts; i += 256) {
+    for (int i = threadIdx.x; i < 16 * TPW * experts; i += 64 * NW) {
         const int r = i / experts, e = i - r * experts;
         const int t = t0 + r;
         if (t >= samples) continue;
-        const float v = ((part[0][r][e] + part[1][r][e]) + part[2][r][e]) + part[3][r][e];
+        float v = part[0][r][e];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) v += part[w][r][e];
         const int64_t o = (int64_t)t * experts + e;
         if (out_dt == PLANMOE_F32) ((float *)logits)[o] = v;
         else if (out_dt == PLANMOE_BF16) ((uint16_t *)logits)[o] = (uint16_t)f32_to_bf16(v);
@@ -59,12 +61,12 @@ static void launch_gate_logits(const void *x, const void *wg, void *logits, int 
                                                                                  samples, model_dim, experts);
         return;
     }
-#define PM_GATE(NT, TPW)                                                                     \
-    gate_logits_kernel<DT, NT, TPW><<<(samples + 16 * TPW - 1) / (16 * TPW), 256, 0, st>>>(  \
+#define PM_GATE(NT, TPW, NW)                                                                      \
+    gate_logits_kernel<DT, NT, TPW, NW><<<(samples + 16 * TPW - 1) / (16 * TPW), 64 * NW, 0, st>>>(  \
         x, wg, logits, out_dt, samples, model_dim, experts)
-    if (experts <= 16) PM_GATE(1, 4);
-    else if (experts <= 32) PM_GATE(2, 2);
-    else PM_GATE(4, 2);
+    if (experts <= 16) PM_GATE(1, 4, 4);
+    else if (experts <= 32) PM_GATE(2, 2, 4);
+    else PM_GATE(4, 2, 4);
 #undef PM_GATE
 }
 

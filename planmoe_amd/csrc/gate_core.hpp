@@ -1,6 +1,7 @@
 // MFMA core of the gate-logits GEMM, shared by the stand-alone and the fused gate kernels.
 #pragma once
 #include "common.hpp"
+#include "int8_core.hpp"
 
 namespace pm {
 
@@ -43,18 +44,28 @@ struct GateFrag {
     uint4 b[NT][4];
 };
 
-// Partial logits of tokens [t0, t0 + 16*TPW) against experts [0, 16*NT): wave w accumulates
-// the K steps w, w+4, ... (a step is 16 vectors = 256 bytes of every row) and leaves its
-// tiles in part[w][token][expert].  Rows past the end of x / wg are clamped to the last valid
+// Partial logits of tokens [t0, t0 + 16*TPW) against experts [0, 16*NT): wave w of the NW waves
+// of the work-group accumulates the K steps w, w+NW, ... (a step is 16 vectors = 256 bytes of
+// every row) and leaves its tiles in part[w][token][expert].  Rows past the end of x / wg are clamped to the last valid
 // row: their products land in tile entries nobody reads.  Loads of the next step are issued
 // before the MFMAs of the current one.
-// Requires model_dim % VEC == 0 and 16-byte aligned x / wg.  Call with all 256 threads.
-template <int DT, int NT, int TPW>
+// With STATS (bf16 only) the wave also keeps the running min / max / NaN scan of every token row
+// it streams (the VALU is idle while the loads are in flight) and leaves, per wave, the three
+// 32-bit words of RowStats<bf16>::reduced() in pstat[w][token][0..2].
+// Requires model_dim % VEC == 0 and 16-byte aligned x / wg.  Call with all 64*NW threads.
+template <int DT, int NT, int TPW, int NW = 4, bool STATS = false>
 __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
                                                    const void *__restrict__ wg, int t0, int samples,
                                                    int model_dim, int experts,
-                                                   float (*part)[16 * TPW][16 * NT + 1])
+                                                   float (*part)[16 * TPW][16 * NT + 1],
+                                                   int32_t (*pstat)[16 * TPW][3] = nullptr)
 {
+    static_assert(!STATS || DT == PLANMOE_BF16, "row statistics ride along for bf16 only");
+    RowStats<PLANMOE_BF16, true> st[TPW];
+    if constexpr (STATS) {
+#pragma unroll
+        for (int tp = 0; tp < TPW; ++tp) st[tp].init();
+    }
     constexpr int V = Elem<DT>::VEC;
     const int w = threadIdx.x >> 6, l = lane_id();
     const int m = l & 15, g = l >> 4;
@@ -100,27 +111,29 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
-            for (int tp = 0; tp < TPW; ++tp)
+            for (int tp = 0; tp < TPW; ++tp) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) Mma<DT>::run(f.a[tp][s], f.b[nt][s], acc[tp][nt]);
+                if constexpr (STATS) st[tp].add(f.a[tp][s]);
+            }
     };
 
     GateFrag<NT, TPW> f0, f1;
     int step = w;
     if (step < full) load(f0, step);
     while (step < full) {
-        const bool more1 = step + 4 < full;
-        if (more1) load(f1, step + 4);
+        const bool more1 = step + NW < full;
+        if (more1) load(f1, step + NW);
         mma(f0);
         if (!more1) break;
-        const bool more2 = step + 8 < full;
-        if (more2) load(f0, step + 8);
+        const bool more2 = step + 2 * NW < full;
+        if (more2) load(f0, step + 2 * NW);
         mma(f1);
-        step += 8;
+        step += 2 * NW;
         if (!more2) break;
     }
 
-    if (rem && (full & 3) == w) {
+    if (rem && (full % NW) == w) {
         // last, partial step: vectors past the row end are read from a clamped index and zeroed
         GateFrag<NT, TPW> f;
         const int o = full * 16;
@@ -132,6 +145,8 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
             for (int tp = 0; tp < TPW; ++tp) {
                 uint4 v = ap[tp][off];
                 f.a[tp][s] = in ? v : make_uint4(0, 0, 0, 0);
+                // vector `o` read again in place of a vector past the row end: harmless for min / max
+                if constexpr (STATS) st[tp].add(v);
             }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
@@ -139,7 +154,28 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
                 f.b[nt][s] = in ? v : make_uint4(0, 0, 0, 0);
             }
         }
-        mma(f);
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int tp = 0; tp < TPW; ++tp)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) Mma<DT>::run(f.a[tp][s], f.b[nt][s], acc[tp][nt]);
+    }
+
+    if constexpr (STATS) {
+        // the 4 lanes (l % 16 == m) of a row hold its k-slices: combine them, lane g == 0 writes
+#pragma unroll
+        for (int tp = 0; tp < TPW; ++tp) {
+            int a, b, n;
+            st[tp].reduced(a, b, n);
+#pragma unroll
+            for (int off = 16; off < 64; off <<= 1) {
+                a = min(a, __shfl_xor(a, off, WAVE));
+                b = max(b, __shfl_xor(b, off, WAVE));
+                n = max(n, __shfl_xor(n, off, WAVE));
+            }
+            if (g == 0) { pstat[w][tp * 16 + m][0] = a; pstat[w][tp * 16 + m][1] = b; pstat[w][tp * 16 + m][2] = n; }
+        }
     }
 
 #pragma unroll

@@ -157,16 +157,28 @@ struct RowStats<PLANMOE_BF16, CANON> {
         if (CANON && bits == 0x8000u) bits = 0u;         // 0 + (-0) = +0
         return bf16_to_f32(bits);
     }
-    __device__ __forceinline__ void finish(float &lo, float &hi) const
+    // this lane's share as three plain integers: min key, max key, largest magnitude
+    __device__ __forceinline__ void reduced(int &a, int &b, int &n) const
     {
-        int a = min((int)mn.x, (int)mn.y), b = max((int)mx.x, (int)mx.y);
-        int n = max((int)mag.x, (int)mag.y);
-        a = wave_allreduce(a, [](int p, int q) { return min(p, q); });
-        b = wave_allreduce(b, [](int p, int q) { return max(p, q); });
-        n = wave_allreduce(n, [](int p, int q) { return max(p, q); });
+        a = min((int)mn.x, (int)mn.y);
+        b = max((int)mx.x, (int)mx.y);
+        n = max((int)mag.x, (int)mag.y);
+    }
+    // min / max of the row from combined integers (any number of shares merged with min / max / max)
+    __device__ static __forceinline__ void decode(int a, int b, int n, float &lo, float &hi)
+    {
         lo = key_to_f32(a);
         hi = key_to_f32(b);
         if (n > 0x7f80) { lo = __uint_as_float(0x7fc00000u); hi = lo; }
+    }
+    __device__ __forceinline__ void finish(float &lo, float &hi) const
+    {
+        int a, b, n;
+        reduced(a, b, n);
+        a = wave_allreduce(a, [](int p, int q) { return min(p, q); });
+        b = wave_allreduce(b, [](int p, int q) { return max(p, q); });
+        n = wave_allreduce(n, [](int p, int q) { return max(p, q); });
+        decode(a, b, n, lo, hi);
     }
 };
 
