@@ -152,6 +152,18 @@ int planmoe_dispatch_int8(const void *x, int dtype, const float *gates, const in
                           uint8_t *codes, void *bias, void *scale,
                           void *workspace, size_t workspace_bytes, void *stream);
 
+/* GatingDecoder.backward followed by the int8 compressor of the backward all-to-all
+ * (fast_dispatch.py:66-79, then Decompress.backward = compress_operation, overlap.py:33-34):
+ *   grad_expert[slot_j, :] = 0 + gate_j * grad_out[t, :]   -> codes / bias / scale as above,
+ *   grad_gates[j][t] = <grad_out[t, :], expert_out[slot_j, :]>  (0 for a dropped pair; fp32 planes
+ *   with the same plane_stride).
+ * gates must not be NULL (the reference computes gate gradients only for real gates). */
+int planmoe_combine_bwd_int8(const void *grad_out, const void *expert_out, int dtype,
+                             const float *gates, const int32_t *indices, const int32_t *locations,
+                             int64_t plane_stride, int top_k, int samples, int model_dim,
+                             int experts, int capacity, uint8_t *codes, void *bias, void *scale,
+                             float *grad_gates, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------- fused forward chain
  * The layer's forward path up to the all-to-all send buffer in three launches: gate GEMM +
  * routing (gates/top.py:20-26, moe_layer.py:230-256, fast_dispatch.py:140-195), then

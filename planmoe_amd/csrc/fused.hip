@@ -16,7 +16,8 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
     const int32_t *__restrict__ indices, const int32_t *__restrict__ locations, int64_t stride,
     int top_k, int samples, int model_dim, int experts, int capacity,
     uint8_t *__restrict__ codes, void *__restrict__ bias_out, void *__restrict__ scale_out,
-    const uint32_t *__restrict__ flags, int token_blocks)
+    const uint32_t *__restrict__ flags, int token_blocks,
+    const void *__restrict__ other, float *__restrict__ grad_gates)
 {
     using E = Elem<DT>;
     constexpr int V = E::VEC;
@@ -51,6 +52,29 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
             if (u < units) cache[c] = src[u];
         }
     }
+    auto cache_ref = [&](int c) -> const uint4 & { return cache[c]; };
+
+    // gate gradient of one choice: <x[t], other[slot]> (GatingDecoder.backward, fast_dispatch.py:73-78)
+    auto dot_with = [&](int s) {
+        const uint4 *orow = reinterpret_cast<const uint4 *>((const char *)other + (int64_t)s * model_dim * (int64_t)sizeof(typename E::store_t));
+        float acc = 0.f;
+        auto visit = [&](const uint4 &a, const uint4 &b) {
+            float fa[V], fb[V];
+            E::unpack(a, fa); E::unpack(b, fb);
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc = fmaf(fb[i], fa[i], acc);
+        };
+        if constexpr (CACHE > 0) {
+            uint4 o[CACHE];
+#pragma unroll
+            for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) o[c] = orow[c * WAVE + lane];
+#pragma unroll
+            for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) visit(cache_ref(c), o[c]);
+        } else {
+            for (int u = lane; u < units; u += WAVE) visit(src[u], orow[u]);
+        }
+        return wave_sum(acc);
+    };
 
     // the row as the dispatcher would store it for gate g: round(0 + g * x)
     auto reduce = [&](float g, float &mn, float &mx) {
@@ -92,6 +116,7 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
         const int np = min(top_k - j0, WAVE);
         int slot; float gate;
         fetch_planes(gates, indices, locations, stride, t, j0, np, experts, capacity, slot, gate);
+        if (grad_gates && lane < np && slot < 0) grad_gates[(int64_t)(j0 + lane) * stride + t] = 0.f;
         if (__ballot(slot >= 0) == 0) continue;
 
         if (!gates) {
@@ -128,6 +153,10 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
                 const int s = rl_i(slot, j);
                 if (s < 0) continue;
                 const float g = rl_f(gate, j);
+                if (grad_gates) {
+                    const float gg = dot_with(s);
+                    if (lane == 0) grad_gates[(int64_t)(j0 + j) * stride + t] = gg;
+                }
                 float mn, mx;
                 reduce(g, mn, mx);
                 const float scale = E::round(mx - mn);
@@ -154,11 +183,13 @@ static void launch_dispatch_int8(int per_lane, unsigned grid, hipStream_t st, co
                                  const float *gates, const int32_t *indices, const int32_t *locations,
                                  int64_t stride, int top_k, int samples, int model_dim, int experts,
                                  int capacity, uint8_t *codes, void *bias, void *scale,
-                                 const uint32_t *flags, int token_blocks)
+                                 const uint32_t *flags, int token_blocks, const void *other,
+                                 float *grad_gates)
 {
 #define PM_DI8(CACHE)                                                                            \
     dispatch_int8_kernel<DT, CACHE><<<grid, 256, 0, st>>>(x, gates, indices, locations, stride,  \
-        top_k, samples, model_dim, experts, capacity, codes, bias, scale, flags, token_blocks)
+        top_k, samples, model_dim, experts, capacity, codes, bias, scale, flags, token_blocks,   \
+        other, grad_gates)
     if (per_lane <= 2) PM_DI8(2);
     else if (per_lane <= 4) PM_DI8(4);
     else if (per_lane <= 8) PM_DI8(8);
@@ -171,28 +202,27 @@ static void launch_dispatch_int8(int per_lane, unsigned grid, hipStream_t st, co
 
 using namespace pm;
 
-extern "C" int planmoe_dispatch_int8(const void *x, int dtype, const float *gates,
-                                     const int32_t *indices, const int32_t *locations,
-                                     int64_t plane_stride, int top_k, int samples, int model_dim,
-                                     int experts, int capacity, uint8_t *codes, void *bias,
-                                     void *scale, void *workspace, size_t workspace_bytes,
-                                     void *stream)
+static int run_dispatch_int8(const char *who, const void *x, int dtype, const float *gates,
+                             const int32_t *indices, const int32_t *locations, int64_t plane_stride,
+                             int top_k, int samples, int model_dim, int experts, int capacity,
+                             uint8_t *codes, void *bias, void *scale, void *workspace,
+                             size_t workspace_bytes, const void *other, float *grad_gates, void *stream)
 {
-    if (check_planes("planmoe_dispatch_int8", indices, locations, plane_stride, top_k, samples)) return 1;
-    PM_REQUIRE(dtype_ok(dtype), "planmoe_dispatch_int8: bad dtype %d", dtype);
-    PM_REQUIRE(model_dim >= 1 && experts >= 1 && capacity >= 0, "planmoe_dispatch_int8: bad shape");
-    PM_REQUIRE((int64_t)experts * capacity < (1ll << 31), "planmoe_dispatch_int8: experts*capacity overflows int32");
-    PM_REQUIRE((int64_t)samples * top_k < (1ll << 31), "planmoe_dispatch_int8: samples*top_k overflows int32");
+    if (check_planes(who, indices, locations, plane_stride, top_k, samples)) return 1;
+    PM_REQUIRE(dtype_ok(dtype), "%s: bad dtype %d", who, dtype);
+    PM_REQUIRE(model_dim >= 1 && experts >= 1 && capacity >= 0, "%s: bad shape", who);
+    PM_REQUIRE((int64_t)experts * capacity < (1ll << 31), "%s: experts*capacity overflows int32", who);
+    PM_REQUIRE((int64_t)samples * top_k < (1ll << 31), "%s: samples*top_k overflows int32", who);
     const int slots = experts * capacity;
     if (slots == 0) return 0;
-    PM_REQUIRE(x || samples == 0, "planmoe_dispatch_int8: x is NULL");
-    PM_REQUIRE(codes && bias && scale, "planmoe_dispatch_int8: NULL output");
+    PM_REQUIRE(x || samples == 0, "%s: x is NULL", who);
+    PM_REQUIRE(codes && bias && scale, "%s: NULL output", who);
     PM_REQUIRE(workspace && workspace_bytes >= planmoe_dispatch_workspace_bytes(experts, capacity),
-               "planmoe_dispatch_int8: workspace too small");
+               "%s: workspace too small", who);
     const int vec = dtype == PLANMOE_F32 ? 4 : 8;
-    PM_REQUIRE(model_dim % vec == 0 && aligned16(x) && ((uintptr_t)codes % 8 == 0),
-               "planmoe_dispatch_int8: model_dim must be a multiple of %d and buffers 16-byte aligned; "
-               "use planmoe_dispatch_fwd + planmoe_int8_compress otherwise", vec);
+    PM_REQUIRE(model_dim % vec == 0 && aligned16(x) && ((uintptr_t)codes % 8 == 0) && (!other || aligned16(other)),
+               "%s: model_dim must be a multiple of %d and buffers 16-byte aligned; "
+               "use the unfused entry points otherwise", who, vec);
     hipStream_t st = (hipStream_t)stream;
     uint32_t *flags = (uint32_t *)workspace;
     launch_slot_flags(flags, indices, locations, plane_stride, top_k, samples, experts, capacity, st);
@@ -202,7 +232,33 @@ extern "C" int planmoe_dispatch_int8(const void *x, int dtype, const float *gate
     PM_DTYPE_SWITCH(dtype, DT,
         launch_dispatch_int8<DT>(per_lane, (unsigned)(token_blocks + fill_blocks), st, x, gates, indices,
                                  locations, plane_stride, top_k, samples, model_dim, experts, capacity,
-                                 codes, bias, scale, flags, token_blocks));
-    PM_LAUNCH_CHECK("planmoe_dispatch_int8");
+                                 codes, bias, scale, flags, token_blocks, other, grad_gates));
+    PM_LAUNCH_CHECK(who);
     return 0;
+}
+
+extern "C" int planmoe_dispatch_int8(const void *x, int dtype, const float *gates,
+                                     const int32_t *indices, const int32_t *locations,
+                                     int64_t plane_stride, int top_k, int samples, int model_dim,
+                                     int experts, int capacity, uint8_t *codes, void *bias,
+                                     void *scale, void *workspace, size_t workspace_bytes,
+                                     void *stream)
+{
+    return run_dispatch_int8("planmoe_dispatch_int8", x, dtype, gates, indices, locations, plane_stride,
+                             top_k, samples, model_dim, experts, capacity, codes, bias, scale, workspace,
+                             workspace_bytes, nullptr, nullptr, stream);
+}
+
+extern "C" int planmoe_combine_bwd_int8(const void *grad_out, const void *expert_out, int dtype,
+                                        const float *gates, const int32_t *indices,
+                                        const int32_t *locations, int64_t plane_stride, int top_k,
+                                        int samples, int model_dim, int experts, int capacity,
+                                        uint8_t *codes, void *bias, void *scale, float *grad_gates,
+                                        void *workspace, size_t workspace_bytes, void *stream)
+{
+    PM_REQUIRE(gates && expert_out && grad_gates,
+               "planmoe_combine_bwd_int8: gates, expert_out and grad_gates must not be NULL");
+    return run_dispatch_int8("planmoe_combine_bwd_int8", grad_out, dtype, gates, indices, locations,
+                             plane_stride, top_k, samples, model_dim, experts, capacity, codes, bias, scale,
+                             workspace, workspace_bytes, expert_out, grad_gates, stream);
 }

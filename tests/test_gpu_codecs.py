@@ -223,3 +223,37 @@ def test_compressor_registry_round_trips():
     assert d.dtype == torch.bfloat16 and d.shape == bx.shape
     rc, rb, rs = oracle.int8_compress(bf16_bits(bx))
     assert np.array_equal(raw(d), np_raw(oracle.int8_decompress(rc, rb, rs)))
+
+
+@pytest.mark.parametrize("T,M,E,k,cf,dtype", [(300, 1024, 8, 2, 0.75, torch.bfloat16), (100, 256, 4, 3, 1.0, torch.float32),
+                                              (64, 20000, 4, 2, 0.5, torch.bfloat16)])
+def test_combine_bwd_int8_equals_the_unfused_backward(T, M, E, k, cf, dtype):
+    """Config-4 fusion: scatter of gate * grad_out, gate gradients and the int8 compress of the
+    gradient buffer in one launch against dispatch_fwd + bwd_gate + int8_compress and the oracle."""
+    from planmoe_amd import ops
+    scores = tie_free_scores(T, E, k, seed=T + 1).numpy()
+    idx, loc, gates, _ = oracle.route_topk(scores, k)
+    C = oracle.capacity(T, E, k, cf, 4)
+    g = torch.Generator().manual_seed(7)
+    dout = torch.randn(T, M, generator=g).to(dtype)
+    eo = torch.randn(E * C, M, generator=g).to(dtype)
+    i = [torch.from_numpy(a).to(DEV) for a in idx]
+    l = [torch.from_numpy(a).to(DEV) for a in loc]
+    gt = [torch.from_numpy(a).to(DEV) for a in gates]
+    codes, bias, scale, gg = ops.combine_bwd_int8(dout.to(DEV), eo.to(DEV), i, l, gt, E, C)
+    d = torch.from_numpy(oracle.encode(dout.float().numpy(), list(idx), list(loc), list(gates), E, C)).to(dtype)
+    rc, rb, rs = oracle.int8_compress(to_np(d))
+    assert np.array_equal(codes.cpu().numpy(), rc)
+    assert np.array_equal(raw(bias), np_raw(rb)) and np.array_equal(raw(scale), np_raw(rs))
+    c2, b2, s2 = ops.int8_compress(ops.dispatch_fwd(dout.to(DEV), i, l, gt, E, C))
+    assert torch.equal(codes, c2) and np.array_equal(raw(bias), raw(b2))
+    g2 = ops.bwd_gate(dout.to(DEV), eo.to(DEV), i, l, C)
+    xd, ed = dout.double().numpy(), eo.double().numpy()
+    rtol = 1e-5 if dtype == torch.float32 else 1e-2
+    for j in range(k):
+        want = oracle.bwd_gate(idx[j], loc[j], xd, ed, C)
+        mag = oracle.bwd_gate(idx[j], loc[j], np.abs(xd), np.abs(ed), C)
+        got = gg[j].cpu().numpy()
+        assert (np.abs(got - want) <= rtol * np.abs(want) + 1e-6 * mag).all()
+        assert (got[loc[j] >= C] == 0).all()
+        assert np.allclose(got, g2[j].cpu().numpy(), rtol=1e-5, atol=1e-6 * mag.max())
