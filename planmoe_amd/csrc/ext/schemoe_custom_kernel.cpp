@@ -1,0 +1,230 @@
+// Torch C++ extension with the reference's pybind surface for the codec pipeline
+// (custom/custom_kernel.cpp:194-321): the AbstractCompressor classes, their registry, and
+// compress_operation / comm_operation / decompress_operation / clear_ptr_lst, plus
+// torch.ops.tutel_ops.cumsum (custom_kernel.cpp:331-385).  All device work goes through the C
+// ABI of libplanmoe_hip; this file only owns tensors and object lifetimes.
+// One GPU: the comm step copies into g_output on the current stream.
+#include "planmoe/compressor/abstract.h"
+#include "planmoe/compressor/int8.h"
+#include "planmoe/compressor/no.h"
+#include "planmoe/compressor/zfpc.h"
+#include "planmoe_hip.h"
+
+#include <hip/hip_runtime_api.h>
+#include <torch/script.h>
+
+static void *current_stream() { return (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
+
+static int pm_dtype(const torch::Tensor &t)
+{
+    switch (t.scalar_type()) {
+    case at::kFloat: return PLANMOE_F32;
+    case at::kBFloat16: return PLANMOE_BF16;
+    case at::kHalf: return PLANMOE_F16;
+    default: AT_ASSERTM(false, "planmoe: unsupported dtype (float32, bfloat16 or float16)"); return -1;
+    }
+}
+#define PM_CALL(expr) AT_ASSERTM((expr) == 0, planmoe_last_error())
+#define CHECK_GPU(x) AT_ASSERTM((x).is_cuda(), #x " must be a GPU tensor (this build has no CPU path)")
+
+// ---------------------------------------------------------------- comm
+AbstractComm::AbstractComm(std::vector<PlanMoEStream> *stream, std::vector<ncclComm_t> g_nccl_comm,
+                           const int &g_world_size, const int &g_world_rank, const int &g_local_size,
+                           const int &g_local_rank) :
+    stream(stream), g_nccl_comm(g_nccl_comm), g_world_size(g_world_size), g_world_rank(g_world_rank),
+    g_local_size(g_local_size), g_local_rank(g_local_rank) {}
+void AbstractComm::pre_comm(const torch::Tensor &) {}
+AbstractComm::~AbstractComm() {}
+
+IdentityComm::IdentityComm(std::vector<PlanMoEStream> *stream, std::vector<ncclComm_t> comm, const int &ws,
+                           const int &wr, const int &ls, const int &lr) :
+    AbstractComm(stream, comm, ws, wr, ls, lr) {}
+void IdentityComm::all_to_all(const torch::Tensor &input, const torch::Tensor &output, size_t length)
+{
+    AT_ASSERTM(g_world_size == 1, "IdentityComm is the one-GPU all-to-all");
+    AT_ASSERTM(hipMemcpyAsync(output.data_ptr(), input.data_ptr(), length, hipMemcpyDeviceToDevice,
+                              (hipStream_t)current_stream()) == hipSuccess, "all_to_all copy failed");
+}
+
+// ---------------------------------------------------------------- compressors
+AbstractCompressor::AbstractCompressor(std::shared_ptr<AbstractComm> comm_ptr) { this->comm_ptr = comm_ptr; }
+AbstractCompressor::~AbstractCompressor() { comm_ptr.reset(); }
+void AbstractCompressor::pre_comm(const PlanMoEStream *) {}
+
+NoCompressor::NoCompressor(std::shared_ptr<AbstractComm> comm_ptr) : AbstractCompressor(comm_ptr) {}
+torch::Tensor NoCompressor::compress(const torch::Tensor &input)
+{
+    g_output = at::empty_like(input);
+    return input;
+}
+torch::Tensor NoCompressor::decompress(const torch::Tensor &input) { return input; }
+void NoCompressor::all_to_all(const torch::Tensor &input, const torch::Tensor &output)
+{
+    comm_ptr->all_to_all(input, output, input.nbytes());
+}
+
+Int8Compressor::Int8Compressor(std::shared_ptr<AbstractComm> comm_ptr) : AbstractCompressor(comm_ptr) {}
+torch::Tensor Int8Compressor::compress(const torch::Tensor &input_)
+{
+    CHECK_GPU(input_);
+    const torch::Tensor input = input_.contiguous();
+    sizes = input.sizes().vec();
+    dtype = input.dtype();
+    length = (size_t)input.numel();
+    AT_ASSERTM(!sizes.empty() && sizes.back() > 0, "int8: empty rows");
+    const int64_t M = sizes.back(), rows = input.numel() / M;
+    std::vector<int64_t> rshape(sizes.begin(), sizes.end());
+    rshape.back() = 1;
+    bias = torch::empty(rshape, input.options());
+    scale = torch::empty(rshape, input.options());
+    torch::Tensor fp_output = torch::empty({(int64_t)((length + 3) / 4)}, input.options().dtype(at::kFloat));
+    PM_CALL(planmoe_int8_compress(input.data_ptr(), pm_dtype(input), rows, (int)M, (uint8_t *)fp_output.data_ptr(),
+                                  bias.data_ptr(), scale.data_ptr(), current_stream()));
+    g_bias = at::empty_like(bias);
+    g_scale = at::empty_like(scale);
+    this->g_output = at::empty_like(fp_output);
+    return fp_output;
+}
+torch::Tensor Int8Compressor::decompress(const torch::Tensor &input)
+{
+    CHECK_GPU(input);
+    std::vector<int64_t> shape(sizes.begin(), sizes.end());
+    torch::Tensor output = torch::empty(shape, input.options().dtype(dtype));
+    const int64_t M = sizes.back(), rows = output.numel() / M;
+    PM_CALL(planmoe_int8_decompress((const uint8_t *)input.data_ptr(), g_bias.data_ptr(), g_scale.data_ptr(),
+                                    pm_dtype(output), rows, (int)M, output.data_ptr(), current_stream()));
+    return output;
+}
+void Int8Compressor::pre_comm(const PlanMoEStream *) {}
+void Int8Compressor::all_to_all(const torch::Tensor &input, const torch::Tensor &output)
+{
+    comm_ptr->all_to_all(input, output, length);
+    comm_ptr->all_to_all(bias, g_bias, bias.nbytes());
+    comm_ptr->all_to_all(scale, g_scale, scale.nbytes());
+}
+
+ZfpCompressor::ZfpCompressor(std::shared_ptr<AbstractComm> comm_ptr, double compress_rate) noexcept :
+    AbstractCompressor(comm_ptr)
+{
+    this->compress_rate = compress_rate;
+    this->buffer = nullptr;
+    this->last_bufsize = 0;
+}
+ZfpCompressor::~ZfpCompressor() { buffer = nullptr; }
+void ZfpCompressor::set_compress_rate(const double &rate) { this->compress_rate = rate; }
+torch::Tensor ZfpCompressor::compress(const torch::Tensor &input_)
+{
+    CHECK_GPU(input_);
+    const torch::Tensor input = input_.contiguous();
+    sizes = input.sizes().vec();
+    AT_ASSERTM(sizes.size() == 3, "zfp fails.");
+    AT_ASSERTM(sizes[0] % 4 == 0, "zfp fails.");
+    AT_ASSERTM(sizes[1] % 4 == 0, "zfp fails.");
+    AT_ASSERTM(sizes[2] % 4 == 0, "zfp fails.");
+    AT_ASSERTM(input.scalar_type() == at::kFloat, "zfp: the codec reads the buffer as fp32; pass a float32 tensor");
+    const int64_t nx = sizes[2], ny = sizes[1] * sizes[0];
+    const size_t bufsize = planmoe_zfp_max_bytes(2, nx, ny, compress_rate);
+    torch::Tensor output = torch::zeros({(int64_t)((bufsize + 1) / 2)}, input.options().dtype(at::kHalf));
+    PM_CALL(planmoe_zfp_compress((const float *)input.data_ptr(), 2, nx, ny, compress_rate, output.data_ptr(),
+                                 bufsize, current_stream()));
+    length = planmoe_zfp_stream_bytes(2, nx, ny, compress_rate);
+    g_output = torch::empty_like(output);
+    return output;
+}
+torch::Tensor ZfpCompressor::decompress(const torch::Tensor &input)
+{
+    CHECK_GPU(input);
+    std::vector<int64_t> shape(sizes.begin(), sizes.end());
+    torch::Tensor output = torch::empty(shape, input.options().dtype(at::kFloat));
+    PM_CALL(planmoe_zfp_decompress(input.data_ptr(), 2, sizes[2], sizes[1] * sizes[0], compress_rate,
+                                   (float *)output.data_ptr(), current_stream()));
+    return output;
+}
+void ZfpCompressor::all_to_all(const torch::Tensor &input, const torch::Tensor &output)
+{
+    comm_ptr->all_to_all(input, output, length);
+}
+
+// ---------------------------------------------------------------- registry (custom_kernel.cpp:194-288)
+static std::vector<PlanMoEStream> g_streams;          // no comm streams on one GPU
+
+static AbstractCompressor *get_compressor(const std::string &name, std::shared_ptr<AbstractComm> comm_ptr)
+{
+    if (name == "int8") return new Int8Compressor(comm_ptr);
+    if (name == "zfp") return new ZfpCompressor(comm_ptr);
+    AT_ASSERTM(name != "lz", "the 'lz' compressor is not part of this build");
+    return new NoCompressor(comm_ptr);
+}
+static std::shared_ptr<AbstractComm> get_comm(const std::string &)
+{
+    // naive / pipe / dd / hetu are all the identity on one GPU
+    return std::make_shared<IdentityComm>(&g_streams, std::vector<ncclComm_t>(), 1, 0, 1, 0);
+}
+
+static std::vector<AbstractCompressor *> compress_ptr_lst;
+static int comm_cnt = 0;
+static int decompress_cnt = 0;
+
+static void clear_ptr_lst()
+{
+    for (auto &p : compress_ptr_lst) { delete p; p = nullptr; }
+    compress_ptr_lst.resize(0);
+    comm_cnt = 0;
+    decompress_cnt = 0;
+}
+static torch::Tensor compress_operation(const torch::Tensor &input, const std::string &str, const std::string &comm_name)
+{
+    compress_ptr_lst.emplace_back(get_compressor(str, get_comm(comm_name)));
+    return compress_ptr_lst.back()->compress(input);
+}
+static torch::Tensor comm_operation(const torch::Tensor &input)
+{
+    AT_ASSERTM(comm_cnt < (int)compress_ptr_lst.size() && compress_ptr_lst[comm_cnt],
+               "comm_operation: no matching compress_operation");
+    const int idx = comm_cnt++;
+    const PlanMoEStream original_stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    compress_ptr_lst[idx]->pre_comm(&original_stream);
+    compress_ptr_lst[idx]->all_to_all(input, compress_ptr_lst[idx]->g_output);
+    return compress_ptr_lst[idx]->g_output;
+}
+static torch::Tensor decompress_operation(const torch::Tensor &input)
+{
+    AT_ASSERTM(decompress_cnt < (int)compress_ptr_lst.size() && compress_ptr_lst[decompress_cnt],
+               "decompress_operation: no matching compress_operation");
+    const int idx = decompress_cnt++;
+    torch::Tensor output = compress_ptr_lst[idx]->decompress(input);
+    delete compress_ptr_lst[idx];
+    compress_ptr_lst[idx] = nullptr;
+    return output;
+}
+
+// the reference's CPU kernels are not part of this build: a CPU path would void the parity claim
+static void invoke_cpu_unavailable(const std::vector<torch::Tensor> &, const std::vector<int> &, int)
+{
+    AT_ASSERTM(false, "invoke_cpu_fp32/fp64: this build has no CPU kernels; pass GPU tensors");
+}
+
+torch::Tensor warp_cumsum(torch::Tensor x)
+{
+    CHECK_GPU(x);
+    AT_ASSERTM(x.dim() == 2, "CHECK_EQ fails.");
+    x = x.to(torch::kInt32).contiguous();
+    auto y = torch::empty_like(x);
+    const int T = (int)x.size(0), E = (int)x.size(1);
+    auto ws = torch::empty({(int64_t)planmoe_cumsum_workspace_bytes(T, E)}, x.options().dtype(at::kByte));
+    PM_CALL(planmoe_cumsum_sub_one((const int32_t *)x.data_ptr(), (int32_t *)y.data_ptr(), T, E, ws.data_ptr(),
+                                   (size_t)ws.numel(), current_stream()));
+    return y;
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    m.def("invoke_cpu_fp32", &invoke_cpu_unavailable, "not available in this build");
+    m.def("invoke_cpu_fp64", &invoke_cpu_unavailable, "not available in this build");
+    m.def("compress_operation", &compress_operation, "Compress Operation");
+    m.def("comm_operation", &comm_operation, "Comm Operation");
+    m.def("decompress_operation", &decompress_operation, "Decompress Operation");
+    m.def("clear_ptr_lst", &clear_ptr_lst, "Clear Ptr Lst");
+}
+
+TORCH_LIBRARY(tutel_ops, m) { m.def("cumsum", warp_cumsum); }
