@@ -89,6 +89,22 @@ int planmoe_route_topk(const void *input, int dtype, int input_is_logits, const 
                        void *scores_out, float *l_aux, int32_t *expert_counts,
                        void *workspace, size_t workspace_bytes, void *stream);
 
+/* Backward of planmoe_route_topk with respect to its input: what autograd derives from the
+ * tensor algebra of extract_critical (fast_dispatch.py:148, 170-172: gates are score entries,
+ * divided by their clamped sum) and of gshard_loss (losses.py:12-19: me depends on the scores,
+ * ce does not).
+ *   scores        [samples, experts] `dtype`, the scores routing ran on (scores_out)
+ *   grad_gates    `dtype` k planes: gradient arriving at the gates
+ *   grad_l_aux    optional fp32 scalar: gradient arriving at l_aux (needs first_choice_counts =
+ *                 row 0 of expert_counts)
+ *   through_softmax != 0: grad_scores receives the gradient of the logits instead
+ *                 (softmax backward applied; for input_is_logits callers)
+ *   grad_scores   out [samples, experts] `dtype` */
+int planmoe_route_bwd(const void *scores, int dtype, const int32_t *indices, const void *grad_gates,
+                      int64_t plane_stride, int samples, int experts, int top_k, int normalize_gate,
+                      const float *grad_l_aux, const int32_t *first_choice_counts,
+                      int through_softmax, void *grad_scores, void *stream);
+
 /* Gate logits  logits[samples, experts] = x[samples, model_dim] . wg[experts, model_dim]^T
  * (gates/top.py:20-26).  x and wg are in `dtype` (BF16: MFMA with fp32 accumulation; F32:
  * fp32 FMA); logits are written in `out_dtype` (F32 = the fp32_gate flow, or `dtype`). */

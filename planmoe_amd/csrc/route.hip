@@ -260,6 +260,52 @@ __global__ __launch_bounds__(TILE) void route_finish_kernel(
     }
 }
 
+// ------------------------------------------------------------------ routing backward
+// Gradient of the gates (and of the GShard loss) with respect to the scores, optionally carried
+// through the softmax to the logits.  One thread per token:
+//   g_j = s_j / D, D = max(sum_i s_i, eps)  =>  ds_j = (dg_j - [sum >= eps] * sum_i dg_i g_i) / D
+//   l_aux = sum_e me[e] ce[e] / T            =>  ds[t][e] += dl * ce[e] / T,  ce[e] = count0[e] * E / T
+//   softmax: dlogit_e = s_e * (ds_e - sum_i ds_i s_i)
+template <int DT>
+__global__ __launch_bounds__(256) void route_bwd_kernel(
+    const void *__restrict__ scores, const int32_t *__restrict__ indices, const void *__restrict__ dgates,
+    int64_t stride, int samples, int experts, int k, int normalize_gate, const float *__restrict__ dl_aux,
+    const int32_t *__restrict__ count0, int through_softmax, void *__restrict__ dscores)
+{
+    using E = Elem<DT>;
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= samples) return;
+    const int64_t base = (int64_t)t * experts;
+    const float dl = dl_aux ? dl_aux[0] : 0.f;
+    const float lscale = dl * ((float)experts / (float)samples) / (float)samples;
+    float sum = 0.f, dot = 0.f;
+    for (int j = 0; j < k; ++j) {
+        const float sj = E::load(scores, base + indices[(int64_t)j * stride + t]);
+        sum = (j == 0) ? sj : E::round(sum + sj);
+        dot += E::load(dgates, (int64_t)j * stride + t) * sj;
+    }
+    const float eps = DT == PLANMOE_F32 ? 1.1920928955078125e-07f : DT == PLANMOE_BF16 ? 0.0078125f : 0.0009765625f;
+    const bool norm = k > 1 && normalize_gate;
+    const float D = norm ? fmaxf(sum, eps) : 1.f;
+    const float corr = (norm && sum >= eps) ? dot / (D * D) : 0.f;      // sum_i dg_i g_i / D
+    auto ds_at = [&](int e) {
+        float v = count0 ? lscale * (float)count0[e] : 0.f;
+        for (int j = 0; j < k; ++j)
+            if (indices[(int64_t)j * stride + t] == e) v += E::load(dgates, (int64_t)j * stride + t) / D - corr;
+        return v;
+    };
+    if (!through_softmax) {
+        for (int e = 0; e < experts; ++e) E::store(dscores, base + e, ds_at(e));
+    } else {
+        float inner = 0.f;
+        for (int e = 0; e < experts; ++e) inner += ds_at(e) * E::load(scores, base + e);
+        for (int e = 0; e < experts; ++e) {
+            const float s = E::load(scores, base + e);
+            E::store(dscores, base + e, s * (ds_at(e) - inner));
+        }
+    }
+}
+
 // ------------------------------------------------------------------ stand-alone cumsum
 // out = cumsum(in, dim 0) - 1 over an int32 [samples, columns] matrix, three phases:
 // per-tile column sums, prefix of the tile sums, per-tile rescan with the tile's offset.
@@ -379,6 +425,26 @@ extern "C" int planmoe_cumsum_sub_one(const int32_t *in, int32_t *out, int sampl
     cumsum_scan_kernel<<<cgroups, 256, 0, st>>>(sums, tiles, columns);
     cumsum_tile_kernel<true><<<dim3(tiles, cgroups), 256, 0, st>>>(in, out, samples, columns, sums);
     PM_LAUNCH_CHECK("planmoe_cumsum_sub_one");
+    return 0;
+}
+
+extern "C" int planmoe_route_bwd(const void *scores, int dtype, const int32_t *indices, const void *grad_gates,
+                                 int64_t plane_stride, int samples, int experts, int top_k, int normalize_gate,
+                                 const float *grad_l_aux, const int32_t *first_choice_counts,
+                                 int through_softmax, void *grad_scores, void *stream)
+{
+    PM_REQUIRE(dtype_ok(dtype), "planmoe_route_bwd: bad dtype %d", dtype);
+    PM_REQUIRE(samples >= 0 && experts >= 1 && top_k >= 1, "planmoe_route_bwd: bad shape");
+    PM_REQUIRE(plane_stride >= samples, "planmoe_route_bwd: plane_stride < samples");
+    PM_REQUIRE(!grad_l_aux || first_choice_counts, "planmoe_route_bwd: grad_l_aux needs first_choice_counts");
+    if (samples == 0) return 0;
+    PM_REQUIRE(scores && indices && grad_gates && grad_scores, "planmoe_route_bwd: NULL argument");
+    const int k = top_k < experts ? top_k : experts;
+    PM_DTYPE_SWITCH(dtype, DT,
+        (route_bwd_kernel<DT><<<(samples + 255) / 256, 256, 0, (hipStream_t)stream>>>(
+            scores, indices, grad_gates, plane_stride, samples, experts, k, normalize_gate, grad_l_aux,
+            grad_l_aux ? first_choice_counts : nullptr, through_softmax, grad_scores)));
+    PM_LAUNCH_CHECK("planmoe_route_bwd");
     return 0;
 }
 

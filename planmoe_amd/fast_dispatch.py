@@ -103,12 +103,45 @@ class TutelMoeFastDispatcher:
 fast_dispatcher = TutelMoeFastDispatcher
 
 
+class _Route(torch.autograd.Function):
+    """Routing with gradients: forward = the routing kernels, backward = planmoe_route_bwd.
+    `inp` are scores, or logits when is_logits (softmax inside the kernel).  Outputs: gates
+    [k, T] and l_aux (differentiable), indices / locations / counts / scores (not)."""
+
+    @staticmethod
+    def forward(ctx, inp, top_k, is_logits, normalize_gate, want_l_aux):
+        r = ops.route_topk(inp.detach().contiguous(), top_k, is_logits=is_logits, normalize_gate=normalize_gate,
+                           want_scores=is_logits, want_l_aux=want_l_aux, want_counts=True)
+        scores = r["scores"] if is_logits else inp.detach().contiguous()
+        ctx.save_for_backward(scores, r["indices"], r["counts"])
+        ctx.normalize_gate, ctx.is_logits, ctx.want_l_aux = normalize_gate, is_logits, want_l_aux
+        l_aux = r["l_aux"] if want_l_aux else inp.new_zeros(())
+        ctx.mark_non_differentiable(r["indices"], r["locations"], r["counts"])
+        return r["gates"], l_aux, r["indices"], r["locations"], r["counts"]
+
+    @staticmethod
+    def backward(ctx, grad_gates, grad_l_aux, *unused):
+        scores, indices, counts = ctx.saved_tensors
+        if grad_gates is None:
+            grad_gates = torch.zeros((indices.shape[0], scores.shape[0]), dtype=scores.dtype, device=scores.device)
+        dl = grad_l_aux if (ctx.want_l_aux and grad_l_aux is not None) else None
+        grad = ops.route_bwd(scores, indices, grad_gates, ctx.normalize_gate, dl, counts if dl is not None else None,
+                             through_softmax=ctx.is_logits)
+        return grad, None, None, None, None
+
+
+def route(inp, top_k, is_logits=False, normalize_gate=True, want_l_aux=True):
+    """(gates [k,T], l_aux, indices [k,T], locations [k,T], counts [k,E]); gates and l_aux carry
+    gradients back to `inp` when it requires them."""
+    return _Route.apply(inp, top_k, is_logits, normalize_gate, want_l_aux)
+
+
 def extract_critical(scores, top_k, loss_fn=losses.gshard_loss, capacity_factor=1.0,
                      batch_prioritized_routing=False, normalize_gate=True, group=None, alignment=1):
     """fast_dispatch.py:140-195.  Returns ((E, indices_s, locations_s, gates_s, capacity), l_loss).
+    gates_s and the GShard l_loss carry gradients back into `scores`.
 
-    Not carried over yet: batch_prioritized_routing=True (raises) and gradients flowing from
-    the returned gates back into `scores`."""
+    Not carried over: batch_prioritized_routing=True (raises)."""
     if batch_prioritized_routing:
         raise NotImplementedError("extract_critical: batch_prioritized_routing is not built yet")
     if not scores.is_cuda:
@@ -116,16 +149,15 @@ def extract_critical(scores, top_k, loss_fn=losses.gshard_loss, capacity_factor=
     num_global_experts = int(scores.size(1))
     top_k = min(top_k, num_global_experts)
     want_kernel_loss = loss_fn is losses.gshard_loss
-    r = ops.route_topk(scores.detach().contiguous(), top_k, is_logits=False,
-                       normalize_gate=normalize_gate, want_l_aux=want_kernel_loss)
-    indices_s = [r["indices"][j] for j in range(top_k)]
-    locations_s = [r["locations"][j] for j in range(top_k)]
-    gates_s = [r["gates"][j] for j in range(top_k)]
+    gates, l_aux, indices, locations, _ = route(scores, top_k, False, normalize_gate, want_kernel_loss)
+    indices_s = [indices[j] for j in range(top_k)]
+    locations_s = [locations[j] for j in range(top_k)]
+    gates_s = [gates[j] for j in range(top_k)]
 
     if loss_fn is None:
         l_loss = None
     elif want_kernel_loss:
-        l_loss = r["l_aux"].to(scores.dtype)
+        l_loss = l_aux.to(scores.dtype)
     else:
         topk_indices = torch.stack(indices_s, dim=1).to(torch.int64)
         l_loss = loss_fn(scores, topk_indices)
@@ -135,7 +167,7 @@ def extract_critical(scores, top_k, loss_fn=losses.gshard_loss, capacity_factor=
         capacity = ops.capacity(samples, num_global_experts, top_k, capacity_factor, alignment)
     else:
         # data-dependent capacity (fast_dispatch.py:183-186); world size 1, so no all-reduce
-        capacity = int(torch.max(r["locations"])) + 1
+        capacity = int(torch.max(locations)) + 1
         if capacity_factor < 0:
             per_expert = (samples + num_global_experts - 1) // num_global_experts
             capacity = min(capacity, top_k * int(-capacity_factor * per_expert))

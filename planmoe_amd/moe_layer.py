@@ -13,7 +13,7 @@ from torch.nn import ModuleList
 from . import experts as _experts
 from . import gates as _gates
 from . import losses, ops
-from .fast_dispatch import extract_critical, fast_decode, fast_encode
+from .fast_dispatch import extract_critical, fast_decode, fast_encode, route
 from .overlap import a2a_ffn_overlap_forward
 
 
@@ -164,13 +164,13 @@ class MOELayer(torch.nn.Module):
         plain = (self.is_gshard_loss and not self.batch_prioritized_routing and cf > 0)
         if plain:
             # softmax, top-k, slots, gates and the GShard loss in one routing call
-            r = ops.route_topk(logits_w_noise.detach().contiguous(), k, is_logits=True,
-                               normalize_gate=self.normalize_gate, want_l_aux=True)
             kk = min(k, self.num_global_experts)
+            gates, l_aux, indices, locations, _ = route(logits_w_noise.contiguous(), kk, True,
+                                                        self.normalize_gate, True)
             cap = ops.capacity(x.size(0), self.num_global_experts, kk, cf, alignment)
-            crit = (self.num_global_experts, [r["indices"][j] for j in range(kk)],
-                    [r["locations"][j] for j in range(kk)], [r["gates"][j] for j in range(kk)], cap)
-            l_aux = r["l_aux"].to(logits.dtype)
+            crit = (self.num_global_experts, [indices[j] for j in range(kk)],
+                    [locations[j] for j in range(kk)], [gates[j] for j in range(kk)], cap)
+            l_aux = l_aux.to(logits.dtype)
         else:
             scores = torch.softmax(logits_w_noise, dim=1)
             if self.is_gshard_loss:

@@ -116,6 +116,25 @@ def route_topk(inp, top_k, is_logits=False, logit_bias=None, normalize_gate=True
     return dict(indices=idx, locations=loc, gates=gates, scores=scores, l_aux=l_aux, counts=counts)
 
 
+def route_bwd(scores, indices, grad_gates, normalize_gate=True, grad_l_aux=None, counts=None,
+              through_softmax=False):
+    """Gradient of route_topk's gates (and l_aux) with respect to the scores [T, E] (or the
+    logits when through_softmax).  indices int32 [k, T], grad_gates [k, T] in scores.dtype."""
+    _need_gpu(scores, "route_bwd")
+    scores = _contig(scores, "route_bwd")
+    T, E = scores.shape
+    k = indices.shape[0]
+    indices = _contig(indices, "route_bwd")
+    gg = grad_gates.to(scores.dtype).contiguous()
+    out = torch.empty_like(scores)
+    dl = None if grad_l_aux is None else grad_l_aux.to(torch.float32).reshape(1).contiguous()
+    c0 = None if counts is None else counts[0].contiguous()
+    check(lib.planmoe_route_bwd(_ptr(scores), _dt(scores, "route_bwd"), _ptr(indices), _ptr(gg), max(T, 1), T, E, k,
+                                int(bool(normalize_gate)), _ptr(dl), _ptr(c0), int(bool(through_softmax)),
+                                _ptr(out), _stream(scores)))
+    return out
+
+
 def gate_logits(x, wg, out_dtype=None):
     """logits[T, E] = x[T, M] @ wg[E, M]^T with fp32 accumulation."""
     _need_gpu(x, "gate_logits")

@@ -148,6 +148,8 @@ def test_moe_layer_trains_with_builtin_ffn():
     (y.float().pow(2).mean() + y.l_aux).backward()
     assert x.grad is not None and torch.isfinite(x.grad).all()
     assert layer.experts.batched_fc1_w.grad is not None
+    wg_grad = layer.gates[0].wg.weight.grad                    # gates and l_aux reach the gate weight
+    assert wg_grad is not None and torch.isfinite(wg_grad).all() and wg_grad.abs().sum() > 0
 
 
 @pytest.mark.parametrize("T,M,E,k,cf,dtype,fp32_gate,use_bias", [

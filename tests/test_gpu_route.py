@@ -138,3 +138,52 @@ def test_extract_critical_structure():
     # custom loss callables see (scores, top-k ids [T, k])
     (_, _, _, _, _), l2 = planmoe_amd.extract_critical(scores.to(DEV), 2, loss_fn=lambda s, ids: ids.float().mean())
     assert abs(float(l2) - float(np.stack(list(idx), 1).mean())) < 1e-5
+
+
+def _torch_routing_reference(scores64, idx, normalize, T, E):
+    """gates and GShard loss from the scores with torch ops in float64 (indices fixed)."""
+    idx_t = torch.from_numpy(idx.astype(np.int64))
+    raw_g = [scores64.gather(1, idx_t[j][:, None])[:, 0] for j in range(idx.shape[0])]
+    if normalize and len(raw_g) > 1:
+        denom = torch.clamp(sum(raw_g), min=torch.finfo(torch.float32).eps)
+        raw_g = [g / denom for g in raw_g]
+    mask = torch.zeros(T, E, dtype=torch.float64)
+    mask.scatter_(1, idx_t[0][:, None], E / T)
+    l_aux = torch.sum(scores64.sum(0) * mask.sum(0)) / T
+    return raw_g, l_aux
+
+
+@pytest.mark.parametrize("T,E,k,normalize", [(500, 8, 2, True), (300, 16, 3, False), (257, 64, 1, True)])
+def test_routing_gradients_match_autograd(T, E, k, normalize):
+    """extract_critical's gates and l_aux carry gradients into the scores: compared with
+    torch autograd of the same algebra in float64 (rtol 1e-5)."""
+    import planmoe_amd
+    scores = tie_free_scores(T, E, k, seed=T)
+    s_dev = scores.to(DEV).requires_grad_()
+    (_, idxs, locs, gates, C), l_aux = planmoe_amd.extract_critical(s_dev, k, normalize_gate=normalize)
+    g = torch.Generator().manual_seed(1)
+    w = [torch.randn(T, generator=g) for _ in range(k)]
+    loss = sum((gates[j] * w[j].to(DEV)).sum() for j in range(k)) + 3.0 * l_aux
+    loss.backward()
+    s64 = scores.double().requires_grad_()
+    idx = np.stack([i.cpu().numpy() for i in idxs])
+    ref_g, ref_l = _torch_routing_reference(s64, idx, normalize, T, E)
+    ref = sum((ref_g[j] * w[j].double()).sum() for j in range(k)) + 3.0 * ref_l
+    ref.backward()
+    assert torch.allclose(s_dev.grad.cpu().double(), s64.grad, rtol=1e-5, atol=1e-7)
+
+
+def test_routing_gradients_through_the_fused_softmax():
+    from planmoe_amd.fast_dispatch import route
+    T, E, k = 400, 8, 2
+    g = torch.Generator().manual_seed(2)
+    logits = torch.randn(T, E, generator=g)
+    l_dev = logits.to(DEV).requires_grad_()
+    gates, l_aux, indices, locations, counts = route(l_dev, k, True, True, True)
+    w = torch.randn(k, T, generator=g)
+    ((gates * w.to(DEV)).sum() + 2.0 * l_aux).backward()
+    l64 = logits.double().requires_grad_()
+    s64 = torch.softmax(l64, 1)
+    ref_g, ref_l = _torch_routing_reference(s64, indices.cpu().numpy(), True, T, E)
+    (sum((ref_g[j] * w[j].double()).sum() for j in range(k)) + 2.0 * ref_l).backward()
+    assert torch.allclose(l_dev.grad.cpu().double(), l64.grad, rtol=1e-4, atol=1e-7)
