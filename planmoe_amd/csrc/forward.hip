@@ -21,6 +21,7 @@
 #include "gate_core.hpp"
 #include "rows.hpp"
 #include "int8_core.hpp"
+#include "offsets.hpp"
 
 namespace pm {
 
@@ -120,9 +121,10 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
         if (l_aux) {
 #pragma unroll
             for (int e = 0; e < CAP; ++e) {
-                if (e >= experts) break;
-                const float v = wave_sum(valid ? s[e] : 0.f);
-                if (lane == 0) ws.me[(int64_t)blockIdx.x * experts + e] = v;
+                if (e < experts) {
+                    const float v = wave_sum(valid ? s[e] : 0.f);
+                    if (lane == 0) ws.me[(int64_t)blockIdx.x * experts + e] = v;
+                }
             }
         }
         float denom = 0.f;
@@ -175,127 +177,6 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
         }
     }
 
-}
-
-// One block per set of experts (all k planes of an expert stay together): 16 column lanes
-// (plane, expert) x 16 row lanes over the groups.  offs[g][j][e] = slots of expert e taken
-// before group g of plane j = all of planes < j + groups < g of plane j.
-constexpr int GO_COLS = 16, GO_ROWS = 16, GO_BATCH = 16, GO_KEEP = 32;
-
-__global__ __launch_bounds__(256) void group_offsets_kernel(
-    const int32_t *__restrict__ hist, int32_t *__restrict__ offs, const float *__restrict__ me,
-    int groups, int k, int experts, int experts_per_block, int samples,
-    int32_t *__restrict__ totals, int32_t *__restrict__ counts_out, float *__restrict__ loss_part,
-    int want_loss)
-{
-    __shared__ int32_t s_sum[GO_ROWS][GO_COLS];
-    __shared__ int32_t s_tot[GO_COLS];
-    __shared__ float s_me[GO_ROWS][GO_COLS];
-    const int cl = threadIdx.x % GO_COLS, rl = threadIdx.x / GO_COLS;
-    const int e0 = blockIdx.x * experts_per_block;
-    const int ne = min(experts_per_block, experts - e0);
-    // column cl = plane j, expert e0 + el, planes outermost so that plane 0 comes first
-    const int j = cl / experts_per_block, el = cl - j * experts_per_block;
-    const bool live = j < k && el < ne;
-    const int e = e0 + el;
-    const int per = (groups + GO_ROWS - 1) / GO_ROWS;
-    const int g0 = min(rl * per, groups), g1 = min(g0 + per, groups);
-
-    int32_t sum = 0;
-    float mes = 0.f;
-    int32_t keep[GO_KEEP];                               // this thread's rows, when they fit
-    const bool kept = per <= GO_KEEP;
-    if (live) {
-        if (kept) {
-#pragma unroll
-            for (int i = 0; i < GO_KEEP; ++i)
-                keep[i] = (g0 + i < g1) ? hist[((int64_t)(g0 + i) * k + j) * experts + e] : 0;
-#pragma unroll
-            for (int i = 0; i < GO_KEEP; ++i) sum += keep[i];
-        } else {
-            for (int g = g0; g < g1; g += GO_BATCH) {
-                int32_t v[GO_BATCH];
-#pragma unroll
-                for (int i = 0; i < GO_BATCH; ++i)
-                    v[i] = (g + i < g1) ? hist[((int64_t)(g + i) * k + j) * experts + e] : 0;
-#pragma unroll
-                for (int i = 0; i < GO_BATCH; ++i) sum += v[i];
-            }
-        }
-        if (want_loss && j == 0) {
-            for (int g = g0; g < g1; g += GO_BATCH) {
-                float v[GO_BATCH];
-#pragma unroll
-                for (int i = 0; i < GO_BATCH; ++i) v[i] = (g + i < g1) ? me[(int64_t)(g + i) * experts + e] : 0.f;
-#pragma unroll
-                for (int i = 0; i < GO_BATCH; ++i) mes += v[i];
-            }
-        }
-    }
-    s_sum[rl][cl] = sum;
-    s_me[rl][cl] = mes;
-    __syncthreads();
-    int32_t before = 0, total = 0;
-#pragma unroll
-    for (int r = 0; r < GO_ROWS; ++r) {
-        const int32_t v = s_sum[r][cl];
-        before += (r < rl) ? v : 0;
-        total += v;
-    }
-    if (rl == 0) s_tot[cl] = total;
-    __syncthreads();
-    int32_t base = 0;                                   // slots taken by the planes before j
-    for (int p = 0; p < j; ++p) base += s_tot[p * experts_per_block + el];
-    if (live) {
-        int32_t run = base + before;
-        if (kept) {
-#pragma unroll
-            for (int i = 0; i < GO_KEEP; ++i) {
-                if (g0 + i < g1) offs[((int64_t)(g0 + i) * k + j) * experts + e] = run;
-                run += keep[i];
-            }
-        } else {
-            for (int g = g0; g < g1; g += GO_BATCH) {
-                int32_t v[GO_BATCH];
-#pragma unroll
-                for (int i = 0; i < GO_BATCH; ++i)
-                    v[i] = (g + i < g1) ? hist[((int64_t)(g + i) * k + j) * experts + e] : 0;
-#pragma unroll
-                for (int i = 0; i < GO_BATCH; ++i) {
-                    if (g + i < g1) offs[((int64_t)(g + i) * k + j) * experts + e] = run;
-                    run += v[i];
-                }
-            }
-        }
-        if (rl == 0) {
-            if (counts_out) counts_out[j * experts + e] = total;
-            if (j == k - 1) totals[e] = base + total;
-        }
-    }
-    if (want_loss) {
-        // this block's share of sum_e(me[e] * ce[e]) / T, ce[e] = count0[e] * (E / T)
-        if (threadIdx.x < WAVE) {
-            float acc = 0.f;
-            if (threadIdx.x < ne) {
-                float m = 0.f;
-#pragma unroll
-                for (int r = 0; r < GO_ROWS; ++r) m += s_me[r][threadIdx.x];
-                acc = m * ((float)s_tot[threadIdx.x] * ((float)experts / (float)samples));
-            }
-            acc = wave_sum(acc);
-            if (threadIdx.x == 0) loss_part[blockIdx.x] = acc;
-        }
-    }
-}
-
-// l_aux = (sum of the per-block shares) / T, written by one thread of the launch
-__device__ __forceinline__ void finish_loss(const float *loss_part, int loss_parts, int samples, float *l_aux)
-{
-    if (l_aux && blockIdx.x == 0 && threadIdx.x == 0) {
-        float a = 0.f;
-        for (int b = 0; b < loss_parts; ++b) a += loss_part[b];
-        *l_aux = a / (float)samples;
-    }
 }
 
 // locations += offset of the token's group (routing only, no dispatch)
@@ -454,7 +335,6 @@ static int fused_check(const char *who, const void *x, const void *wg, int dtype
     PM_REQUIRE(samples >= 1 && model_dim >= 1 && experts >= 1 && top_k >= 1, "%s: bad shape", who);
     PM_REQUIRE(experts <= 64, "%s: the fused path supports up to 64 experts (got %d); use "
                "planmoe_gate_logits + planmoe_route_topk", who, experts);
-    PM_REQUIRE((top_k < experts ? top_k : experts) <= GO_COLS, "%s: the fused path supports top_k <= %d", who, GO_COLS);
     const int vec = dtype == PLANMOE_F32 ? 4 : 8;
     PM_REQUIRE(model_dim % vec == 0 && aligned16(x) && aligned16(wg),
                "%s: model_dim must be a multiple of %d and x / wg 16-byte aligned", who, vec);
@@ -478,8 +358,7 @@ static int run_gate_route(const void *x, const void *wg, int dtype, int fp32_gat
     plan.k = top_k < experts ? top_k : experts;
     plan.group_tokens = fwd_group_tokens(experts);
     plan.groups = (samples + plan.group_tokens - 1) / plan.group_tokens;
-    plan.experts_per_block = GO_COLS / plan.k;
-    if (plan.experts_per_block > experts) plan.experts_per_block = experts;
+    plan.experts_per_block = go_experts_per_block(experts, plan.k);
     plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
     plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts, samples);
     const int k = plan.k, groups = plan.groups;
@@ -606,8 +485,7 @@ extern "C" int planmoe_forward_int8_redispatch(const void *x, int dtype, int sam
     plan.k = top_k < experts ? top_k : experts;
     plan.group_tokens = fwd_group_tokens(experts);
     plan.groups = (samples + plan.group_tokens - 1) / plan.group_tokens;
-    plan.experts_per_block = GO_COLS / plan.k;
-    if (plan.experts_per_block > experts) plan.experts_per_block = experts;
+    plan.experts_per_block = go_experts_per_block(experts, plan.k);
     plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
     plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts, samples);
     if (run_dispatch_routed(x, dtype, samples, model_dim, experts, capacity, indices, locations,

@@ -8,12 +8,14 @@
 //                       k-fold arg-max, rank of the token among the tile's tokens that
 //                       chose the same expert (wave ballots + an LDS table), per-tile
 //                       expert histograms and per-tile column sums of the scores
-//   route_scan_kernel   exclusive prefix of the histograms over tiles, choice plane after
+//   group_offsets_kernel exclusive prefix of the histograms over tiles, choice plane after
 //                       choice plane, so that all first choices precede all second choices
 //   route_finish_kernel location = rank in tile + prefix; GShard loss
 //
-// Workspace layout (int32 words): hist[tiles][k][E] then me[tiles][E] (fp32).
+// Workspace layout (32-bit words): hist[tiles][k][E], offs[tiles][k][E], me[tiles][E] (fp32),
+// loss_part[E] (fp32).
 #include "common.hpp"
+#include "offsets.hpp"
 
 namespace pm {
 
@@ -100,9 +102,10 @@ __global__ __launch_bounds__(TILE) void route_tile_kernel(
         if constexpr (CAP > 0) {
 #pragma unroll
             for (int e = 0; e < CAP; ++e) {
-                if (e >= experts) break;
-                const float v = wave_sum(valid ? s[e] : 0.f);
-                if (lane == 0) wsum[wave * experts + e] = v;
+                if (e < experts) {
+                    const float v = wave_sum(valid ? s[e] : 0.f);
+                    if (lane == 0) wsum[wave * experts + e] = v;
+                }
             }
         } else {
             for (int e = 0; e < experts; ++e) {
@@ -181,82 +184,18 @@ __global__ __launch_bounds__(TILE) void route_tile_kernel(
     }
 }
 
-// One block per group of up to 64 experts; 256 threads = expert lanes x tile chunks.
-// hist[tile][j][e] is replaced by the number of slots of expert e taken before tile `tile`
-// of plane j: all of planes < j plus the tiles before it in plane j.
-__global__ __launch_bounds__(256) void route_scan_kernel(int32_t *__restrict__ hist, int tiles,
-                                                         int k, int experts,
-                                                         int32_t *__restrict__ counts_out,
-                                                         int32_t *__restrict__ counts_ws)
-{
-    __shared__ int32_t part[256];
-    const int eb = min(64, experts);                 // expert lanes in this block
-    int lanes_e = 1; while (lanes_e < eb) lanes_e <<= 1;
-    const int chunks = 256 / lanes_e;
-    const int el = threadIdx.x % lanes_e, ch = threadIdx.x / lanes_e;
-    const int e = blockIdx.x * 64 + el;
-    const bool live = el < eb && e < experts;
-    const int per = (tiles + chunks - 1) / chunks;
-    const int t0 = min(ch * per, tiles), t1 = min(t0 + per, tiles);
-
-    int32_t carry = 0;
-    for (int j = 0; j < k; ++j) {
-        int32_t s = 0;
-        if (live)
-            for (int t = t0; t < t1; ++t) s += hist[((int64_t)t * k + j) * experts + e];
-        part[threadIdx.x] = s;
-        __syncthreads();
-        int32_t before = 0, total = 0;
-        for (int c = 0; c < chunks; ++c) {
-            const int32_t v = part[c * lanes_e + el];
-            before += (c < ch) ? v : 0;
-            total += v;
-        }
-        if (live) {
-            int32_t run = carry + before;
-            for (int t = t0; t < t1; ++t) {
-                const int64_t o = ((int64_t)t * k + j) * experts + e;
-                const int32_t v = hist[o];
-                hist[o] = run;
-                run += v;
-            }
-            if (ch == 0) {
-                if (counts_out) counts_out[j * experts + e] = total;
-                if (j == 0) counts_ws[e] = total;
-            }
-        }
-        carry += total;
-        __syncthreads();
-    }
-}
-
+// location = rank in tile + offset of the tile; one thread of the launch finishes the loss
 __global__ __launch_bounds__(TILE) void route_finish_kernel(
     const int32_t *__restrict__ indices, int32_t *__restrict__ locations, int64_t stride,
-    int samples, int experts, int k, const int32_t *__restrict__ hist,
-    const float *__restrict__ me_part, const int32_t *__restrict__ counts_ws, int tiles,
-    float *__restrict__ l_aux)
+    int samples, int experts, int k, const int32_t *__restrict__ offs,
+    const float *__restrict__ loss_part, int loss_parts, float *__restrict__ l_aux)
 {
+    finish_loss(loss_part, loss_parts, samples, l_aux);
     const int t = blockIdx.x * TILE + threadIdx.x;
-    if (t < samples) {
-        for (int j = 0; j < k; ++j) {
-            const int64_t o = (int64_t)j * stride + t;
-            locations[o] += hist[((int64_t)blockIdx.x * k + j) * experts + indices[o]];
-        }
-    }
-    if (l_aux && blockIdx.x == 0) {
-        // l_aux = sum_e(me[e] * ce[e]) / T, ce[e] = count0[e] * (E / T)
-        __shared__ float red[TILE / WAVE];
-        float acc = 0.f;
-        for (int e = threadIdx.x; e < experts; e += TILE) {
-            float me = 0.f;
-            for (int tl = 0; tl < tiles; ++tl) me += me_part[(int64_t)tl * experts + e];
-            const float ce = (float)counts_ws[e] * ((float)experts / (float)samples);
-            acc += me * ce;
-        }
-        acc = wave_sum(acc);
-        if (lane_id() == 0) red[threadIdx.x >> 6] = acc;
-        __syncthreads();
-        if (threadIdx.x == 0) *l_aux = (((red[0] + red[1]) + red[2]) + red[3]) / (float)samples;
+    if (t >= samples) return;
+    for (int j = 0; j < k; ++j) {
+        const int64_t o = (int64_t)j * stride + t;
+        locations[o] += offs[((int64_t)blockIdx.x * k + j) * experts + indices[o]];
     }
 }
 
@@ -365,36 +304,6 @@ __global__ __launch_bounds__(256) void cumsum_tile_kernel(const int32_t *__restr
     }
 }
 
-// exclusive prefix over tiles, in place; same thread geometry as route_scan_kernel
-__global__ __launch_bounds__(256) void cumsum_scan_kernel(int32_t *__restrict__ tile_sums, int tiles,
-                                                          int columns)
-{
-    __shared__ int32_t part[256];
-    const int cb = min(64, columns);
-    int lanes_c = 1; while (lanes_c < cb) lanes_c <<= 1;
-    const int chunks = 256 / lanes_c;
-    const int cl = threadIdx.x % lanes_c, ch = threadIdx.x / lanes_c;
-    const int c = blockIdx.x * 64 + cl;
-    const bool live = cl < cb && c < columns;
-    const int per = (tiles + chunks - 1) / chunks;
-    const int t0 = min(ch * per, tiles), t1 = min(t0 + per, tiles);
-    int32_t s = 0;
-    if (live) for (int t = t0; t < t1; ++t) s += tile_sums[(int64_t)t * columns + c];
-    part[threadIdx.x] = s;
-    __syncthreads();
-    int32_t before = 0;
-    for (int q = 0; q < ch; ++q) before += part[q * lanes_c + cl];
-    if (live) {
-        int32_t run = before;
-        for (int t = t0; t < t1; ++t) {
-            const int64_t o = (int64_t)t * columns + c;
-            const int32_t v = tile_sums[o];
-            tile_sums[o] = run;
-            run += v;
-        }
-    }
-}
-
 } // namespace pm
 
 using namespace pm;
@@ -404,7 +313,7 @@ extern "C" size_t planmoe_cumsum_workspace_bytes(int samples, int columns)
     if (samples <= 0 || columns <= 0) return 16;
     const CsGeom g = cs_geom(columns);
     const size_t tiles = ((size_t)samples + g.tile_rows - 1) / g.tile_rows;
-    return round_up(tiles * (size_t)columns * sizeof(int32_t), 256);
+    return round_up(2 * tiles * (size_t)columns * sizeof(int32_t), 256);     // tile sums + their prefix
 }
 
 extern "C" int planmoe_cumsum_sub_one(const int32_t *in, int32_t *out, int samples, int columns,
@@ -421,9 +330,12 @@ extern "C" int planmoe_cumsum_sub_one(const int32_t *in, int32_t *out, int sampl
     PM_REQUIRE(cgroups <= 65535, "planmoe_cumsum_sub_one: too many columns");
     hipStream_t st = (hipStream_t)stream;
     int32_t *sums = (int32_t *)workspace;
+    int32_t *prefix = sums + (size_t)tiles * columns;
     cumsum_tile_kernel<false><<<dim3(tiles, cgroups), 256, 0, st>>>(in, out, samples, columns, sums);
-    cumsum_scan_kernel<<<cgroups, 256, 0, st>>>(sums, tiles, columns);
-    cumsum_tile_kernel<true><<<dim3(tiles, cgroups), 256, 0, st>>>(in, out, samples, columns, sums);
+    const int epb = go_experts_per_block(columns, 1);
+    group_offsets_kernel<<<(columns + epb - 1) / epb, 256, 0, st>>>(sums, prefix, nullptr, tiles, 1, columns, epb,
+                                                                   samples, nullptr, nullptr, nullptr, 0);
+    cumsum_tile_kernel<true><<<dim3(tiles, cgroups), 256, 0, st>>>(in, out, samples, columns, prefix);
     PM_LAUNCH_CHECK("planmoe_cumsum_sub_one");
     return 0;
 }
@@ -455,8 +367,8 @@ extern "C" size_t planmoe_route_workspace_bytes(int samples, int experts, int to
     if (samples <= 0 || experts <= 0 || top_k <= 0) return 16;
     const size_t k = (size_t)(top_k < experts ? top_k : experts);
     const size_t tiles = route_tiles(samples);
-    // hist[tiles][k][E] + me[tiles][E] + count0[E]
-    return round_up((tiles * k * experts + tiles * experts + (size_t)experts) * 4, 256);
+    // hist[tiles][k][E] + offs[tiles][k][E] + me[tiles][E] + loss_part[E]
+    return round_up((2 * tiles * k * experts + tiles * experts + (size_t)experts) * 4, 256);
 }
 
 template <int DT>
@@ -502,17 +414,21 @@ extern "C" int planmoe_route_topk(const void *input, int dtype, int input_is_log
                planmoe_route_workspace_bytes(samples, experts, top_k));
     const int tiles = (int)route_tiles(samples);
     int32_t *hist = (int32_t *)workspace;
-    float *me = (float *)(hist + (size_t)tiles * k * experts);
-    int32_t *count0 = (int32_t *)(me + (size_t)tiles * experts);
+    int32_t *offs = hist + (size_t)tiles * k * experts;
+    float *me = (float *)(offs + (size_t)tiles * k * experts);
+    float *loss_part = me + (size_t)tiles * experts;
     const size_t lds = sizeof(int32_t) * 4 * (size_t)experts;
 
     PM_DTYPE_SWITCH(dtype, DT,
         launch_route_tile<DT>(experts, dim3(tiles), lds, st, input, input_is_logits, logit_bias,
                               samples, experts, k, normalize_gate, indices, locations, gates,
                               plane_stride, scores_out, hist, l_aux ? me : nullptr));
-    route_scan_kernel<<<(experts + 63) / 64, 256, 0, st>>>(hist, tiles, k, experts, expert_counts, count0);
-    route_finish_kernel<<<tiles, TILE, 0, st>>>(indices, locations, plane_stride, samples, experts, k,
-                                               hist, me, count0, tiles, l_aux);
+    const int epb = go_experts_per_block(experts, k);
+    const int blocks = (experts + epb - 1) / epb;
+    group_offsets_kernel<<<blocks, 256, 0, st>>>(hist, offs, me, tiles, k, experts, epb, samples, nullptr,
+                                                 expert_counts, loss_part, l_aux != nullptr);
+    route_finish_kernel<<<tiles, TILE, 0, st>>>(indices, locations, plane_stride, samples, experts, k, offs,
+                                               loss_part, blocks, l_aux);
     PM_LAUNCH_CHECK("planmoe_route_topk");
     return 0;
 }
