@@ -1,11 +1,12 @@
 // Gate logits: logits[T, E] = x[T, M] . wg[E, M]^T  (gates/top.py:20-26).
 //
-// The GEMM is skinny (E is 2..64) and bound by reading x once from HBM; the matrix cores
+// The GEMM is skinny (E is 2..128) and bound by reading x once from HBM; the matrix cores
 // (MFMA 16x16 tiles, fp32 accumulation) keep the arithmetic off the critical path.
-// A work-group of 4 waves owns 16*TPW tokens; the K axis is dealt to the 4 waves in 16-vector
-// steps (round robin, so the group streams 1 KB of every token row at a time) and the 4
-// partial tiles meet in LDS, summed in a fixed order.  Both MFMA operands use the same
-// lane -> k mapping, chosen so that each lane reads 64 contiguous bytes of its row per step.
+// Up to 16 experts: a work-group of 4 waves owns 16*TPW tokens; the K axis is dealt to the 4
+// waves in 16-vector steps (round robin, so the group streams 1 KB of every token row at a
+// time) and the 4 partial tiles meet in LDS, summed in a fixed order.  Both MFMA operands use
+// the same lane -> k mapping.  17..128 experts: the gate weights are staged through LDS once per
+// work-group of 64 tokens and every wave runs the whole K axis for its 16 tokens.
 #include "gate_core.hpp"
 
 namespace pm {
@@ -27,6 +28,28 @@ __global__ __launch_bounds__(64 * NW) void gate_logits_kernel(
 #pragma unroll
         for (int w = 1; w < NW; ++w) v += part[w][r][e];
         const int64_t o = (int64_t)t * experts + e;
+        if (out_dt == PLANMOE_F32) ((float *)logits)[o] = v;
+        else if (out_dt == PLANMOE_BF16) ((uint16_t *)logits)[o] = (uint16_t)f32_to_bf16(v);
+        else ((uint16_t *)logits)[o] = (uint16_t)f32_to_f16(v);
+    }
+}
+
+// more than 16 experts: gate weights shared through LDS, 64 tokens per work-group
+template <int DT, int NT>
+__global__ __launch_bounds__(256) void gate_logits_lds_kernel(
+    const void *__restrict__ x, const void *__restrict__ wg, void *__restrict__ logits, int out_dt,
+    int samples, int model_dim, int experts)
+{
+    __shared__ uint4 smem[gate_lds_vectors<NT>()];
+    const int t0 = blockIdx.x * 64;
+    gate_tile_lds<DT, NT>(x, wg, t0, samples, model_dim, experts, smem);
+    __syncthreads();
+    const float (*tile)[16 * NT + 1] = reinterpret_cast<const float (*)[16 * NT + 1]>(smem);
+    const int rows = min(64, samples - t0);
+    for (int i = threadIdx.x; i < rows * experts; i += 256) {
+        const int r = i / experts, e = i - r * experts;
+        const float v = tile[r][e];
+        const int64_t o = (int64_t)t0 * experts + i;
         if (out_dt == PLANMOE_F32) ((float *)logits)[o] = v;
         else if (out_dt == PLANMOE_BF16) ((uint16_t *)logits)[o] = (uint16_t)f32_to_bf16(v);
         else ((uint16_t *)logits)[o] = (uint16_t)f32_to_f16(v);
@@ -64,9 +87,14 @@ static void launch_gate_logits(const void *x, const void *wg, void *logits, int 
 #define PM_GATE(NT, TPW, NW)                                                                      \
     gate_logits_kernel<DT, NT, TPW, NW><<<(samples + 16 * TPW - 1) / (16 * TPW), 64 * NW, 0, st>>>(  \
         x, wg, logits, out_dt, samples, model_dim, experts)
+#define PM_GATE_LDS(NT)                                                                           \
+    gate_logits_lds_kernel<DT, NT><<<(samples + 63) / 64, 256, 0, st>>>(x, wg, logits, out_dt, samples, \
+                                                                        model_dim, experts)
     if (experts <= 16) PM_GATE(1, 4, 4);
-    else if (experts <= 32) PM_GATE(2, 2, 4);
-    else PM_GATE(4, 2, 4);
+    else if (experts <= 32) PM_GATE_LDS(2);
+    else if (experts <= 64) PM_GATE_LDS(4);
+    else PM_GATE_LDS(8);
+#undef PM_GATE_LDS
 #undef PM_GATE
 }
 
@@ -85,7 +113,7 @@ extern "C" int planmoe_gate_logits(const void *x, const void *wg, int dtype, voi
     if (samples == 0) return 0;
     PM_REQUIRE(x && wg && logits, "planmoe_gate_logits: NULL argument");
     const int vec = dtype == PLANMOE_F32 ? 4 : 8;
-    const bool mfma = experts <= 64 && model_dim % vec == 0 && aligned16(x) && aligned16(wg);
+    const bool mfma = experts <= 128 && model_dim % vec == 0 && aligned16(x) && aligned16(wg);
     PM_DTYPE_SWITCH(dtype, DT, launch_gate_logits<DT>(x, wg, logits, out_dtype, samples, model_dim,
                                                       experts, mfma, (hipStream_t)stream));
     PM_LAUNCH_CHECK("planmoe_gate_logits");

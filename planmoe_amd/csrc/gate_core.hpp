@@ -12,6 +12,9 @@ typedef _Float16 f16x8  __attribute__((ext_vector_type(8)));
 // One 16-byte vector per lane of each operand -> one 16x16 tile update.
 // Lane l carries row (l % 16) of its operand and the k-slice selected by (l / 16); both
 // operands use the same k-slice, so any assignment of k values to (l / 16, element) is valid.
+// Here vector s of lane (m, g) is vector 4 s + g of the step: the four lanes of a row read 64
+// contiguous bytes with one load instruction, which keeps the number of cache lines an
+// instruction touches at 16.
 template <int DT> struct Mma;
 
 template <> struct Mma<PLANMOE_BF16> {
@@ -77,12 +80,12 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
     bool bv[NT];                                     // lane holds a real gate-weight row
 #pragma unroll
     for (int tp = 0; tp < TPW; ++tp)
-        ap[tp] = reinterpret_cast<const uint4 *>(x) + (int64_t)min(t0 + tp * 16 + m, samples - 1) * nv + g * 4;
+        ap[tp] = reinterpret_cast<const uint4 *>(x) + (int64_t)min(t0 + tp * 16 + m, samples - 1) * nv + g;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
     {
         bv[nt] = nt * 16 + m < experts;
-        bp[nt] = reinterpret_cast<const uint4 *>(wg) + (int64_t)min(nt * 16 + m, experts - 1) * nv + g * 4;
+        bp[nt] = reinterpret_cast<const uint4 *>(wg) + (int64_t)min(nt * 16 + m, experts - 1) * nv + g;
     }
 
     f32x4 acc[TPW][NT];
@@ -96,14 +99,14 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
 #pragma unroll
         for (int tp = 0; tp < TPW; ++tp)
 #pragma unroll
-            for (int s = 0; s < 4; ++s) f.a[tp][s] = ap[tp][o + s];
+            for (int s = 0; s < 4; ++s) f.a[tp][s] = ap[tp][o + s * 4];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             // lanes past the last expert skip the load: whatever their registers hold only
             // reaches tile columns nobody reads
             if (bv[nt]) {
 #pragma unroll
-                for (int s = 0; s < 4; ++s) f.b[nt][s] = bp[nt][o + s];
+                for (int s = 0; s < 4; ++s) f.b[nt][s] = bp[nt][o + s * 4];
             }
         }
     };
@@ -139,8 +142,8 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
         const int o = full * 16;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const bool in = g * 4 + s < rem;
-            const int off = in ? o + s : o - g * 4;   // out of range: re-read vector `o` of the row, then zero it
+            const bool in = s * 4 + g < rem;
+            const int off = in ? o + s * 4 : o - g;   // out of range: re-read vector `o` of the row, then zero it
 #pragma unroll
             for (int tp = 0; tp < TPW; ++tp) {
                 uint4 v = ap[tp][off];
@@ -184,6 +187,139 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) part[w][tp * 16 + 4 * g + i][nt * 16 + m] = acc[tp][nt][i];
+}
+
+// ---------------------------------------------------------------------------------------------
+// Variant for more than 16 experts: the gate weights are the larger operand per token tile, so
+// the work-group shares them through LDS instead of every wave streaming them from L2.
+//   * a work-group of 4 waves owns 64 tokens, wave w the tokens [16 w, 16 w + 16) over the
+//     whole K axis (no split-K: the accumulators of a token stay in one wave);
+//   * K is walked in chunks of 16 vectors (256 bytes of every row).  The chunk of all 16*NT
+//     gate-weight rows is copied global -> registers -> LDS by the 256 threads with fully
+//     coalesced 16-byte loads, double buffered, one barrier per chunk;
+//   * inside LDS a row's 16 vectors are stored at (vector ^ (row % 16)): the 16 lanes of an
+//     MFMA fragment read (different rows, same logical vector) hit 16 different vector slots,
+//     i.e. all 64 banks once;
+//   * token fragments go straight from global memory to registers, one chunk ahead.
+// Result: logits[token][expert] (fp32) in LDS.  `smem` must hold gate_lds_vectors<NT>() uint4;
+// the logits alias the weight buffers (a barrier separates the two uses).
+// With STATS the wave leaves the words of RowStats<bf16>::reduced() of its rows in pstat[token].
+template <int NT> __host__ __device__ constexpr int gate_lds_vectors()
+{
+    // 2 buffers x (16 NT rows x 16 vectors)  vs  64 x (16 NT + 1) floats
+    return (2 * 16 * NT * 16) > ((64 * (16 * NT + 1) + 3) / 4) ? (2 * 16 * NT * 16) : ((64 * (16 * NT + 1) + 3) / 4);
+}
+
+template <int DT, int NT, bool STATS = false>
+__device__ __forceinline__ void gate_tile_lds(const void *__restrict__ x, const void *__restrict__ wg,
+                                              int t0, int samples, int model_dim, int experts,
+                                              uint4 *smem, int32_t (*pstat)[3] = nullptr)
+{
+    static_assert(!STATS || DT == PLANMOE_BF16, "row statistics ride along for bf16 only");
+    static_assert(NT == 1 || NT == 2 || NT == 4 || NT == 8, "16 NT rows are dealt to 256 threads, 16 per row");
+    constexpr int V = Elem<DT>::VEC;
+    constexpr int ROWS = 16 * NT;
+    constexpr int BV = ROWS / 16;                    // weight vectors per thread and chunk
+    const int tid = threadIdx.x, w = tid >> 6, l = lane_id();
+    const int m = l & 15, g = l >> 4;
+    const int nv = model_dim / V;                    // 16-byte vectors per row
+    const int chunks = (nv + 15) / 16;
+
+    RowStats<PLANMOE_BF16, true> st;
+    if constexpr (STATS) st.init();
+
+    const uint4 *ap = reinterpret_cast<const uint4 *>(x) + (int64_t)min(t0 + w * 16 + m, samples - 1) * nv;
+    const int bvec = tid & 15;                       // thread's vector inside the chunk
+    const uint4 *bp[BV];
+    int bdst[BV];
+#pragma unroll
+    for (int i = 0; i < BV; ++i) {
+        const int row = i * 16 + (tid >> 4);
+        bp[i] = reinterpret_cast<const uint4 *>(wg) + (int64_t)min(row, experts - 1) * nv + bvec;
+        bdst[i] = row * 16 + (bvec ^ (row & 15));
+    }
+
+    f32x4 acc[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // vectors past the row end read as zero in BOTH operands
+    auto load_a = [&](uint4 (&a)[4], int c) {
+        const int o = c * 16 + g;
+        if (c * 16 + 16 <= nv) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) a[s] = ap[o + 4 * s];
+        } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                a[s] = make_uint4(0, 0, 0, 0);
+                if (o + 4 * s < nv) a[s] = ap[o + 4 * s];
+            }
+        }
+    };
+    auto load_b = [&](uint4 (&b)[BV], int c) {
+        const int o = c * 16;
+        const bool in = o + bvec < nv;
+#pragma unroll
+        for (int i = 0; i < BV; ++i) {
+            b[i] = make_uint4(0, 0, 0, 0);
+            if (in) b[i] = bp[i][o];
+        }
+    };
+    auto store_b = [&](const uint4 (&b)[BV], int buf) {
+#pragma unroll
+        for (int i = 0; i < BV; ++i) smem[buf * ROWS * 16 + bdst[i]] = b[i];
+    };
+    auto compute = [&](const uint4 (&a)[4], int buf) {
+        const uint4 *bb = smem + buf * ROWS * 16 + m * 16;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            uint4 bf[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) bf[nt] = bb[nt * 256 + ((4 * s + g) ^ m)];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) Mma<DT>::run(a[s], bf[nt], acc[nt]);
+            if constexpr (STATS) st.add(a[s]);
+        }
+    };
+
+    uint4 a0[4], a1[4], bs[BV];
+    load_a(a0, 0);
+    load_b(bs, 0);
+    store_b(bs, 0);
+    __syncthreads();
+    for (int c = 0; c < chunks; c += 2) {
+        const bool more1 = c + 1 < chunks;
+        if (more1) { load_a(a1, c + 1); load_b(bs, c + 1); }
+        compute(a0, 0);
+        if (more1) store_b(bs, 1);
+        __syncthreads();
+        if (!more1) break;
+        const bool more2 = c + 2 < chunks;
+        if (more2) { load_a(a0, c + 2); load_b(bs, c + 2); }
+        compute(a1, 1);
+        if (more2) store_b(bs, 0);
+        __syncthreads();
+    }
+
+    if constexpr (STATS) {
+        int a, b, n;
+        st.reduced(a, b, n);
+#pragma unroll
+        for (int off = 16; off < 64; off <<= 1) {
+            a = min(a, __shfl_xor(a, off, WAVE));
+            b = max(b, __shfl_xor(b, off, WAVE));
+            n = max(n, __shfl_xor(n, off, WAVE));
+        }
+        if (g == 0) { pstat[w * 16 + m][0] = a; pstat[w * 16 + m][1] = b; pstat[w * 16 + m][2] = n; }
+    }
+
+    // every wave is past its last read of the weight buffers (barrier above): reuse them
+    float (*logits)[ROWS + 1] = reinterpret_cast<float (*)[ROWS + 1]>(smem);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) logits[w * 16 + 4 * g + i][nt * 16 + m] = acc[nt][i];
 }
 
 } // namespace pm

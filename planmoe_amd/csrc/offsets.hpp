@@ -49,8 +49,16 @@ static __global__ __launch_bounds__(256) void group_offsets_kernel(
         const int j = j0 + jc;
         const bool live = jc < planes_per_chunk && j < k && el < ne;
         int32_t sum = 0;
+        int32_t keep[GO_BATCH];                          // first batch stays in registers for pass 2
+#pragma unroll
+        for (int i = 0; i < GO_BATCH; ++i) keep[i] = 0;
         if (live) {
-            for (int g = g0; g < g1; g += GO_BATCH) {
+#pragma unroll
+            for (int i = 0; i < GO_BATCH; ++i)
+                if (g0 + i < g1) keep[i] = hist[((int64_t)(g0 + i) * k + j) * experts + e];
+#pragma unroll
+            for (int i = 0; i < GO_BATCH; ++i) sum += keep[i];
+            for (int g = g0 + GO_BATCH; g < g1; g += GO_BATCH) {
                 int32_t v[GO_BATCH];
 #pragma unroll
                 for (int i = 0; i < GO_BATCH; ++i)
@@ -75,7 +83,12 @@ static __global__ __launch_bounds__(256) void group_offsets_kernel(
         for (int p = 0; p < jc; ++p) base += s_tot[p * experts_per_block + el];
         if (live) {
             int32_t run = base + before;
-            for (int g = g0; g < g1; g += GO_BATCH) {
+#pragma unroll
+            for (int i = 0; i < GO_BATCH; ++i) {
+                if (g0 + i < g1) offs[((int64_t)(g0 + i) * k + j) * experts + e] = run;
+                run += keep[i];
+            }
+            for (int g = g0 + GO_BATCH; g < g1; g += GO_BATCH) {
                 int32_t v[GO_BATCH];
 #pragma unroll
                 for (int i = 0; i < GO_BATCH; ++i)

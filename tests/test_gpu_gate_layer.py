@@ -13,7 +13,9 @@ DEV = "cuda:0"
 
 @pytest.mark.parametrize("T,M,E,dtype", [(100, 512, 8, torch.bfloat16), (1000, 4096, 8, torch.bfloat16), (777, 2048, 64, torch.bfloat16),
                                          (100, 2048, 2, torch.float32), (50, 100, 5, torch.float32), (50, 1000, 20, torch.float32),
-                                         (31, 136, 17, torch.bfloat16), (16, 4100, 8, torch.bfloat16), (10, 64, 100, torch.float32)])
+                                         (31, 136, 17, torch.bfloat16), (16, 4100, 8, torch.bfloat16), (10, 64, 100, torch.float32),
+                                         (300, 2056, 32, torch.bfloat16), (129, 520, 128, torch.bfloat16), (65, 36, 24, torch.float32),
+                                         (200, 264, 130, torch.bfloat16)])
 def test_gate_logits(T, M, E, dtype):
     """fp32-accumulated logits against the oracle's fp64 dot products: rtol 1e-5 of the row scale
     (products of bf16 values are exact in fp32, only the summation order differs)."""
@@ -156,7 +158,8 @@ def test_moe_layer_trains_with_builtin_ffn():
     (1000, 512, 8, 2, 1.25, torch.bfloat16, True, False), (33, 256, 4, 2, 1.0, torch.bfloat16, True, False),
     (4096, 1024, 64, 1, 1.0, torch.bfloat16, True, True), (500, 2048, 2, 2, 1.0, torch.float32, True, False),
     (700, 264, 16, 3, 0.5, torch.bfloat16, False, False), (257, 128, 33, 4, 1.0, torch.float16, True, False),
-    (31, 64, 5, 5, 2.0, torch.float32, False, True)])
+    (31, 64, 5, 5, 2.0, torch.float32, False, True), (1500, 776, 48, 2, 1.25, torch.bfloat16, True, True),
+    (900, 260, 24, 20, 1.0, torch.float32, True, False), (640, 512, 64, 17, 1.0, torch.bfloat16, False, False)])
 def test_fused_forward_matches_unfused_and_oracle(T, M, E, k, cf, dtype, fp32_gate, use_bias):
     """planmoe_forward_int8 / planmoe_gate_route against the stage-by-stage entry points and the
     oracle (routing evaluated on the scores the kernel reports)."""
