@@ -10,7 +10,9 @@
 namespace pm {
 
 // CACHE = 16-byte vectors per lane held in registers (0: re-read the row from cache)
-template <int DT, int CACHE>
+// GATED: rows are scaled by their gate first (one code row per choice); GRAD: the gate gradient
+// <x[t], other[slot]> rides along (GATED only)
+template <int DT, int CACHE, bool GATED, bool GRAD>
 __global__ __launch_bounds__(256) void dispatch_int8_kernel(
     const void *__restrict__ x, const float *__restrict__ gates,
     const int32_t *__restrict__ indices, const int32_t *__restrict__ locations, int64_t stride,
@@ -116,10 +118,10 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
         const int np = min(top_k - j0, WAVE);
         int slot; float gate;
         fetch_planes(gates, indices, locations, stride, t, j0, np, experts, capacity, slot, gate);
-        if (grad_gates && lane < np && slot < 0) grad_gates[(int64_t)(j0 + lane) * stride + t] = 0.f;
+        if (GRAD && lane < np && slot < 0) grad_gates[(int64_t)(j0 + lane) * stride + t] = 0.f;
         if (__ballot(slot >= 0) == 0) continue;
 
-        if (!gates) {
+        if constexpr (!GATED) {
             // one code row shared by all live choices; 0 + 1 * x needs no rounding
             RowStats<DT, true> stats;
             stats.init();
@@ -149,16 +151,33 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
                 for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
             }
         } else {
+            // min / max of the unscaled row once: rounding and scaling by a finite non-zero gate
+            // are monotonic, so the extremes of round(0 + g * x) are the images of the extremes
+            RowStats<DT, true> stats;
+            stats.init();
+            if constexpr (CACHE > 0) {
+#pragma unroll
+                for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) stats.add(cache[c]);
+            } else {
+                for (int u = lane; u < units; u += WAVE) stats.add(src[u]);
+            }
+            float xmn, xmx;
+            stats.finish(xmn, xmx);
             for (int j = 0; j < np; ++j) {
                 const int s = rl_i(slot, j);
                 if (s < 0) continue;
                 const float g = rl_f(gate, j);
-                if (grad_gates) {
+                if constexpr (GRAD) {
                     const float gg = dot_with(s);
                     if (lane == 0) grad_gates[(int64_t)(j0 + j) * stride + t] = gg;
                 }
                 float mn, mx;
-                reduce(g, mn, mx);
+                if (g != 0.f && fabsf(g) < INFINITY && xmn == xmn) {
+                    mn = E::round(0.f + g * (g > 0.f ? xmn : xmx));
+                    mx = E::round(0.f + g * (g > 0.f ? xmx : xmn));
+                } else {
+                    reduce(g, mn, mx);           // 0 * inf, NaN rows and the like: element by element
+                }
                 const float scale = E::round(mx - mn);
                 if (lane == 0) { E::store(bias_out, s, mn); E::store(scale_out, s, scale); }
                 const RowQuant<DT> rq(mn, scale);
@@ -186,16 +205,23 @@ static void launch_dispatch_int8(int per_lane, unsigned grid, hipStream_t st, co
                                  const uint32_t *flags, int token_blocks, const void *other,
                                  float *grad_gates)
 {
-#define PM_DI8(CACHE)                                                                            \
-    dispatch_int8_kernel<DT, CACHE><<<grid, 256, 0, st>>>(x, gates, indices, locations, stride,  \
+#define PM_DI8_(CACHE, GATED, GRAD)                                                              \
+    dispatch_int8_kernel<DT, CACHE, GATED, GRAD><<<grid, 256, 0, st>>>(x, gates, indices, locations, stride, \
         top_k, samples, model_dim, experts, capacity, codes, bias, scale, flags, token_blocks,   \
         other, grad_gates)
+#define PM_DI8(CACHE)                                                                            \
+    do {                                                                                         \
+        if (!gates) PM_DI8_(CACHE, false, false);                                                \
+        else if (!grad_gates) PM_DI8_(CACHE, true, false);                                       \
+        else PM_DI8_(CACHE, true, true);                                                         \
+    } while (0)
     if (per_lane <= 2) PM_DI8(2);
     else if (per_lane <= 4) PM_DI8(4);
     else if (per_lane <= 8) PM_DI8(8);
     else if (per_lane <= 16) PM_DI8(16);
     else PM_DI8(0);
 #undef PM_DI8
+#undef PM_DI8_
 }
 
 } // namespace pm

@@ -80,12 +80,45 @@ __global__ __launch_bounds__(TILE) void route_tile_kernel(
     row.experts = experts; row.logits = input_is_logits != 0;
 
     float s[CAP > 0 ? CAP : 1];
-    if (valid) {
-        row.prepare();
-        if constexpr (CAP > 0) {
+    if constexpr (CAP > 0) {
+        // the tile's rows come in with coalesced loads, half a tile at a time, and every thread
+        // picks its row out of LDS (row length + 1 keeps the banks apart)
+        float *stage = reinterpret_cast<float *>(wave_cnt + 4 * experts);       // [TILE / 2][experts + 1]
+        const int64_t tile_base = (int64_t)blockIdx.x * TILE * experts;
 #pragma unroll
-            for (int e = 0; e < CAP; ++e) s[e] = (e < experts) ? row.score(e) : -INFINITY;
+        for (int half = 0; half < 2; ++half) {
+            const int r0 = half * (TILE / 2);
+            const int nrows = max(0, min(TILE / 2, samples - (int)blockIdx.x * TILE - r0));
+            for (int i = tid; i < nrows * experts; i += TILE) {
+                const int r = i / experts, e = i - r * experts;
+                stage[r * (experts + 1) + e] = E::load(input, tile_base + (int64_t)r0 * experts + i);
+            }
+            __syncthreads();
+            if (valid && tid / (TILE / 2) == half) {
+#pragma unroll
+                for (int e = 0; e < CAP; ++e)
+                    s[e] = (e < experts) ? stage[(tid - r0) * (experts + 1) + e] : -INFINITY;
+            }
+            __syncthreads();
         }
+        if (valid && row.logits) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < CAP; ++e) {
+                if (e < experts) {
+                    if (logit_bias) s[e] = E::round(s[e] + logit_bias[e]);
+                    mx = fmaxf(mx, s[e]);
+                }
+            }
+            float sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < CAP; ++e) if (e < experts) { s[e] = expf(s[e] - mx); sum += s[e]; }
+#pragma unroll
+            for (int e = 0; e < CAP; ++e) if (e < experts) s[e] = E::round(s[e] / sum);
+        }
+    }
+    if (valid) {
+        if constexpr (CAP == 0) row.prepare();
         if (scores_out) {
             if constexpr (CAP > 0) {
 #pragma unroll
@@ -417,7 +450,8 @@ extern "C" int planmoe_route_topk(const void *input, int dtype, int input_is_log
     int32_t *offs = hist + (size_t)tiles * k * experts;
     float *me = (float *)(offs + (size_t)tiles * k * experts);
     float *loss_part = me + (size_t)tiles * experts;
-    const size_t lds = sizeof(int32_t) * 4 * (size_t)experts;
+    // 4 waves x experts counters, and for rows held in registers the staging area of half a tile
+    const size_t lds = 4 * (4 * (size_t)experts + (experts <= 64 ? (size_t)(TILE / 2) * (experts + 1) : 0));
 
     PM_DTYPE_SWITCH(dtype, DT,
         launch_route_tile<DT>(experts, dim3(tiles), lds, st, input, input_is_logits, logit_bias,
