@@ -244,8 +244,8 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
             if (s - e * capacity < totals[e]) continue;          // slot holds a token
             uint8_t *row = codes + (int64_t)s * model_dim;
             for (int u = lane; u < units; u += WAVE) {
-                if constexpr (V == 8) reinterpret_cast<uint2 *>(row)[u] = make_uint2(0u, 0u);
-                else reinterpret_cast<uint32_t *>(row)[u] = 0u;
+                if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(row) + u, make_uint2(0u, 0u));
+                else stream_store(reinterpret_cast<uint32_t *>(row) + u, 0u);
             }
             if (lane == 0) { E::store(bias_out, s, 0.f); E::store(scale_out, s, 0.f); }
         }
@@ -302,8 +302,8 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
             const int s = rl_i(slot, j);
             if (s < 0) continue;
             uint8_t *row = codes + (int64_t)s * model_dim;
-            if constexpr (V == 8) reinterpret_cast<uint2 *>(row)[u] = make_uint2(w[0], w[1]);
-            else reinterpret_cast<uint32_t *>(row)[u] = w[0];
+            if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(row) + u, make_uint2(w[0], w[1]));
+            else stream_store(reinterpret_cast<uint32_t *>(row) + u, w[0]);
         }
     };
     if constexpr (CACHE > 0) {

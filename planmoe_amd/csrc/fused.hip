@@ -34,8 +34,8 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
             if (flags[s]) continue;
             uint8_t *row = codes + (int64_t)s * model_dim;
             for (int u = lane; u < units; u += WAVE) {
-                if constexpr (V == 8) reinterpret_cast<uint2 *>(row)[u] = make_uint2(0u, 0u);
-                else reinterpret_cast<uint32_t *>(row)[u] = 0u;
+                if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(row) + u, make_uint2(0u, 0u));
+                else stream_store(reinterpret_cast<uint32_t *>(row) + u, 0u);
             }
             if (lane == 0) { E::store(bias_out, s, 0.f); E::store(scale_out, s, 0.f); }
         }
@@ -110,8 +110,8 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
     };
     auto put = [&](int s, int u, const uint32_t *w) {
         uint8_t *row = codes + (int64_t)s * model_dim;
-        if constexpr (V == 8) reinterpret_cast<uint2 *>(row)[u] = make_uint2(w[0], w[1]);
-        else reinterpret_cast<uint32_t *>(row)[u] = w[0];
+        if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(row) + u, make_uint2(w[0], w[1]));
+        else stream_store(reinterpret_cast<uint32_t *>(row) + u, w[0]);
     };
 
     for (int j0 = 0; j0 < top_k; j0 += WAVE) {

@@ -31,7 +31,7 @@ __global__ __launch_bounds__(256) void int8_compress_vec_kernel(
 #pragma unroll
         for (int c = 0; c < CACHE; ++c) {
             const int u = c * WAVE + lane;
-            if (u < units) cache[c] = src[u];
+            if (u < units) cache[c] = stream_load(src + u);
         }
 #pragma unroll
         for (int c = 0; c < CACHE; ++c)
@@ -49,8 +49,8 @@ __global__ __launch_bounds__(256) void int8_compress_vec_kernel(
     auto emit = [&](int u, const uint4 &raw) {
         uint32_t w[2];
         enc.encode(raw, w);
-        if constexpr (V == 8) reinterpret_cast<uint2 *>(dst)[u] = make_uint2(w[0], w[1]);
-        else reinterpret_cast<uint32_t *>(dst)[u] = w[0];
+        if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(dst) + u, make_uint2(w[0], w[1]));
+        else stream_store(reinterpret_cast<uint32_t *>(dst) + u, w[0]);
     };
     if constexpr (CACHE > 0) {
 #pragma unroll
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void int8_decompress_vec_kernel(
         float f[V];
 #pragma unroll
         for (int i = 0; i < V; ++i) f[i] = dq((w[i / 4] >> (8 * (i % 4))) & 0xffu);
-        dst[u] = E::pack(f);
+        stream_store(dst + u, E::pack(f));
     }
 }
 

@@ -13,14 +13,21 @@ struct RowIO {
         if constexpr (VECTOR) E::unpack(reinterpret_cast<const uint4 *>(row)[unit], f);
         else f[0] = E::load(row, unit);
     }
+    // for launches that store nothing in bulk (measured: streaming loads next to streaming
+    // stores slow the dispatch / combine kernels down, alone they help)
+    __device__ static __forceinline__ void load_stream(const void *row, int unit, float *f)
+    {
+        if constexpr (VECTOR) E::unpack(stream_load(reinterpret_cast<const uint4 *>(row) + unit), f);
+        else f[0] = E::load(row, unit);
+    }
     __device__ static __forceinline__ void store(void *row, int unit, const float *f)
     {
-        if constexpr (VECTOR) reinterpret_cast<uint4 *>(row)[unit] = E::pack(f);
+        if constexpr (VECTOR) stream_store(reinterpret_cast<uint4 *>(row) + unit, E::pack(f));
         else E::store(row, unit, f[0]);
     }
     __device__ static __forceinline__ void store_zero(void *row, int unit)
     {
-        if constexpr (VECTOR) reinterpret_cast<uint4 *>(row)[unit] = make_uint4(0, 0, 0, 0);
+        if constexpr (VECTOR) stream_store(reinterpret_cast<uint4 *>(row) + unit, make_uint4(0, 0, 0, 0));
         else E::store(row, unit, 0.f);
     }
 };

@@ -170,12 +170,12 @@ __global__ __launch_bounds__(256) void bwd_gate_kernel(
         float acc[G] = {0.f, 0.f, 0.f, 0.f};
         for (int u = lane; u < units; u += WAVE) {
             float a[IO::U];
-            IO::load(xr, u, a);
+            IO::load_stream(xr, u, a);
 #pragma unroll
             for (int j = 0; j < G; ++j) {
                 if (s[j] < 0) continue;
                 float d[IO::U];
-                IO::load((const char *)dispatched + (int64_t)s[j] * row_bytes, u, d);
+                IO::load_stream((const char *)dispatched + (int64_t)s[j] * row_bytes, u, d);
 #pragma unroll
                 for (int i = 0; i < IO::U; ++i) acc[j] = fmaf(d[i], a[i], acc[j]);
             }
