@@ -45,6 +45,18 @@ static __global__ __launch_bounds__(256) void group_offsets_kernel(
     const int g0 = min(rl * per, groups), g1 = min(g0 + per, groups);
     if (threadIdx.x < GO_COLS) s_base[threadIdx.x] = 0;
 
+    // column sums of the scores first: their loads overlap those of the histograms
+    float mes = 0.f;
+    if (want_loss && jc == 0 && el < ne) {
+        for (int g = g0; g < g1; g += GO_BATCH) {
+            float v[GO_BATCH];
+#pragma unroll
+            for (int i = 0; i < GO_BATCH; ++i) v[i] = (g + i < g1) ? me[(int64_t)(g + i) * experts + e] : 0.f;
+#pragma unroll
+            for (int i = 0; i < GO_BATCH; ++i) mes += v[i];
+        }
+    }
+
     for (int j0 = 0; j0 < k; j0 += planes_per_chunk) {
         const int j = j0 + jc;
         const bool live = jc < planes_per_chunk && j < k && el < ne;
@@ -115,16 +127,6 @@ static __global__ __launch_bounds__(256) void group_offsets_kernel(
     if (totals && threadIdx.x < ne) totals[e0 + threadIdx.x] = s_base[threadIdx.x];
 
     if (want_loss) {
-        float mes = 0.f;
-        if (jc == 0 && el < ne) {
-            for (int g = g0; g < g1; g += GO_BATCH) {
-                float v[GO_BATCH];
-#pragma unroll
-                for (int i = 0; i < GO_BATCH; ++i) v[i] = (g + i < g1) ? me[(int64_t)(g + i) * experts + e] : 0.f;
-#pragma unroll
-                for (int i = 0; i < GO_BATCH; ++i) mes += v[i];
-            }
-        }
         s_me[rl][cl] = mes;
         __syncthreads();
         if (threadIdx.x < WAVE) {

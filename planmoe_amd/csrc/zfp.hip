@@ -11,32 +11,34 @@
 
 namespace pm {
 
+// The words of a block's bit stream are parked in LDS while the block is coded (word i of thread
+// t at lds[i * 256 + t]): a register array would need a select per word on every flush, since
+// the word index differs from lane to lane.
 template <int NW>
 struct BitWriter {
-    uint32_t w[NW];
+    uint32_t *slot;
     uint64_t acc;
-    int fill, wi;
-    __device__ __forceinline__ void init()
+    int fill;
+    __device__ __forceinline__ void init(uint32_t *lds)
     {
+        slot = lds + threadIdx.x;
 #pragma unroll
-        for (int i = 0; i < NW; ++i) w[i] = 0u;
-        acc = 0; fill = 0; wi = 0;
-    }
-    __device__ __forceinline__ void flush_word()
-    {
-        const uint32_t x = (uint32_t)acc;
-#pragma unroll
-        for (int i = 0; i < NW; ++i) if (i == wi) w[i] = x;
-        ++wi; acc >>= 32; fill -= 32;
+        for (int i = 0; i < NW; ++i) slot[i * 256] = 0u;
+        acc = 0; fill = 0;
     }
     // append the low n (<= 32) bits of v; bits of v above n must be zero
     __device__ __forceinline__ void put(uint32_t v, int n)
     {
         acc |= (uint64_t)v << fill;
         fill += n;
-        if (fill >= 32) flush_word();
+        if (fill >= 32) { *slot = (uint32_t)acc; slot += 256; acc >>= 32; fill -= 32; }
     }
-    __device__ __forceinline__ void finish() { if (fill > 0) flush_word(); }
+    __device__ __forceinline__ void finish() { if (fill > 0) *slot = (uint32_t)acc; }
+    __device__ __forceinline__ void words(uint32_t *lds, uint32_t *w) const
+    {
+#pragma unroll
+        for (int i = 0; i < NW; ++i) w[i] = lds[i * 256 + threadIdx.x];
+    }
 };
 
 template <int NW>
@@ -90,6 +92,29 @@ __device__ __forceinline__ void inv_lift(int32_t &x, int32_t &y, int32_t &z, int
 __device__ __forceinline__ uint32_t to_negabinary(int32_t v) { return ((uint32_t)v + 0xaaaaaaaau) ^ 0xaaaaaaaau; }
 __device__ __forceinline__ int32_t from_negabinary(uint32_t v) { return (int32_t)((v ^ 0xaaaaaaaau) - 0xaaaaaaaau); }
 
+// 16 x 16 bit matrix transpose.  w[j] holds row 2j in its low and row 2j+1 in its high half;
+// afterwards bit i of row k is what bit k of row i was.  Used to turn the upper halves of the 16
+// coefficients of a 2-D block into their 16 upper bit planes (and back) in about 100
+// instructions instead of 32 per plane.
+__device__ __forceinline__ void transpose16(uint32_t (&w)[8])
+{
+    auto swap_blocks = [](uint32_t &a, uint32_t &b, int s, uint32_t m) {
+        const uint32_t t = ((a >> s) ^ b) & m;
+        b ^= t; a ^= t << s;
+    };
+#pragma unroll
+    for (int j = 0; j < 4; ++j) swap_blocks(w[j], w[j + 4], 8, 0x00ff00ffu);
+    swap_blocks(w[0], w[2], 4, 0x0f0f0f0fu); swap_blocks(w[1], w[3], 4, 0x0f0f0f0fu);
+    swap_blocks(w[4], w[6], 4, 0x0f0f0f0fu); swap_blocks(w[5], w[7], 4, 0x0f0f0f0fu);
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) swap_blocks(w[j], w[j + 1], 2, 0x33333333u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t t = ((w[j] >> 15) ^ w[j]) & 0x0000aaaau;
+        w[j] ^= t | (t << 15);
+    }
+}
+
 // sequency order of the 4x4 coefficients (index into the i + 4j block layout)
 __device__ constexpr int perm2(int i)
 {
@@ -97,11 +122,40 @@ __device__ constexpr int perm2(int i)
     return P[i];
 }
 
+// Group-test code of one bit plane without a data-dependent loop.
+// For the not yet significant part r of a plane (bit p = value nsig + p) zfp emits, segment by
+// segment, a test bit '1', the zeros below the next one bit and that one bit; i.e. the bits of r
+// up to its highest one with a '1' put in front of bit 0 and of every bit that follows a one.
+// The table holds that expansion for 8 bits of r at a time: entry [prev][byte] = code in the low
+// 16 bits, its length (8 + prev + ones among the low 7 bits) above.  What follows the highest
+// one (a single '0' test bit, or nothing at the block end) and the implicit last one are a
+// matter of the total length, see encode_block.
+__device__ inline uint32_t group_code_entry(int prev, int byte)
+{
+    uint32_t code = 0; int len = 0;
+    for (int p = 0; p < 8; ++p) {
+        const int bit = (byte >> p) & 1;
+        if (prev) { code |= 1u << len; ++len; }
+        code |= (uint32_t)bit << len; ++len;
+        prev = bit;
+    }
+    return code | ((uint32_t)len << 16);
+}
+// all 256 threads of the work-group; tab has 512 entries
+__device__ __forceinline__ void group_code_table(uint32_t *tab)
+{
+    tab[threadIdx.x] = group_code_entry(0, threadIdx.x);
+    tab[256 + threadIdx.x] = group_code_entry(1, threadIdx.x);
+    __syncthreads();
+}
+__device__ __forceinline__ uint32_t low_bits(int n) { return (uint32_t)(((uint64_t)1 << n) - 1u); }   // n in 0..32
+
 // N = values per block (4 or 16).  f is consumed; the block's maxbits = 32*NW bits land in bw.
 template <int N, int NW>
-__device__ __forceinline__ void encode_block(const float *f, BitWriter<NW> &bw)
+__device__ __forceinline__ void encode_block(const float *f, BitWriter<NW> &bw, uint32_t *lds,
+                                             const uint32_t *tab)
 {
-    bw.init();
+    bw.init(lds);
     float m = 0.f;
 #pragma unroll
     for (int i = 0; i < N; ++i) m = fmaxf(m, fabsf(f[i]));
@@ -118,7 +172,8 @@ __device__ __forceinline__ void encode_block(const float *f, BitWriter<NW> &bw)
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         const float v = f[i] * s;
-        q[i] = (v >= 2147483648.0f || v < -2147483648.0f || v != v) ? (int32_t)0x80000000 : (int32_t)v;
+        // -2^31 itself converts to INT_MIN either way
+        q[i] = fabsf(v) < 2147483648.0f ? (int32_t)v : (int32_t)0x80000000;
     }
     uint32_t u[N];
     if constexpr (N == 4) {
@@ -137,28 +192,53 @@ __device__ __forceinline__ void encode_block(const float *f, BitWriter<NW> &bw)
     // embedded coding: bit planes from the top, group-tested, until the budget is spent
     int bits = 32 * NW - 9;
     int nsig = 0;
-    for (int k = 31; k >= 0 && bits > 0; --k) {
-        uint32_t x = 0;
-#pragma unroll
-        for (int i = 0; i < N; ++i) x |= ((u[i] >> k) & 1u) << i;
+    auto code_plane = [&](uint32_t x) __attribute__((always_inline)) {
         const int mm = min(nsig, bits);
         bits -= mm;
         bw.put(x & ((1u << mm) - 1u), mm);
-        x >>= mm;
-        while (nsig < N && bits > 0) {
-            --bits;
-            bw.put(x != 0u ? 1u : 0u, 1);
-            if (x == 0u) break;
-            // zeros up to the next one bit, then the one (implicit when it is the last value)
-            const int z = __builtin_ctz(x);
-            const int r = N - 1 - nsig;
-            const int cnt = min(z + 1, r);
-            const int emit = min(cnt, bits);
-            const uint32_t pat = (z < r ? (1u << z) : 0u) & ((1u << emit) - 1u);
-            bw.put(pat, emit);
+        if (nsig < N && bits > 0) {
+            const uint32_t r = x >> mm;                   // mm == nsig here
+            // r == 0 runs through the same formulas: top = -1, no code bits, length 1 (the '0')
+            const int top = 31 - __clz((int)r), ones = __builtin_popcount(r);
+            const uint32_t e0 = tab[256 + (r & 0xffu)];
+            uint32_t code = e0 & 0xffffu;
+            if constexpr (N > 8) {
+                const uint32_t e1 = tab[((r >> 7) & 1u) * 256 + (r >> 8)];
+                code |= (e1 & 0xffffu) << (e0 >> 16);
+            }
+            // cut after the highest one bit (not emitted when it is the block's last value),
+            // then one more '0' test bit unless the block ends there
+            const int last = nsig + top == N - 1;
+            const int lt = top + 1 + ones - last;
+            const int len = lt + (nsig + top + 1 < N ? 1 : 0);
+            const int emit = min(len, bits);
+            code &= low_bits(min(lt, emit));
+            bw.put(code, emit);
             bits -= emit;
-            x >>= z; x >>= 1;
-            nsig += z + 1;
+            nsig += top + 1;
+        }
+    };
+    if constexpr (N == 16) {
+        // planes 31..16 by one bit transpose of the coefficients' upper halves
+        uint32_t w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = (u[2 * j] >> 16) | (u[2 * j + 1] & 0xffff0000u);
+        transpose16(w);
+#pragma unroll
+        for (int k = 15; k >= 0; --k)
+            if (bits > 0) code_plane((k & 1) ? w[k >> 1] >> 16 : w[k >> 1] & 0xffffu);
+        for (int k = 15; k >= 0 && bits > 0; --k) {
+            uint32_t x = 0;
+#pragma unroll
+            for (int i = 0; i < N; ++i) x |= ((u[i] >> k) & 1u) << i;
+            code_plane(x);
+        }
+    } else {
+        for (int k = 31; k >= 0 && bits > 0; --k) {
+            uint32_t x = 0;
+#pragma unroll
+            for (int i = 0; i < N; ++i) x |= ((u[i] >> k) & 1u) << i;
+            code_plane(x);
         }
     }
     bw.finish();
@@ -179,7 +259,7 @@ __device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f)
     for (int i = 0; i < N; ++i) u[i] = 0u;
     int bits = 32 * NW - 9;
     int nsig = 0;
-    for (int k = 31; k >= 0 && bits > 0; --k) {
+    auto read_plane = [&]() __attribute__((always_inline)) {
         const int mm = min(nsig, bits);
         bits -= mm;
         uint32_t x = br.get(mm);
@@ -197,8 +277,30 @@ __device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f)
             x |= 1u << nsig;
             ++nsig;
         }
+        return x;
+    };
+    if constexpr (N == 16) {
+        // planes 31..16 are collected as rows and transposed into the coefficients' upper halves
+        uint32_t w[8];
 #pragma unroll
-        for (int i = 0; i < N; ++i) u[i] |= ((x >> i) & 1u) << k;
+        for (int j = 0; j < 8; ++j) w[j] = 0u;
+#pragma unroll
+        for (int k = 15; k >= 0; --k)
+            if (bits > 0) w[k >> 1] |= read_plane() << (16 * (k & 1));
+        transpose16(w);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { u[2 * j] = w[j] << 16; u[2 * j + 1] = w[j] & 0xffff0000u; }
+        for (int k = 15; k >= 0 && bits > 0; --k) {
+            const uint32_t x = read_plane();
+#pragma unroll
+            for (int i = 0; i < N; ++i) u[i] |= ((x >> i) & 1u) << k;
+        }
+    } else {
+        for (int k = 31; k >= 0 && bits > 0; --k) {
+            const uint32_t x = read_plane();
+#pragma unroll
+            for (int i = 0; i < N; ++i) u[i] |= ((x >> i) & 1u) << k;
+        }
     }
     int32_t q[N];
     if constexpr (N == 4) {
@@ -248,13 +350,18 @@ template <int NW>
 __global__ __launch_bounds__(256) void zfp_encode1_kernel(const float *__restrict__ field, int64_t blocks,
                                                           uint32_t *__restrict__ out)
 {
+    __shared__ uint32_t lds[NW * 256];
+    __shared__ uint32_t tab[512];
+    group_code_table(tab);
     const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (b >= blocks) return;
     const float4 v = reinterpret_cast<const float4 *>(field)[b];
     const float f[4] = {v.x, v.y, v.z, v.w};
     BitWriter<NW> bw;
-    encode_block<4, NW>(f, bw);
-    store_words<NW>(out + b * NW, bw.w);
+    encode_block<4, NW>(f, bw, lds, tab);
+    uint32_t w[NW];
+    bw.words(lds, w);
+    store_words<NW>(out + b * NW, w);
     // an odd count of 32-bit words leaves half of the last 64-bit stream word as padding
     if (b == blocks - 1 && ((blocks * NW) & 1)) out[blocks * NW] = 0u;
 }
@@ -277,6 +384,9 @@ __global__ __launch_bounds__(256) void zfp_encode2_kernel(const float *__restric
                                                           int64_t nbx, int64_t blocks,
                                                           uint32_t *__restrict__ out)
 {
+    __shared__ uint32_t lds[NW * 256];
+    __shared__ uint32_t tab[512];
+    group_code_table(tab);
     const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (b >= blocks) return;
     const int64_t by = b / nbx, bx = b - by * nbx;
@@ -288,8 +398,10 @@ __global__ __launch_bounds__(256) void zfp_encode2_kernel(const float *__restric
         f[4 * j] = v.x; f[4 * j + 1] = v.y; f[4 * j + 2] = v.z; f[4 * j + 3] = v.w;
     }
     BitWriter<NW> bw;
-    encode_block<16, NW>(f, bw);
-    store_words<NW>(out + b * NW, bw.w);
+    encode_block<16, NW>(f, bw, lds, tab);
+    uint32_t w[NW];
+    bw.words(lds, w);
+    store_words<NW>(out + b * NW, w);
 }
 
 template <int NW>
