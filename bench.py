@@ -61,6 +61,101 @@ def cpu_baseline(T_sample, M, E, k, cf, x_bits, wg_bits, min_seconds):
     return T_sample * reps / dt, dt, reps
 
 
+def kernel_table():
+    """Every entry point at the full size of its workload (BASELINE configs 1-5): device time over
+    back-to-back launches (HIP events) against the algorithmic bytes = inputs read once + outputs
+    written once.  One line per entry point; an entry point may be several launches."""
+    import torch
+    from planmoe_amd import ops
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(0)
+    rows = []
+
+    def add(name, cfg, nbytes, fn, iters=20):
+        # the calls are recorded into a HIP graph once and the graph is replayed: the Python
+        # wrappers (output allocation + ctypes call) are slower than the short kernels
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(iters):
+                fn()
+        avg, med, best = event_time_us(graph.replay, 1, 1, rounds=5)
+        rows.append((name, cfg, nbytes, avg / iters, best / iters))
+        del graph
+
+    # configs 2 / 4: 16384 tokens x 4096, 8 experts, top-2, capacity_factor 1.25, bf16
+    T, M, E, k = 16384, 4096, 8, 2
+    C = ops.capacity(T, E, k, 1.25, 4); R = E * C
+    x = torch.randn(T, M, generator=g).bfloat16().to(dev)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(dev)
+    r = ops.gate_route(x, wg, k)
+    idx, loc, gates = list(r["indices"]), list(r["locations"]), list(r["gates"])
+    live = int(sum(((l >= 0) & (l < C)).sum() for l in loc))                 # token rows that reach a slot
+    xb, db, plane = T * M * 2, R * M * 2, T * k * 12
+    add("gate_logits", "2", xb + E * M * 2 + T * E * 4, lambda: ops.gate_logits(x, wg, torch.float32))
+    add("gate_route (gate + routing)", "2", xb + E * M * 2 + plane, lambda: ops.gate_route(x, wg, k))
+    sc = torch.softmax(ops.gate_logits(x, wg, torch.float32), 1)
+    add("route_topk (scores in)", "2", T * E * 4 + plane, lambda: ops.route_topk(sc, k))
+    add("dispatch_fwd", "2", xb + db + plane, lambda: ops.dispatch_fwd(x, idx, loc, None, E, C))
+    d = ops.dispatch_fwd(x, idx, loc, None, E, C)
+    add("combine_fwd", "2", live * M * 2 + xb + plane, lambda: ops.combine_fwd(d, idx, loc, gates, T, C))
+    add("bwd_gate", "2", live * M * 2 + xb + plane, lambda: ops.bwd_gate(x, d, idx, loc, C))
+    add("int8_compress", "2", db + R * M + R * 4, lambda: ops.int8_compress(d))
+    codes, b, s_ = ops.int8_compress(d)
+    add("int8_decompress", "2", db + R * M + R * 4, lambda: ops.int8_decompress(codes, b, s_))
+    add("dispatch_int8 (fused)", "2", xb + R * M + R * 4 + plane, lambda: ops.dispatch_int8(x, idx, loc, None, E, C))
+    add("combine_bwd_int8 (fused)", "4", xb + live * M * 2 + R * M + R * 4 + plane + T * k * 4,
+        lambda: ops.combine_bwd_int8(x, d, idx, loc, gates, E, C))
+    plan = ops.ForwardInt8Plan(x, wg, k, C, fp32_gate=True)
+    add("forward_int8 (chain)", "2", xb + E * M * 2 + R * M + R * 4 + plane, plan.run)
+    del d, codes, plan
+
+    # config 1: 8192 x 2048 fp32, 2 experts, top-2
+    T1, M1, E1 = 8192, 2048, 2
+    x1 = torch.randn(T1, M1, generator=g).to(dev)
+    w1 = (torch.randn(E1, M1, generator=g) * M1 ** -0.5).to(dev)
+    C1 = ops.capacity(T1, E1, 2, 1.0, 4)
+    r1 = ops.gate_route(x1, w1, 2)
+    i1, l1, g1 = list(r1["indices"]), list(r1["locations"]), list(r1["gates"])
+    add("gate_route (gate + routing)", "1", T1 * M1 * 4 + T1 * 24, lambda: ops.gate_route(x1, w1, 2))
+    add("dispatch_fwd", "1", T1 * M1 * 4 + E1 * C1 * M1 * 4, lambda: ops.dispatch_fwd(x1, i1, l1, None, E1, C1))
+    d1 = ops.dispatch_fwd(x1, i1, l1, None, E1, C1)
+    add("combine_fwd", "1", 3 * T1 * M1 * 4, lambda: ops.combine_fwd(d1, i1, l1, g1, T1, C1))
+    del d1
+
+    # config 3: 32768 x 2048 bf16, 64 experts, top-1, skewed logits
+    T3, M3, E3 = 32768, 2048, 64
+    x3 = torch.randn(T3, M3, generator=g).bfloat16().to(dev)
+    w3 = (torch.randn(E3, M3, generator=g) * M3 ** -0.5).bfloat16().to(dev)
+    pz = torch.arange(1, E3 + 1, dtype=torch.float64) ** -1.2
+    bias = torch.log(pz / pz.sum()).float().to(dev)
+    C3 = ops.capacity(T3, E3, 1, 1.0, 4)
+    add("gate_logits", "3", T3 * M3 * 2 + T3 * E3 * 4, lambda: ops.gate_logits(x3, w3, torch.float32))
+    add("gate_route (gate + routing)", "3", T3 * M3 * 2 + T3 * 12, lambda: ops.gate_route(x3, w3, 1, logit_bias=bias))
+    add("forward_int8 (chain)", "3", T3 * M3 * 2 + E3 * C3 * M3 + T3 * 12,
+        lambda: ops.forward_int8(x3, w3, 1, C3, logit_bias=bias))
+    lg = ops.gate_logits(x3, w3, torch.float32)
+    add("route_topk (logits in)", "3", T3 * E3 * 4 + T3 * 12, lambda: ops.route_topk(lg, 1, is_logits=True, logit_bias=bias))
+    mask = (torch.rand(T3, E3, device=dev) < 0.1).to(torch.int32)
+    add("cumsum_sub_one", "3", 2 * T3 * E3 * 4, lambda: ops.cumsum_sub_one(mask))
+
+    # config 5: zfp rate 8 on a [16, 8192, 1024] fp32 buffer
+    f = torch.randn(16 * 8192, 1024, generator=g).to(dev)
+    nx, ny = 1024, 16 * 8192
+    zb = f.numel() * 4 + f.numel()
+    for dims in (2, 1):
+        add("zfp_compress %d-D" % dims, "5", zb, lambda: ops.zfp_compress(f, nx, ny, dims), iters=5)
+        st = ops.zfp_compress(f, nx, ny, dims)
+        add("zfp_decompress %d-D" % dims, "5", zb, lambda: ops.zfp_decompress(st, nx, ny, dims), iters=5)
+
+    print("%-30s %-4s %10s %9s %9s %8s %6s" % ("entry point", "cfg", "alg MB", "avg us", "best us", "GB/s", "frac"))
+    for name, cfg, nbytes, avg, best in rows:
+        gbs = nbytes / avg / 1e3
+        print("%-30s %-4s %10.1f %9.1f %9.1f %8.0f %6.2f" % (name, cfg, nbytes / 1e6, avg, best, gbs, gbs / HBM_PEAK_GBS))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -71,10 +166,16 @@ def main():
     ap.add_argument("--copy-reference", action="store_true",
                     help="also run a plain 256 MiB device copy a few times (a kernel of known traffic, "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings against)")
+    ap.add_argument("--kernels", action="store_true",
+                    help="instead of the JSON line, print a table of every entry point at full size "
+                         "(device time, algorithmic bytes, fraction of the HBM peak)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
                  "(nothing here uses a second GPU)" % args.gpus)
+    if args.kernels:
+        kernel_table()
+        return
 
     import numpy as np
     import torch

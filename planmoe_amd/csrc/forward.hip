@@ -262,7 +262,9 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
 #pragma unroll
         for (int c = 0; c < CACHE; ++c) {
             const int u = c * WAVE + lane;
-            if (u < units) cache[c] = src[u];
+            // (index clamped, not predicated: straight-line loads let the compiler wait for exactly these
+            // loads; the re-read last vector is harmless for min / max and is never stored)
+            cache[c] = src[min(u, units - 1)];
         }
     }
 
@@ -285,7 +287,7 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
         stats.init();
         if constexpr (CACHE > 0) {
 #pragma unroll
-            for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) stats.add(cache[c]);
+            for (int c = 0; c < CACHE; ++c) stats.add(cache[c]);
         } else {
             for (int u = lane; u < units; u += WAVE) stats.add(src[u]);
         }
@@ -295,23 +297,26 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     if (slot >= 0) { E::store(bias_out, slot, mn); E::store(scale_out, slot, scale); }
     const RowEncoder<DT> enc(mn, scale);
 
-    auto emit = [&](int u, const uint4 &raw) {
-        uint32_t w[2];
-        enc.encode(raw, w);
-        for (int j = 0; j < top_k; ++j) {
-            const int s = rl_i(slot, j);
-            if (s < 0) continue;
-            uint8_t *row = codes + (int64_t)s * model_dim;
-            if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(row) + u, make_uint2(w[0], w[1]));
-            else stream_store(reinterpret_cast<uint32_t *>(row) + u, w[0]);
+    auto body = [&](auto mode) {
+        auto emit = [&](int u, const uint4 &raw) {
+            uint32_t w[2];
+            enc.template encode<decltype(mode)::value>(raw, w);
+            for (int j = 0; j < top_k; ++j) {
+                const int s = rl_i(slot, j);
+                if (s < 0) continue;
+                uint8_t *row = codes + (int64_t)s * model_dim;
+                if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(row) + u, make_uint2(w[0], w[1]));
+                else stream_store(reinterpret_cast<uint32_t *>(row) + u, w[0]);
+            }
+        };
+        if constexpr (CACHE > 0) {
+#pragma unroll
+            for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) emit(c * WAVE + lane, cache[c]);
+        } else {
+            for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
         }
     };
-    if constexpr (CACHE > 0) {
-#pragma unroll
-        for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) emit(c * WAVE + lane, cache[c]);
-    } else {
-        for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
-    }
+    if (enc.fast()) body(std::true_type{}); else body(std::false_type{});
 }
 
 template <int DT, int SDT>

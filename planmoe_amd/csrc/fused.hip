@@ -51,7 +51,9 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
 #pragma unroll
         for (int c = 0; c < CACHE; ++c) {
             const int u = c * WAVE + lane;
-            if (u < units) cache[c] = src[u];
+            // (index clamped, not predicated: straight-line loads let the compiler wait for exactly these
+            // loads; the re-read last vector is harmless for min / max and is never stored)
+            cache[c] = src[min(u, units - 1)];
         }
     }
     auto cache_ref = [&](int c) -> const uint4 & { return cache[c]; };
@@ -127,7 +129,7 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
             stats.init();
             if constexpr (CACHE > 0) {
 #pragma unroll
-                for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) stats.add(cache[c]);
+                for (int c = 0; c < CACHE; ++c) stats.add(cache[c]);
             } else {
                 for (int u = lane; u < units; u += WAVE) stats.add(src[u]);
             }
@@ -136,20 +138,23 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
             const float scale = E::round(mx - mn);
             if (lane < np && slot >= 0) { E::store(bias_out, slot, mn); E::store(scale_out, slot, scale); }
             const RowEncoder<DT> enc(mn, scale);
-            auto emit = [&](int u, const uint4 &raw) {
-                uint32_t w[2];
-                enc.encode(raw, w);
-                for (int j = 0; j < np; ++j) {
-                    const int s = rl_i(slot, j);
-                    if (s >= 0) put(s, u, w);
+            auto body = [&](auto mode) {
+                auto emit = [&](int u, const uint4 &raw) {
+                    uint32_t w[2];
+                    enc.template encode<decltype(mode)::value>(raw, w);
+                    for (int j = 0; j < np; ++j) {
+                        const int s = rl_i(slot, j);
+                        if (s >= 0) put(s, u, w);
+                    }
+                };
+                if constexpr (CACHE > 0) {
+#pragma unroll
+                    for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) emit(c * WAVE + lane, cache[c]);
+                } else {
+                    for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
                 }
             };
-            if constexpr (CACHE > 0) {
-#pragma unroll
-                for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) emit(c * WAVE + lane, cache[c]);
-            } else {
-                for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
-            }
+            if (enc.fast()) body(std::true_type{}); else body(std::false_type{});
         } else {
             // min / max of the unscaled row once: rounding and scaling by a finite non-zero gate
             // are monotonic, so the extremes of round(0 + g * x) are the images of the extremes
@@ -157,7 +162,7 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
             stats.init();
             if constexpr (CACHE > 0) {
 #pragma unroll
-                for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) stats.add(cache[c]);
+                for (int c = 0; c < CACHE; ++c) stats.add(cache[c]);
             } else {
                 for (int u = lane; u < units; u += WAVE) stats.add(src[u]);
             }

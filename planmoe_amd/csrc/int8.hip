@@ -11,7 +11,9 @@
 namespace pm {
 
 // VECTOR: row_len % VEC == 0 and 16-byte aligned rows; CACHE = vectors per lane kept in registers
-template <int DT, int CACHE>
+// WIDE (16-bit types, row_len % 16 == 0, 16-byte aligned code rows): a lane takes two adjacent
+// vectors (32 bytes of the row) so that its 16 codes leave as one 16-byte store
+template <int DT, int CACHE, bool WIDE>
 __global__ __launch_bounds__(256) void int8_compress_vec_kernel(
     const void *__restrict__ x, int64_t rows, int row_len, uint8_t *__restrict__ codes,
     void *__restrict__ bias_out, void *__restrict__ scale_out)
@@ -24,18 +26,22 @@ __global__ __launch_bounds__(256) void int8_compress_vec_kernel(
     const int units = row_len / V;
     const uint4 *src = reinterpret_cast<const uint4 *>((const char *)x + r * row_len * (int64_t)sizeof(typename E::store_t));
 
+    static_assert(!WIDE || (V == 8 && CACHE > 0 && CACHE % 2 == 0), "wide stores pair up cached vectors");
+    auto unit_of = [&](int c) { return WIDE ? (c >> 1) * (2 * WAVE) + 2 * lane + (c & 1) : c * WAVE + lane; };
     uint4 cache[CACHE > 0 ? CACHE : 1];
     RowStats<DT, false> stats;
     stats.init();
     if constexpr (CACHE > 0) {
 #pragma unroll
         for (int c = 0; c < CACHE; ++c) {
-            const int u = c * WAVE + lane;
-            if (u < units) cache[c] = stream_load(src + u);
+            const int u = unit_of(c);
+            // (index clamped, not predicated: straight-line loads let the compiler wait for exactly these
+            // loads; the re-read last vector is harmless for min / max and is never stored)
+            cache[c] = stream_load(src + min(u, units - 1));
         }
 #pragma unroll
         for (int c = 0; c < CACHE; ++c)
-            if (c * WAVE + lane < units) stats.add(cache[c]);
+            stats.add(cache[c]);
     } else {
         for (int u = lane; u < units; u += WAVE) stats.add(src[u]);
     }
@@ -46,21 +52,36 @@ __global__ __launch_bounds__(256) void int8_compress_vec_kernel(
 
     uint8_t *dst = codes + r * row_len;
     const RowEncoder<DT> enc(mn, scale);
-    auto emit = [&](int u, const uint4 &raw) {
-        uint32_t w[2];
-        enc.encode(raw, w);
-        if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(dst) + u, make_uint2(w[0], w[1]));
-        else stream_store(reinterpret_cast<uint32_t *>(dst) + u, w[0]);
-    };
-    if constexpr (CACHE > 0) {
+    auto body = [&](auto mode) {
+        constexpr bool FAST = decltype(mode)::value;
+        auto emit = [&](int u, const uint4 &raw) {
+            uint32_t w[2];
+            enc.template encode<FAST>(raw, w);
+            if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(dst) + u, make_uint2(w[0], w[1]));
+            else stream_store(reinterpret_cast<uint32_t *>(dst) + u, w[0]);
+        };
+        if constexpr (WIDE) {
 #pragma unroll
-        for (int c = 0; c < CACHE; ++c) {
-            const int u = c * WAVE + lane;
-            if (u < units) emit(u, cache[c]);
+            for (int c = 0; c < CACHE; c += 2) {
+                const int u = unit_of(c);             // even, and units is even: u + 1 < units as well
+                if (u < units) {
+                    uint32_t w[4];
+                    enc.template encode<FAST>(cache[c], w);
+                    enc.template encode<FAST>(cache[c + 1], w + 2);
+                    stream_store(reinterpret_cast<uint4 *>(dst) + (u >> 1), make_uint4(w[0], w[1], w[2], w[3]));
+                }
+            }
+        } else if constexpr (CACHE > 0) {
+#pragma unroll
+            for (int c = 0; c < CACHE; ++c) {
+                const int u = c * WAVE + lane;
+                if (u < units) emit(u, cache[c]);
+            }
+        } else {
+            for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
         }
-    } else {
-        for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
-    }
+    };
+    if (enc.fast()) body(std::true_type{}); else body(std::false_type{});
 }
 
 // any row length / alignment: one element per lane access
@@ -137,11 +158,23 @@ static void launch_compress(const void *x, int64_t rows, int row_len, uint8_t *c
         return;
     }
     const int per_lane = (row_len / Elem<DT>::VEC + WAVE - 1) / WAVE;
-    if (per_lane <= 2)       int8_compress_vec_kernel<DT, 2><<<blocks, 256, 0, st>>>(x, rows, row_len, codes, bias, scale);
-    else if (per_lane <= 4)  int8_compress_vec_kernel<DT, 4><<<blocks, 256, 0, st>>>(x, rows, row_len, codes, bias, scale);
-    else if (per_lane <= 8)  int8_compress_vec_kernel<DT, 8><<<blocks, 256, 0, st>>>(x, rows, row_len, codes, bias, scale);
-    else if (per_lane <= 16) int8_compress_vec_kernel<DT, 16><<<blocks, 256, 0, st>>>(x, rows, row_len, codes, bias, scale);
-    else                     int8_compress_vec_kernel<DT, 0><<<blocks, 256, 0, st>>>(x, rows, row_len, codes, bias, scale);
+#define PM_I8C(CACHE, WIDE) \
+    int8_compress_vec_kernel<DT, CACHE, WIDE><<<blocks, 256, 0, st>>>(x, rows, row_len, codes, bias, scale)
+    if constexpr (Elem<DT>::VEC == 8) {
+        if (row_len % 16 == 0 && aligned16(codes) && per_lane <= 16) {
+            if (per_lane <= 2) PM_I8C(2, true);
+            else if (per_lane <= 4) PM_I8C(4, true);
+            else if (per_lane <= 8) PM_I8C(8, true);
+            else PM_I8C(16, true);
+            return;
+        }
+    }
+    if (per_lane <= 2) PM_I8C(2, false);
+    else if (per_lane <= 4) PM_I8C(4, false);
+    else if (per_lane <= 8) PM_I8C(8, false);
+    else if (per_lane <= 16) PM_I8C(16, false);
+    else PM_I8C(0, false);
+#undef PM_I8C
 }
 
 } // namespace pm

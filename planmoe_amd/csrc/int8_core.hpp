@@ -1,6 +1,7 @@
 // Element-level arithmetic of the "int8" codec, shared by the stand-alone and fused kernels.
 #pragma once
 #include "common.hpp"
+#include <type_traits>
 
 namespace pm {
 
@@ -15,12 +16,12 @@ __device__ __forceinline__ uint32_t quantise(float v, float bias, float scale)
     return (m >= 1.0f) ? (uint32_t)fminf(m, 255.0f) : 0u;
 }
 
-// Per-row quantiser.  For bf16 the quotient (x - bias) / scale is a ratio of two 8-bit
-// significands: it can only sit on a bf16 rounding boundary when it is exactly representable,
-// and every other quotient is more than 2^-17 (relative) away from one.  So a reciprocal
-// multiply with one residual correction -- exact whenever the quotient is representable, within
-// a few 2^-24 otherwise -- rounds to the same bf16 value as the IEEE division.  Scales outside
-// [2^-100, 2^100] and the other dtypes take the IEEE division.
+// Per-row quantiser.  For bf16 the quotient (x - bias) / scale is a ratio a / b of two 8-bit
+// significands.  It is never a bf16 rounding boundary (a 9-bit midpoint m / 2^9 with m odd would
+// need a = m * b / 2^k >= 257), and it is at least 1 / (512 b) > 2^-17 (relative) away from
+// every boundary, while d * fl(1 / scale) is within 2^-23 of it.  So the reciprocal multiply
+// rounds to the same bf16 value as the IEEE division followed by the bf16 rounding.  Scales
+// outside [2^-100, 2^100] and the other dtypes take the IEEE division.
 template <int DT>
 struct RowQuant {
     float bias, scale, inv;
@@ -38,10 +39,7 @@ struct RowQuant {
             if (fast) {
                 using E = Elem<DT>;
                 const float d = E::round(v - bias);
-                float t = d * inv;
-                const float r = fmaf(-t, scale, d);
-                t = fmaf(r, inv, t);
-                const float q = E::round(t);
+                const float q = E::round(d * inv);
                 const float m = E::round(q * 255.0f);
                 return (m >= 1.0f) ? (uint32_t)fminf(m, 255.0f) : 0u;
             }
@@ -61,7 +59,7 @@ __device__ __forceinline__ float dequantise(uint32_t code, float bias, float sca
 }
 
 // Per-row dequantiser.  code / 255 is again a ratio of two 8-bit integers, so the bf16 path
-// can use the corrected reciprocal multiply (see RowQuant).
+// can use the reciprocal multiply (see RowQuant).
 template <int DT>
 struct RowDequant {
     float bias, scale;
@@ -72,10 +70,7 @@ struct RowDequant {
             using E = Elem<DT>;
             const float c = (float)code;
             constexpr float inv = 1.0f / 255.0f;
-            float t = c * inv;
-            const float r = fmaf(-t, 255.0f, c);
-            t = fmaf(r, inv, t);
-            float v = E::round(t);
+            float v = E::round(c * inv);
             v = E::round(v * scale);
             return E::round(v + bias);
         } else {
@@ -113,6 +108,9 @@ struct RowEncoder {
     using E = Elem<DT>;
     RowQuant<DT> rq;
     __device__ __forceinline__ RowEncoder(float bias, float scale) : rq(bias, scale) {}
+    // no reciprocal path for this dtype: both modes are the IEEE division
+    __device__ __forceinline__ constexpr bool fast() const { return false; }
+    template <bool FAST>
     __device__ __forceinline__ void encode(const uint4 &raw, uint32_t *w) const
     {
         float f[E::VEC];
@@ -186,27 +184,29 @@ template <>
 struct RowEncoder<PLANMOE_BF16> {
     RowQuant<PLANMOE_BF16> rq;
     __device__ __forceinline__ RowEncoder(float bias, float scale) : rq(bias, scale) {}
+    // The mode is a property of the row, hence of the whole wave: callers branch on it once
+    // (a scalar branch) and run one of two straight-line encoders.
+    __device__ __forceinline__ bool fast() const { return __builtin_amdgcn_readfirstlane((int)rq.fast) != 0; }
     // two bf16 in w -> code0 | code1 << 8
+    template <bool FAST>
     __device__ __forceinline__ uint32_t pair(uint32_t w) const
     {
         const float f0 = __uint_as_float(w << 16), f1 = __uint_as_float(w & 0xffff0000u);
-        if (!rq.fast) return rq(0.f + f0) | (rq(0.f + f1) << 8);
+        if constexpr (!FAST) return quantise<PLANMOE_BF16>(0.f + f0, rq.bias, rq.scale) | (quantise<PLANMOE_BF16>(0.f + f1, rq.bias, rq.scale) << 8);
         uint32_t pk = f32x2_to_bf16x2(f0 - rq.bias, f1 - rq.bias);
         const float d0 = __uint_as_float(pk << 16), d1 = __uint_as_float(pk & 0xffff0000u);
-        float t0 = d0 * rq.inv, t1 = d1 * rq.inv;
-        t0 = fmaf(fmaf(-t0, rq.scale, d0), rq.inv, t0);
-        t1 = fmaf(fmaf(-t1, rq.scale, d1), rq.inv, t1);
-        pk = f32x2_to_bf16x2(t0, t1);
+        pk = f32x2_to_bf16x2(d0 * rq.inv, d1 * rq.inv);
         const float q0 = __uint_as_float(pk << 16), q1 = __uint_as_float(pk & 0xffff0000u);
         pk = f32x2_to_bf16x2(q0 * 255.0f, q1 * 255.0f);
         const float m0 = __uint_as_float(pk << 16), m1 = __uint_as_float(pk & 0xffff0000u);
         // truncation; the conversion saturates NaN (0/0 rows) and negatives to 0, m <= 255
         return __float2uint_rz(m0) | (__float2uint_rz(m1) << 8);
     }
+    template <bool FAST>
     __device__ __forceinline__ void encode(const uint4 &raw, uint32_t *w) const
     {
-        w[0] = pair(raw.x) | (pair(raw.y) << 16);
-        w[1] = pair(raw.z) | (pair(raw.w) << 16);
+        w[0] = pair<FAST>(raw.x) | (pair<FAST>(raw.y) << 16);
+        w[1] = pair<FAST>(raw.z) | (pair<FAST>(raw.w) << 16);
     }
 };
 

@@ -401,7 +401,10 @@ def zfp_compress(field, nx, ny, dims=2, rate=8.0, out=None):
     _need_gpu(field, "zfp_compress")
     field = _contig(field, "zfp_compress")
     if out is None:
-        out = torch.zeros((zfp_max_bytes(dims, nx, ny, rate),), dtype=torch.uint8, device=field.device)
+        # the kernel writes every byte of the stream; only the slack up to the maximum size
+        # (what the reference's torch::zeros leaves as zeros) is cleared here
+        out = torch.empty((zfp_max_bytes(dims, nx, ny, rate),), dtype=torch.uint8, device=field.device)
+        out[zfp_stream_bytes(dims, nx, ny, rate):].zero_()
     check(lib.planmoe_zfp_compress(_ptr(field), dims, nx, ny, float(rate), _ptr(out), out.numel(),
                                    _stream(field)))
     return out

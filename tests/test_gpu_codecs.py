@@ -56,7 +56,8 @@ def test_int8_against_oracle(R, M, dtype):
 def test_int8_exhaustive_bf16():
     from planmoe_amd import ops
     allv = from_bf16_bits(np.arange(0, 65536, dtype=np.uint32).astype(np.uint16)).float()
-    for lo, hi in ((-1.0, 1.0), (0.0, 3.140625), (-250.0, 7.5)):
+    for lo, hi in ((-1.0, 1.0), (0.0, 3.140625), (-250.0, 7.5), (0.0, 1.9921875), (-0.5, 0.5078125),
+                   (-3.0517578125e-05, 2.2172927856445312e-05), (-1e20, 3e20), (0.33203125, 5.03125)):
         vals = allv[torch.isfinite(allv) & (allv >= lo) & (allv <= hi) & (allv != 0)]
         row = torch.cat([torch.tensor([lo, hi, 0.0]), vals])
         row = torch.cat([row, row.new_full(((-len(row)) % 8,), lo)]).to(torch.bfloat16)[None, :]
