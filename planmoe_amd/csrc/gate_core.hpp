@@ -77,16 +77,12 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
 
     const uint4 *ap[TPW];
     const uint4 *bp[NT];
-    bool bv[NT];                                     // lane holds a real gate-weight row
 #pragma unroll
     for (int tp = 0; tp < TPW; ++tp)
         ap[tp] = reinterpret_cast<const uint4 *>(x) + (int64_t)min(t0 + tp * 16 + m, samples - 1) * nv + g;
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
-    {
-        bv[nt] = nt * 16 + m < experts;
         bp[nt] = reinterpret_cast<const uint4 *>(wg) + (int64_t)min(nt * 16 + m, experts - 1) * nv + g;
-    }
 
     f32x4 acc[TPW][NT];
 #pragma unroll
@@ -100,15 +96,14 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
         for (int tp = 0; tp < TPW; ++tp)
 #pragma unroll
             for (int s = 0; s < 4; ++s) f.a[tp][s] = ap[tp][o + s * 4];
+        // lanes past the last expert re-read the last gate-weight row (clamped above): their
+        // products only reach tile columns nobody reads.  No predicate here, and no branch around
+        // a prefetch below: the compiler counts outstanding loads per basic block, and a load
+        // that may or may not have been issued makes it wait for everything.
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            // lanes past the last expert skip the load: whatever their registers hold only
-            // reaches tile columns nobody reads
-            if (bv[nt]) {
+        for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-                for (int s = 0; s < 4; ++s) f.b[nt][s] = bp[nt][o + s * 4];
-            }
-        }
+            for (int s = 0; s < 4; ++s) f.b[nt][s] = bp[nt][o + s * 4];
     };
     auto mma = [&](const GateFrag<NT, TPW> &f) {
 #pragma unroll
@@ -122,18 +117,22 @@ __device__ __forceinline__ void gate_tile_partials(const void *__restrict__ x,
     };
 
     GateFrag<NT, TPW> f0, f1;
-    int step = w;
-    if (step < full) load(f0, step);
-    while (step < full) {
-        const bool more1 = step + NW < full;
-        if (more1) load(f1, step + NW);
-        mma(f0);
-        if (!more1) break;
-        const bool more2 = step + 2 * NW < full;
-        if (more2) load(f0, step + 2 * NW);
-        mma(f1);
-        step += 2 * NW;
-        if (!more2) break;
+    if (w < full) {
+        const int nsteps = (full - w + NW - 1) / NW;     // steps of this wave: w, w + NW, ...
+        const int last = w + (nsteps - 1) * NW;
+        int step = w;
+        if (nsteps & 1) { load(f0, step); mma(f0); step += NW; }
+        if (step <= last) {
+            // pairs of steps, one straight-line body: each buffer is re-filled while the MFMAs of
+            // the other run.  The last prefetch re-reads the wave's last step (a cache hit).
+            load(f0, step);
+            for (; step <= last; step += 2 * NW) {
+                load(f1, step + NW);
+                mma(f0);
+                load(f0, min(step + 2 * NW, last));
+                mma(f1);
+            }
+        }
     }
 
     if (rem && (full % NW) == w) {
@@ -243,28 +242,17 @@ __device__ __forceinline__ void gate_tile_lds(const void *__restrict__ x, const 
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) acc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // vectors past the row end read as zero in BOTH operands
+    const int full = nv / 16, rem = nv % 16;
+    // full chunks: straight-line loads (no predicate, no branch around a prefetch, so that the
+    // compiler can count the loads in flight and wait for the older buffer only)
     auto load_a = [&](uint4 (&a)[4], int c) {
         const int o = c * 16 + g;
-        if (c * 16 + 16 <= nv) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) a[s] = ap[o + 4 * s];
-        } else {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                a[s] = make_uint4(0, 0, 0, 0);
-                if (o + 4 * s < nv) a[s] = ap[o + 4 * s];
-            }
-        }
+        for (int s = 0; s < 4; ++s) a[s] = ap[o + 4 * s];
     };
     auto load_b = [&](uint4 (&b)[BV], int c) {
-        const int o = c * 16;
-        const bool in = o + bvec < nv;
 #pragma unroll
-        for (int i = 0; i < BV; ++i) {
-            b[i] = make_uint4(0, 0, 0, 0);
-            if (in) b[i] = bp[i][o];
-        }
+        for (int i = 0; i < BV; ++i) b[i] = bp[i][c * 16];
     };
     auto store_b = [&](const uint4 (&b)[BV], int buf) {
 #pragma unroll
@@ -279,26 +267,57 @@ __device__ __forceinline__ void gate_tile_lds(const void *__restrict__ x, const 
             for (int nt = 0; nt < NT; ++nt) bf[nt] = bb[nt * 256 + ((4 * s + g) ^ m)];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) Mma<DT>::run(a[s], bf[nt], acc[nt]);
-            if constexpr (STATS) st.add(a[s]);
+        }
+    };
+    auto scan = [&](const uint4 (&a)[4]) {
+        if constexpr (STATS) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) st.add(a[s]);
         }
     };
 
     uint4 a0[4], a1[4], bs[BV];
-    load_a(a0, 0);
-    load_b(bs, 0);
-    store_b(bs, 0);
-    __syncthreads();
-    for (int c = 0; c < chunks; c += 2) {
-        const bool more1 = c + 1 < chunks;
-        if (more1) { load_a(a1, c + 1); load_b(bs, c + 1); }
-        compute(a0, 0);
-        if (more1) store_b(bs, 1);
+    if (full > 0) {
+        load_a(a0, 0);
+        load_b(bs, 0);
+        store_b(bs, 0);
         __syncthreads();
-        if (!more1) break;
-        const bool more2 = c + 2 < chunks;
-        if (more2) { load_a(a0, c + 2); load_b(bs, c + 2); }
-        compute(a1, 1);
-        if (more2) store_b(bs, 0);
+        int c = 0;
+        while (true) {
+            if (c + 1 >= full) { compute(a0, 0); scan(a0); __syncthreads(); break; }
+            load_a(a1, c + 1); load_b(bs, c + 1);
+            compute(a0, 0); scan(a0);
+            store_b(bs, 1);
+            __syncthreads();
+            ++c;
+            if (c + 1 >= full) { compute(a1, 1); scan(a1); __syncthreads(); break; }
+            load_a(a0, c + 1); load_b(bs, c + 1);
+            compute(a1, 1); scan(a1);
+            store_b(bs, 0);
+            __syncthreads();
+            ++c;
+        }
+    }
+    if (rem) {
+        // last, partial chunk: vectors past the row end are read from a clamped index (valid
+        // memory, harmless for the min / max scan) and enter the products as zero in BOTH operands
+        const int o = full * 16;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int v = 4 * s + g;
+            a0[s] = ap[o + min(v, rem - 1)];
+        }
+        scan(a0);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) if (4 * s + g >= rem) a0[s] = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < BV; ++i) {
+            bs[i] = bp[i][o + min(bvec, rem - 1) - bvec];
+            if (bvec >= rem) bs[i] = make_uint4(0, 0, 0, 0);
+        }
+        store_b(bs, 0);                                  // every wave is past the barrier of the loop
+        __syncthreads();
+        compute(a0, 0);
         __syncthreads();
     }
 

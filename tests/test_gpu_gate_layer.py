@@ -201,3 +201,23 @@ def test_fused_forward_matches_unfused_and_oracle(T, M, E, k, cf, dtype, fp32_ga
             assert torch.equal(r2[name], out[name])
         assert np.array_equal(raw(r2["gates"]), raw(out["gates"]))
         assert abs(float(r2["l_aux"]) - float(out["l_aux"])) == 0
+
+
+@pytest.mark.parametrize("T,M,E,k", [(300, 776, 24, 2), (200, 264, 8, 2), (130, 1032, 64, 1)])
+def test_fused_forward_rows_of_one_sign(T, M, E, k):
+    """Row min / max come out of the gate kernel's scan of the rows it streams: rows that do not
+    straddle zero and a model_dim that is not a multiple of a K chunk (128 bf16 values) show a
+    scan that picks up padding."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(T + M)
+    x = (torch.randn(T, M, generator=g).abs() + 0.5)
+    x[::3] *= -1
+    x = x.bfloat16().to(DEV)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
+    C = ops.capacity(T, E, k, 1.5, 4)
+    out = ops.forward_int8(x, wg, k, C)
+    c2, b2, s2 = ops.dispatch_int8(x, list(out["indices"]), list(out["locations"]), None, E, C)
+    assert torch.equal(out["codes"], c2)
+    assert np.array_equal(raw(out["bias"]), raw(b2)) and np.array_equal(raw(out["scale"]), raw(s2))
+    rc, rb, rs = oracle.int8_compress(bf16_bits(ops.dispatch_fwd(x, list(out["indices"]), list(out["locations"]), None, E, C).cpu()))
+    assert np.array_equal(c2.cpu().numpy().reshape(rc.shape), rc)
