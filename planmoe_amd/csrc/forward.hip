@@ -30,14 +30,22 @@ namespace pm {
 __host__ __device__ inline int fwd_group_tokens(int) { return 64; }
 constexpr int FWD_LOSS_PARTS = 64;
 
+// hist_t / me_t are the transposes of hist / me with the group index running fastest (rows of
+// gstride = groups rounded up to 4 entries, the padding zero): a column of the histogram, which
+// is what a prefix over groups reads, is contiguous there.
 struct FwdWs {
-    int32_t *totals, *hist, *offs, *rank;
-    float *loss_part, *me, *row_min, *row_max;
+    int32_t *totals, *hist, *offs, *rank, *hist_t;
+    float *loss_part, *me, *row_min, *row_max, *me_t;
+    int gstride;
 };
+__host__ __device__ inline size_t fwd_pad4(size_t words) { return (words + 3) & ~(size_t)3; }
 __host__ __device__ inline FwdWs fwd_ws(void *ws, int groups, int k, int experts, int samples)
 {
     FwdWs w;
-    w.totals = (int32_t *)ws;
+    w.gstride = (int)fwd_pad4((size_t)groups);
+    w.hist_t = (int32_t *)ws;                                   // 16-byte aligned rows
+    w.me_t = (float *)(w.hist_t + (size_t)k * experts * w.gstride);
+    w.totals = (int32_t *)(w.me_t + (size_t)experts * w.gstride);
     w.loss_part = (float *)(w.totals + experts);
     w.hist = (int32_t *)(w.loss_part + FWD_LOSS_PARTS);
     w.offs = w.hist + (size_t)groups * k * experts;
@@ -46,6 +54,38 @@ __host__ __device__ inline FwdWs fwd_ws(void *ws, int groups, int k, int experts
     w.row_min = (float *)(w.rank + (size_t)k * samples);
     w.row_max = w.row_min + samples;
     return w;
+}
+
+// This lane's share of the sum of col[0 .. limit): col is 16-byte aligned and readable up to the
+// next multiple of 4 entries, limit is the same in every lane.  The wave reduction is left to the
+// caller so that several columns can be loaded back to back and reduced together (one memory
+// round trip and interleaved shuffle chains instead of one after the other).
+__device__ __forceinline__ int column_partial(const int32_t *__restrict__ col, int limit)
+{
+    int s = 0;
+    for (int i = lane_id() * 4; i < limit; i += 4 * WAVE) {
+        const int4 v = *reinterpret_cast<const int4 *>(col + i);
+        s += v.x + (i + 1 < limit ? v.y : 0) + (i + 2 < limit ? v.z : 0) + (i + 3 < limit ? v.w : 0);
+    }
+    return s;
+}
+__device__ __forceinline__ float column_partial(const float *__restrict__ col, int limit)
+{
+    float s = 0.f;
+    for (int i = lane_id() * 4; i < limit; i += 4 * WAVE) {
+        const float4 v = *reinterpret_cast<const float4 *>(col + i);
+        s += (v.x + (i + 1 < limit ? v.y : 0.f)) + ((i + 2 < limit ? v.z : 0.f) + (i + 3 < limit ? v.w : 0.f));
+    }
+    return s;
+}
+// wave sums of N values at once
+template <typename T, int N>
+__device__ __forceinline__ void wave_sum_n(T (&v)[N])
+{
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1)
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] += __shfl_xor(v[i], off, WAVE);
 }
 
 __device__ __forceinline__ uint64_t lanes_below() { return ((uint64_t)1 << lane_id()) - 1; }
@@ -133,7 +173,10 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
                 for (int e = 0; e < CAP; ++e) {
                     if (e < experts) {
                         const float v = wave_sum(valid ? s[e] : 0.f);
-                        if (lane == 0) ws.me[(int64_t)blockIdx.x * experts + e] = v;
+                        if (lane == 0) {
+                            ws.me[(int64_t)blockIdx.x * experts + e] = v;
+                            ws.me_t[(int64_t)e * ws.gstride + blockIdx.x] = v;
+                        }
                     }
                 }
             } else {
@@ -147,6 +190,7 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
 #pragma unroll 8
                     for (int r = 0; r < GROUP; ++r) v += part[0][r][e];
                     ws.me[(int64_t)blockIdx.x * experts + e] = v;
+                    ws.me_t[(int64_t)e * ws.gstride + blockIdx.x] = v;
                 }
             }
         }
@@ -184,7 +228,13 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
             }
             if (valid) ws.rank[(int64_t)j * samples + t] = rank;
             __builtin_amdgcn_wave_barrier();
-            if (lane < experts) ws.hist[((int64_t)blockIdx.x * k + j) * experts + lane] = s_hist[lane];
+            if (lane < experts) {
+                ws.hist[((int64_t)blockIdx.x * k + j) * experts + lane] = s_hist[lane];
+                int32_t *col = ws.hist_t + ((int64_t)j * experts + lane) * ws.gstride;
+                col[blockIdx.x] = s_hist[lane];
+                if ((int)blockIdx.x == groups - 1)             // the last group also clears the padding
+                    for (int p = groups; p < ws.gstride; ++p) col[p] = 0;
+            }
         }
         if (valid && k > 1 && normalize_gate) {
             const float eps = SDT == PLANMOE_F32 ? 1.1920928955078125e-07f
@@ -221,27 +271,105 @@ __global__ __launch_bounds__(256) void route_offsets_kernel(const int32_t *__res
 
 // Dispatch + int8 with the slot offsets still to be added (see dispatch_int8_kernel for the
 // stand-alone variant).  Only the all-ones gate helper (is_postscore) is fused here.
-template <int DT, int CACHE>
+//
+// MERGED: there was no group_offsets launch.  Every wave sums the histogram columns it needs
+// itself (hist_t: one or two 16-byte loads per lane and column, k (k + 1) / 2 columns per token),
+// the zero-fill blocks sum the expert totals, and one more block at the end of the grid finishes
+// the GShard loss and the per-plane expert counts.  Used for top_k <= 4.
+template <int DT, int CACHE, bool MERGED>
 __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     const void *__restrict__ x, const int32_t *__restrict__ indices, int32_t *__restrict__ locations,
     int64_t stride, int top_k, int samples, int model_dim, int experts, int capacity,
     uint8_t *__restrict__ codes, void *__restrict__ bias_out, void *__restrict__ scale_out,
     const int32_t *__restrict__ hist, const int32_t *__restrict__ totals, const int32_t *__restrict__ rank,
     int group_tokens, int token_blocks, const float *__restrict__ loss_part, int loss_parts,
-    float *__restrict__ l_aux, const float *__restrict__ row_min, const float *__restrict__ row_max)
+    float *__restrict__ l_aux, const float *__restrict__ row_min, const float *__restrict__ row_max,
+    const int32_t *__restrict__ hist_t, const float *__restrict__ me_t, int groups, int gstride,
+    int fill_blocks, int32_t *__restrict__ counts_out, int fill_first)
 {
     using E = Elem<DT>;
     constexpr int V = E::VEC;
     const int wave = threadIdx.x >> 6, lane = lane_id();
     const int units = model_dim / V;
-    finish_loss(loss_part, loss_parts, samples, l_aux);
+    __shared__ int32_t s_tot[64];
+    __shared__ float s_loss[64];
+    if constexpr (!MERGED) finish_loss(loss_part, loss_parts, samples, l_aux);
 
-    if ((int)blockIdx.x >= token_blocks) {
+    // grid order: the block that finishes the loss (MERGED only; it starts with a few dependent
+    // round trips over the histogram, which the streaming blocks behind it hide), then the token
+    // blocks and the zero-fill blocks; the fill blocks go first when their own histogram pass is
+    // long (many experts), last otherwise (measured both ways at 8 and at 64 experts).
+    const int stat_blocks = (int)gridDim.x - fill_blocks - token_blocks;
+    int bid = (int)blockIdx.x - stat_blocks;                              // < token_blocks: token block
+    if (fill_first && bid >= 0) bid = bid < fill_blocks ? token_blocks + bid : bid - fill_blocks;
+    if constexpr (MERGED) {
+        if ((int)blockIdx.x < stat_blocks) {
+            // the one block that finishes the loss: l_aux = sum_e me[e] * ce[e] / T with
+            // me[e] = column sum of the scores, ce[e] = first-choice count * E / T
+            // four experts per pass and wave: the loads of a pass are in flight together
+            for (int e0 = wave * 4; e0 < experts; e0 += 16) {
+                int c0[4] = {0, 0, 0, 0};
+                float m[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if (e0 + q < experts) {
+                        c0[q] = column_partial(hist_t + (int64_t)(e0 + q) * gstride, groups);
+                        if (l_aux) m[q] = column_partial(me_t + (int64_t)(e0 + q) * gstride, groups);
+                    }
+                }
+                wave_sum_n(c0);
+                wave_sum_n(m);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if (lane == 0 && e0 + q < experts) {
+                        if (counts_out) counts_out[e0 + q] = c0[q];
+                        s_loss[e0 + q] = m[q] * ((float)c0[q] * ((float)experts / (float)samples));
+                    }
+                }
+                if (counts_out) {
+                    for (int j = 1; j < top_k; ++j) {
+                        int c[4] = {0, 0, 0, 0};
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            if (e0 + q < experts) c[q] = column_partial(hist_t + ((int64_t)j * experts + e0 + q) * gstride, groups);
+                        wave_sum_n(c);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) if (lane == 0 && e0 + q < experts) counts_out[j * experts + e0 + q] = c[q];
+                    }
+                }
+            }
+            __syncthreads();
+            if (l_aux && threadIdx.x == 0) {
+                float a = 0.f;
+                for (int e = 0; e < experts; ++e) a += s_loss[e];
+                *l_aux = a / (float)samples;
+            }
+            return;
+        }
+    }
+
+    if (bid >= token_blocks) {
         const int slots = experts * capacity;
-        const int nwaves = (gridDim.x - token_blocks) * 4;
-        for (int s = (blockIdx.x - token_blocks) * 4 + wave; s < slots; s += nwaves) {
+        const int nwaves = fill_blocks * 4;
+        const int fid = bid - token_blocks;
+        if constexpr (MERGED) {
+            // expert totals, four experts per pass and wave: the loads of a pass are in flight together
+            for (int e0 = wave * 4; e0 < experts; e0 += 16) {
+                int c[4] = {0, 0, 0, 0};
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (e0 + q < experts)
+                        for (int j = 0; j < top_k; ++j) c[q] += column_partial(hist_t + ((int64_t)j * experts + e0 + q) * gstride, groups);
+                wave_sum_n(c);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) if (lane == 0 && e0 + q < experts) s_tot[e0 + q] = c[q];
+            }
+            __syncthreads();
+        }
+        for (int s = fid * 4 + wave; s < slots; s += nwaves) {
             const int e = s / capacity;
-            if (s - e * capacity < totals[e]) continue;          // slot holds a token
+            const int filled = MERGED ? s_tot[e] : totals[e];
+            if (s - e * capacity < filled) continue;             // slot holds a token
             uint8_t *row = codes + (int64_t)s * model_dim;
             for (int u = lane; u < units; u += WAVE) {
                 if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(row) + u, make_uint2(0u, 0u));
@@ -254,7 +382,7 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
 
     // tokens are walked from the last to the first: the rows the gate kernel read most recently
     // are the likeliest to still sit in cache
-    const int t = samples - 1 - (int)(blockIdx.x * 4 + wave);
+    const int t = samples - 1 - (bid * 4 + wave);
     if (t < 0) return;
     const uint4 *src = reinterpret_cast<const uint4 *>((const char *)x + (int64_t)t * model_dim * (int64_t)sizeof(typename E::store_t));
     uint4 cache[CACHE > 0 ? CACHE : 1];
@@ -270,7 +398,32 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
 
     // lane j finalises choice j: slot = expert * capacity + rank in group + group offset
     int slot = -1;
-    if (lane < top_k) {
+    if constexpr (MERGED) {
+        int e_l = 0, l = 0;
+        if (lane < top_k) {
+            e_l = indices[(int64_t)lane * stride + t];
+            l = rank[(int64_t)lane * samples + t];
+        }
+        const int g = t / group_tokens;
+        // slots of expert e taken before this group's plane-j tokens: every entry of the planes
+        // before j, and the groups before g in plane j
+        int before[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (j < top_k) {
+                const int e = rl_i(e_l, j);
+                before[j] = column_partial(hist_t + ((int64_t)j * experts + e) * gstride, g);
+                for (int jp = 0; jp < j; ++jp) before[j] += column_partial(hist_t + ((int64_t)jp * experts + e) * gstride, groups);
+            }
+        }
+        wave_sum_n(before);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) if (lane == j) l += before[j];
+        if (lane < top_k) {
+            locations[(int64_t)lane * stride + t] = l;
+            if (l < capacity) slot = e_l * capacity + l;
+        }
+    } else if (lane < top_k) {
         const int64_t o = (int64_t)lane * stride + t;
         const int e = indices[o];
         const int l = rank[(int64_t)lane * samples + t] + hist[((int64_t)(t / group_tokens) * top_k + lane) * experts + e];
@@ -344,18 +497,23 @@ static void launch_dispatch_routed(int per_lane, unsigned grid, hipStream_t st, 
                                    void *bias, void *scale, const int32_t *offs, const int32_t *totals,
                                    const int32_t *rank, int group_tokens, int token_blocks,
                                    const float *loss_part, int loss_parts, float *l_aux,
-                                   const float *row_min, const float *row_max)
+                                   const float *row_min, const float *row_max, bool merged,
+                                   const int32_t *hist_t, const float *me_t, int groups, int gstride,
+                                   int fill_blocks, int32_t *counts, int fill_first)
 {
-#define PM_DR(CACHE)                                                                                 \
-    dispatch_int8_routed_kernel<DT, CACHE><<<grid, 256, 0, st>>>(x, indices, locations, stride, top_k, \
+#define PM_DR_(CACHE, MERGED)                                                                        \
+    dispatch_int8_routed_kernel<DT, CACHE, MERGED><<<grid, 256, 0, st>>>(x, indices, locations, stride, top_k, \
         samples, model_dim, experts, capacity, codes, bias, scale, offs, totals, rank, group_tokens,  \
-        token_blocks, loss_part, loss_parts, l_aux, row_min, row_max)
+        token_blocks, loss_part, loss_parts, l_aux, row_min, row_max, hist_t, me_t, groups, gstride,  \
+        fill_blocks, counts, fill_first)
+#define PM_DR(CACHE) do { if (merged) PM_DR_(CACHE, true); else PM_DR_(CACHE, false); } while (0)
     if (per_lane <= 2) PM_DR(2);
     else if (per_lane <= 4) PM_DR(4);
     else if (per_lane <= 8) PM_DR(8);
     else if (per_lane <= 16) PM_DR(16);
     else PM_DR(0);
 #undef PM_DR
+#undef PM_DR_
 }
 
 static int fused_check(const char *who, const void *x, const void *wg, int dtype, int samples,
@@ -375,22 +533,29 @@ static int fused_check(const char *who, const void *x, const void *wg, int dtype
 
 struct FwdPlan {
     int k, groups, group_tokens, experts_per_block, blocks;
+    bool merged;          // the dispatch launch does the prefix over groups itself
     FwdWs ws;
 };
-
-// launches gate_route_kernel and group_offsets_kernel
-static int run_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
-                          const float *logit_bias, int samples, int model_dim, int experts, int top_k,
-                          int normalize_gate, int32_t *indices, int32_t *locations, void *gates,
-                          int64_t stride, void *logits_out, void *scores_out, float *l_aux,
-                          int32_t *counts, void *workspace, hipStream_t st, FwdPlan &plan)
+static void fwd_plan(FwdPlan &plan, void *workspace, int samples, int experts, int top_k)
 {
     plan.k = top_k < experts ? top_k : experts;
     plan.group_tokens = fwd_group_tokens(experts);
     plan.groups = (samples + plan.group_tokens - 1) / plan.group_tokens;
     plan.experts_per_block = go_experts_per_block(experts, plan.k);
     plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
+    plan.merged = plan.k <= 4;
     plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts, samples);
+}
+
+// launches gate_route_kernel and, unless the dispatch launch will do that part, group_offsets_kernel
+static int run_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
+                          const float *logit_bias, int samples, int model_dim, int experts, int top_k,
+                          int normalize_gate, int32_t *indices, int32_t *locations, void *gates,
+                          int64_t stride, void *logits_out, void *scores_out, float *l_aux,
+                          int32_t *counts, void *workspace, hipStream_t st, FwdPlan &plan,
+                          bool offsets_follow)
+{
+    fwd_plan(plan, workspace, samples, experts, top_k);
     const int k = plan.k, groups = plan.groups;
     if (fp32_gate || dtype == PLANMOE_F32) {
         PM_DTYPE_SWITCH(dtype, DT, (launch_gate_route<DT, PLANMOE_F32>(
@@ -405,30 +570,39 @@ static int run_gate_route(const void *x, const void *wg, int dtype, int fp32_gat
             model_dim, k, normalize_gate, indices, locations, gates, stride, logits_out, scores_out,
             l_aux, counts, workspace);
     }
-    group_offsets_kernel<<<plan.blocks, 256, 0, st>>>(plan.ws.hist, plan.ws.offs, plan.ws.me, groups, k,
-                                                      experts, plan.experts_per_block, samples,
-                                                      plan.ws.totals, counts, plan.ws.loss_part,
-                                                      l_aux != nullptr);
+    if (offsets_follow)
+        group_offsets_kernel<<<plan.blocks, 256, 0, st>>>(plan.ws.hist, plan.ws.offs, plan.ws.me, groups, k,
+                                                          experts, plan.experts_per_block, samples,
+                                                          plan.ws.totals, counts, plan.ws.loss_part,
+                                                          l_aux != nullptr);
     return 0;
 }
 
 static int run_dispatch_routed(const void *x, int dtype, int samples, int model_dim, int experts,
                                int capacity, const int32_t *indices, int32_t *locations, int64_t stride,
-                               float *l_aux, uint8_t *codes, void *bias, void *scale, const FwdPlan &plan,
-                               hipStream_t st)
+                               float *l_aux, int32_t *counts, uint8_t *codes, void *bias, void *scale,
+                               const FwdPlan &plan, hipStream_t st)
 {
     const int slots = experts * capacity;
     const int token_blocks = (samples + 3) / 4;
-    const int fill_blocks = min((slots + 3) / 4, 2048);
+    int fill_blocks = min((slots + 3) / 4, 2048);
+    if (plan.merged) {
+        // every zero-fill block reads the whole transposed histogram once: keep that under ~32 MB
+        const int64_t table = (int64_t)plan.k * experts * plan.ws.gstride * 4;
+        fill_blocks = min(fill_blocks, (int)max((int64_t)64, ((int64_t)32 << 20) / table));
+    }
+    const int stat_blocks = plan.merged && (l_aux || counts) ? 1 : 0;
     const int vec = dtype == PLANMOE_F32 ? 4 : 8;
     const int per_lane = (model_dim / vec + WAVE - 1) / WAVE;
     PM_DTYPE_SWITCH(dtype, DT,
-        launch_dispatch_routed<DT>(per_lane, (unsigned)(token_blocks + fill_blocks), st, x, indices, locations,
-                                   stride, plan.k, samples, model_dim, experts, capacity, codes, bias,
+        launch_dispatch_routed<DT>(per_lane, (unsigned)(token_blocks + fill_blocks + stat_blocks), st, x, indices,
+                                   locations, stride, plan.k, samples, model_dim, experts, capacity, codes, bias,
                                    scale, plan.ws.offs, plan.ws.totals, plan.ws.rank, plan.group_tokens, token_blocks,
                                    plan.ws.loss_part, plan.blocks, l_aux,
                                    dtype == PLANMOE_BF16 ? plan.ws.row_min : nullptr,
-                                   dtype == PLANMOE_BF16 ? plan.ws.row_max : nullptr));
+                                   dtype == PLANMOE_BF16 ? plan.ws.row_max : nullptr, plan.merged,
+                                   plan.ws.hist_t, plan.ws.me_t, plan.groups, plan.ws.gstride, fill_blocks, counts,
+                                   plan.merged && plan.k * experts > 32));
     return 0;
 }
 
@@ -442,7 +616,7 @@ extern "C" size_t planmoe_forward_workspace_bytes(int samples, int experts, int 
     const size_t k = (size_t)(top_k < experts ? top_k : experts);
     const size_t groups = ((size_t)samples + 31) / 32;      // upper bound over the group sizes
     return round_up(((size_t)experts + FWD_LOSS_PARTS + 2 * groups * k * experts + groups * experts +
-                     (k + 2) * (size_t)samples) * 4, 256);
+                     (k + 2) * (size_t)samples + (k + 1) * experts * fwd_pad4(groups)) * 4, 256);
 }
 
 extern "C" int planmoe_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
@@ -461,7 +635,7 @@ extern "C" int planmoe_gate_route(const void *x, const void *wg, int dtype, int 
     FwdPlan plan;
     if (run_gate_route(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
                        normalize_gate, indices, locations, gates, plane_stride, logits_out, scores_out,
-                       l_aux, expert_counts, workspace, st, plan)) return 1;
+                       l_aux, expert_counts, workspace, st, plan, true)) return 1;
     route_offsets_kernel<<<(samples * plan.k + 255) / 256, 256, 0, st>>>(
         indices, locations, plane_stride, samples, experts, plan.k, plan.ws.offs, plan.ws.rank,
         plan.group_tokens, plan.ws.loss_part, plan.blocks, l_aux);
@@ -486,11 +660,12 @@ extern "C" int planmoe_forward_int8(const void *x, const void *wg, int dtype, in
                "planmoe_forward_int8: workspace too small");
     hipStream_t st = (hipStream_t)stream;
     FwdPlan plan;
+    fwd_plan(plan, workspace, samples, experts, top_k);
     if (run_gate_route(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
                        normalize_gate, indices, locations, gates, plane_stride, logits_out, scores_out,
-                       l_aux, expert_counts, workspace, st, plan)) return 1;
+                       l_aux, expert_counts, workspace, st, plan, !plan.merged)) return 1;
     if (run_dispatch_routed(x, dtype, samples, model_dim, experts, capacity, indices, locations,
-                            plane_stride, l_aux, codes, bias, scale, plan, st)) return 1;
+                            plane_stride, l_aux, expert_counts, codes, bias, scale, plan, st)) return 1;
     PM_LAUNCH_CHECK("planmoe_forward_int8");
     return 0;
 }
@@ -512,14 +687,9 @@ extern "C" int planmoe_forward_int8_redispatch(const void *x, int dtype, int sam
     PM_REQUIRE(model_dim % vec == 0 && aligned16(x) && (uintptr_t)codes % 8 == 0,
                "planmoe_forward_int8_redispatch: bad alignment");
     FwdPlan plan;
-    plan.k = top_k < experts ? top_k : experts;
-    plan.group_tokens = fwd_group_tokens(experts);
-    plan.groups = (samples + plan.group_tokens - 1) / plan.group_tokens;
-    plan.experts_per_block = go_experts_per_block(experts, plan.k);
-    plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
-    plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts, samples);
+    fwd_plan(plan, workspace, samples, experts, top_k);
     if (run_dispatch_routed(x, dtype, samples, model_dim, experts, capacity, indices, locations,
-                            plane_stride, nullptr, codes, bias, scale, plan, (hipStream_t)stream)) return 1;
+                            plane_stride, nullptr, nullptr, codes, bias, scale, plan, (hipStream_t)stream)) return 1;
     PM_LAUNCH_CHECK("planmoe_forward_int8_redispatch");
     return 0;
 }

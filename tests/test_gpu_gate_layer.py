@@ -200,7 +200,8 @@ def test_fused_forward_matches_unfused_and_oracle(T, M, E, k, cf, dtype, fp32_ga
         for name in ("indices", "locations", "counts"):
             assert torch.equal(r2[name], out[name])
         assert np.array_equal(raw(r2["gates"]), raw(out["gates"]))
-        assert abs(float(r2["l_aux"]) - float(out["l_aux"])) == 0
+        # the two entry points add the per-group shares of the loss up in different orders
+        assert abs(float(r2["l_aux"]) - float(out["l_aux"])) <= 1e-6 * abs(float(out["l_aux"]))
 
 
 @pytest.mark.parametrize("T,M,E,k", [(300, 776, 24, 2), (200, 264, 8, 2), (130, 1032, 64, 1)])
