@@ -178,12 +178,42 @@ template <> struct Elem<PLANMOE_F16> {
 // ---------------------------------------------------------------- wavefront helpers (wave64)
 __device__ __forceinline__ int lane_id() { return (int)(threadIdx.x & (WAVE - 1)); }
 
+// Partner exchange for reductions inside a row of 16 lanes with DPP modifiers (register-file
+// speed; a __shfl is an LDS round trip).  STEP 1, 2: lane ^ 1, lane ^ 2 (quad permutes);
+// STEP 4: lane <-> 7 - lane inside each group of 8; STEP 8: lane <-> 15 - lane inside the row.
+// After steps 1, 2, .., N / 2 every lane holds the reduction over its aligned group of N lanes,
+// provided the operation is commutative and associative.
+template <int STEP, typename T>
+__device__ __forceinline__ T row_partner(T v)
+{
+    static_assert(sizeof(T) == 4, "32-bit values");
+    constexpr int ctrl = STEP == 1 ? 0xB1 : STEP == 2 ? 0x4E : STEP == 4 ? 0x141 : 0x140;
+    const int x = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(x, x, ctrl, 0xf, 0xf, false));
+}
+
+// reduction over aligned groups of N <= 16 lanes, result in every lane of the group
+template <int N, typename T, typename Op>
+__device__ __forceinline__ T row_allreduce(T v, Op op)
+{
+    if constexpr (N >= 2) v = op(v, row_partner<1>(v));
+    if constexpr (N >= 4) v = op(v, row_partner<2>(v));
+    if constexpr (N >= 8) v = op(v, row_partner<4>(v));
+    if constexpr (N >= 16) v = op(v, row_partner<8>(v));
+    return v;
+}
+
 template <typename T, typename Op>
 __device__ __forceinline__ T wave_allreduce(T v, Op op)
 {
-#pragma unroll
-    for (int off = WAVE / 2; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, WAVE));
-    return v;
+    v = row_allreduce<16>(v, op);
+    // the four rows meet through scalar registers
+    const int x = __builtin_bit_cast(int, v);
+    const T r0 = __builtin_bit_cast(T, __builtin_amdgcn_readlane(x, 0));
+    const T r1 = __builtin_bit_cast(T, __builtin_amdgcn_readlane(x, 16));
+    const T r2 = __builtin_bit_cast(T, __builtin_amdgcn_readlane(x, 32));
+    const T r3 = __builtin_bit_cast(T, __builtin_amdgcn_readlane(x, 48));
+    return op(op(r0, r1), op(r2, r3));
 }
 
 __device__ __forceinline__ float wave_sum(float v)

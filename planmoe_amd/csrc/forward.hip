@@ -83,9 +83,7 @@ template <typename T, int N>
 __device__ __forceinline__ void wave_sum_n(T (&v)[N])
 {
 #pragma unroll
-    for (int off = WAVE / 2; off > 0; off >>= 1)
-#pragma unroll
-        for (int i = 0; i < N; ++i) v[i] += __shfl_xor(v[i], off, WAVE);
+    for (int i = 0; i < N; ++i) v[i] = wave_allreduce(v[i], [](T a, T b) { return a + b; });
 }
 
 __device__ __forceinline__ uint64_t lanes_below() { return ((uint64_t)1 << lane_id()) - 1; }
@@ -120,10 +118,129 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
     else gate_tile_lds<DT, NT, STATS>(x, wg, t0, samples, model_dim, experts, smem, pstat[0]);
     __syncthreads();
 
-    if (tid < WAVE) {                                  // wave 0: one lane per token of the group
+    // ---- routing epilogue, part 1: all four waves, wave w owns tokens [16 w, 16 w + 16).
+    // LPT lanes share a token, lane el holding the experts el, el + LPT, ...: softmax and the
+    // k-fold arg-max are butterflies over those lanes instead of loops over the experts.
+    constexpr int LPT = CAP < 16 ? CAP : 16;           // lanes per token
+    constexpr int EPL = CAP / LPT;                     // experts per lane
+    constexpr int TPP = WAVE / LPT;                    // tokens per pass of a wave
+    __shared__ uint8_t s_best[64][GROUP];              // [plane][token] chosen expert
+    __shared__ float s_me[4][CAP];
+    const int wave = tid >> 6, el = lane % LPT, tk = lane / LPT;
+    auto token_reduce = [&](auto v, auto op) { return row_allreduce<LPT>(v, op); };   // over the lanes of a token
+    float me_acc[EPL];
+#pragma unroll
+    for (int q = 0; q < EPL; ++q) me_acc[q] = 0.f;
+    const float eps = SDT == PLANMOE_F32 ? 1.1920928955078125e-07f
+                    : SDT == PLANMOE_BF16 ? 0.0078125f : 0.0009765625f;
+
+    for (int p = 0; p < 16 / TPP; ++p) {
+        const int tok = wave * 16 + p * TPP + tk;
+        const int t = t0 + tok;
+        const bool valid = t < samples;
+        float sc[EPL];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) {
+            const int e = q * LPT + el;
+            float v = -INFINITY;
+            if (e < experts) {
+                if constexpr (SPLITK) v = ((part[0][tok][e] + part[1][tok][e]) + part[2][tok][e]) + part[3][tok][e];
+                else v = part[0][tok][e];
+                v = S::round(v);
+                if (logits_out && valid) S::store(logits_out, (int64_t)t * experts + e, v);
+                if (logit_bias) v = S::round(v + logit_bias[e]);
+            }
+            sc[q] = v;
+            mx = fmaxf(mx, v);
+        }
+        mx = token_reduce(mx, [](float a, float b) { return fmaxf(a, b); });
+        float sum = 0.f;
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) {
+            sc[q] = (q * LPT + el < experts) ? expf(sc[q] - mx) : 0.f;
+            sum += sc[q];
+        }
+        sum = token_reduce(sum, [](float a, float b) { return a + b; });
+        const float inv = 1.0f / sum;                     // scores are tolerance-level quantities
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) {
+            const int e = q * LPT + el;
+            if (e < experts) {
+                sc[q] = S::round(sc[q] * inv);
+                if (scores_out && valid) S::store(scores_out, (int64_t)t * experts + e, sc[q]);
+            } else {
+                sc[q] = -INFINITY;
+            }
+        }
+        // column sums of the wave's scores (GShard loss): over the tokens of the pass, then passes
+        if (l_aux) {
+#pragma unroll
+            for (int q = 0; q < EPL; ++q) {
+                float c = (valid && q * LPT + el < experts) ? sc[q] : 0.f;
+#pragma unroll
+                for (int off = LPT; off < WAVE; off <<= 1) c += __shfl_xor(c, off, WAVE);
+                me_acc[q] += c;
+            }
+        }
+        // k-fold arg-max, the lower expert id wins among equal scores
+        uint32_t taken = 0;
+        float denom = 0.f, my_gate = 0.f;
+        int my_idx = 0;
+        for (int j = 0; j < k; ++j) {
+            float bv = -INFINITY; int bi = 0x7fffffff;
+#pragma unroll
+            for (int q = 0; q < EPL; ++q) {
+                const bool free_ = !((taken >> q) & 1u) && q * LPT + el < experts;
+                if (free_ && (bi == 0x7fffffff || sc[q] > bv)) { bv = sc[q]; bi = q * LPT + el; }
+            }
+            auto merge = [&](float ov, int oi) {
+                const bool better = oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi));
+                if (better) { bv = ov; bi = oi; }
+            };
+            if constexpr (LPT >= 2) merge(row_partner<1>(bv), row_partner<1>(bi));
+            if constexpr (LPT >= 4) merge(row_partner<2>(bv), row_partner<2>(bi));
+            if constexpr (LPT >= 8) merge(row_partner<4>(bv), row_partner<4>(bi));
+            if constexpr (LPT >= 16) merge(row_partner<8>(bv), row_partner<8>(bi));
+#pragma unroll
+            for (int q = 0; q < EPL; ++q) if (bi == q * LPT + el) taken |= 1u << q;
+            denom = (j == 0) ? bv : S::round(denom + bv);
+            if (el == 0) s_best[j][tok] = (uint8_t)bi;
+            if (j < LPT) {
+                if (el == j) { my_gate = bv; my_idx = bi; }
+            } else if (valid && el == j % LPT) {
+                // more planes than lanes per token: index and raw gate go out now, the gate is
+                // normalised below
+                indices[(int64_t)j * stride + t] = bi;
+                S::store(gates, (int64_t)j * stride + t, bv);
+            }
+        }
+        if (valid) {
+            const bool norm = k > 1 && normalize_gate;
+            const float d = fmaxf(denom, eps);
+            if (el < k) {
+                indices[(int64_t)el * stride + t] = my_idx;
+                S::store(gates, (int64_t)el * stride + t, norm ? my_gate / d : my_gate);
+            }
+            if (norm) {
+                for (int j = LPT + el; j < k; j += LPT) {
+                    const float g = S::load(gates, (int64_t)j * stride + t);
+                    S::store(gates, (int64_t)j * stride + t, g / d);
+                }
+            }
+        }
+    }
+    if (l_aux && tk == 0) {
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) if (q * LPT + el < experts) s_me[wave][q * LPT + el] = me_acc[q];
+    }
+    __syncthreads();
+
+    // ---- part 2: wave 0, one lane per token: rank of every token among the group's tokens with
+    // the same choice (wave ballots), the group's histograms, row min / max, score column sums
+    if (tid < WAVE) {
         const int t = t0 + tid;
-        const bool valid = tid < GROUP && t < samples;
-        float s[CAP];
+        const bool valid = t < samples;
         if constexpr (STATS) {
             if (valid) {
                 // row min / max for the int8 codec of the dispatch launch
@@ -139,81 +256,13 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
                 ws.row_min[t] = lo; ws.row_max[t] = hi;
             }
         }
-        if (valid) {
-            float mx = -INFINITY;
-#pragma unroll
-            for (int e = 0; e < CAP; ++e) {
-                float v = -INFINITY;
-                if (e < experts) {
-                    if constexpr (SPLITK) v = ((part[0][tid][e] + part[1][tid][e]) + part[2][tid][e]) + part[3][tid][e];
-                    else v = part[0][tid][e];
-                    v = S::round(v);
-                    if (logits_out) S::store(logits_out, (int64_t)t * experts + e, v);
-                    if (logit_bias) v = S::round(v + logit_bias[e]);
-                }
-                s[e] = v;
-                mx = fmaxf(mx, v);
-            }
-            float sum = 0.f;
-#pragma unroll
-            for (int e = 0; e < CAP; ++e) if (e < experts) { s[e] = expf(s[e] - mx); sum += s[e]; }
-            const float inv = 1.0f / sum;                 // scores are tolerance-level quantities
-#pragma unroll
-            for (int e = 0; e < CAP; ++e) {
-                if (e < experts) {
-                    s[e] = S::round(s[e] * inv);
-                    if (scores_out) S::store(scores_out, (int64_t)t * experts + e, s[e]);
-                }
-            }
+        if (l_aux && lane < experts) {
+            const float v = ((s_me[0][lane] + s_me[1][lane]) + s_me[2][lane]) + s_me[3][lane];
+            ws.me[(int64_t)blockIdx.x * experts + lane] = v;
+            ws.me_t[(int64_t)lane * ws.gstride + blockIdx.x] = v;
         }
-        // column sums of the group's scores (GShard loss)
-        if (l_aux) {
-            if constexpr (CAP <= 16) {
-#pragma unroll
-                for (int e = 0; e < CAP; ++e) {
-                    if (e < experts) {
-                        const float v = wave_sum(valid ? s[e] : 0.f);
-                        if (lane == 0) {
-                            ws.me[(int64_t)blockIdx.x * experts + e] = v;
-                            ws.me_t[(int64_t)e * ws.gstride + blockIdx.x] = v;
-                        }
-                    }
-                }
-            } else {
-                // many experts: every lane puts its token's scores back into its own tile row,
-                // then lane e adds up column e (the padded row length keeps the banks apart)
-#pragma unroll
-                for (int e = 0; e < CAP; ++e) if (e < experts) part[0][tid][e] = valid ? s[e] : 0.f;
-                __builtin_amdgcn_wave_barrier();
-                for (int e = lane; e < experts; e += WAVE) {
-                    float v = 0.f;
-#pragma unroll 8
-                    for (int r = 0; r < GROUP; ++r) v += part[0][r][e];
-                    ws.me[(int64_t)blockIdx.x * experts + e] = v;
-                    ws.me_t[(int64_t)e * ws.gstride + blockIdx.x] = v;
-                }
-            }
-        }
-        float denom = 0.f;
-        uint64_t taken = 0;
-        constexpr int KREG = 4;                          // raw gates of the first planes stay in registers
-        float gv[KREG] = {0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < k; ++j) {
-            int best = -1; float bv = -INFINITY;
-            if (valid) {
-#pragma unroll
-                for (int e = 0; e < CAP; ++e) {
-                    const bool free_ = !((taken >> e) & 1u) && e < experts;
-                    if (free_ && (best < 0 || s[e] > bv)) { best = e; bv = s[e]; }
-                }
-                taken |= (uint64_t)1 << best;
-                indices[(int64_t)j * stride + t] = best;
-#pragma unroll
-                for (int q = 0; q < KREG; ++q) if (q == j) gv[q] = bv;
-                if (j >= KREG || !(k > 1 && normalize_gate)) S::store(gates, (int64_t)j * stride + t, bv);
-                denom = (j == 0) ? bv : S::round(denom + bv);
-            }
-            __builtin_amdgcn_wave_barrier();
+            const int best = valid ? (int)s_best[j][tid] : -1;
             if (lane < CAP) s_hist[lane] = 0;
             __builtin_amdgcn_wave_barrier();
             int rank = 0;
@@ -235,21 +284,9 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
                 if ((int)blockIdx.x == groups - 1)             // the last group also clears the padding
                     for (int p = groups; p < ws.gstride; ++p) col[p] = 0;
             }
-        }
-        if (valid && k > 1 && normalize_gate) {
-            const float eps = SDT == PLANMOE_F32 ? 1.1920928955078125e-07f
-                            : SDT == PLANMOE_BF16 ? 0.0078125f : 0.0009765625f;
-            const float d = fmaxf(denom, eps);
-#pragma unroll
-            for (int j = 0; j < KREG; ++j)
-                if (j < k) S::store(gates, (int64_t)j * stride + t, gv[j] / d);
-            for (int j = KREG; j < k; ++j) {
-                const float g = S::load(gates, (int64_t)j * stride + t);
-                S::store(gates, (int64_t)j * stride + t, g / d);
-            }
+            __builtin_amdgcn_wave_barrier();
         }
     }
-
 }
 
 // locations += offset of the token's group (routing only, no dispatch)
