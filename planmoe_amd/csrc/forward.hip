@@ -266,14 +266,24 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
             if (lane < CAP) s_hist[lane] = 0;
             __builtin_amdgcn_wave_barrier();
             int rank = 0;
-            uint64_t todo = __ballot(valid);
-            while (todo) {
-                const int leader = __ffsll((unsigned long long)todo) - 1;
-                const int le = __builtin_amdgcn_readlane(best, leader);
-                const uint64_t m = __ballot(valid && best == le);
-                if (valid && best == le) rank = __popcll(m & lanes_below());
-                if (lane == leader) s_hist[le] = __popcll(m);
-                todo &= ~m;
+            if constexpr (CAP <= 16) {
+                // few experts: one ballot per expert, no serial dependence between them
+#pragma unroll
+                for (int e = 0; e < CAP; ++e) {
+                    const uint64_t m = __ballot(best == e);
+                    if (best == e) rank = __popcll(m & lanes_below());
+                    if (lane == e) s_hist[e] = __popcll(m);
+                }
+            } else {
+                uint64_t todo = __ballot(valid);
+                while (todo) {
+                    const int leader = __ffsll((unsigned long long)todo) - 1;
+                    const int le = __builtin_amdgcn_readlane(best, leader);
+                    const uint64_t m = __ballot(valid && best == le);
+                    if (valid && best == le) rank = __popcll(m & lanes_below());
+                    if (lane == leader) s_hist[le] = __popcll(m);
+                    todo &= ~m;
+                }
             }
             if (valid) ws.rank[(int64_t)j * samples + t] = rank;
             __builtin_amdgcn_wave_barrier();
