@@ -190,7 +190,8 @@ def main():
     wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16()
     xd, wd = x.to(dev), wg.to(dev)
 
-    # the whole chain is one C-ABI call (three launches) writing into buffers allocated once
+    # the whole chain is one C-ABI call (two launches: gate + routing, then dispatch + int8 with the
+    # prefix over the routing groups folded in) writing into buffers allocated once
     plan = ops.ForwardInt8Plan(xd, wd, k, C, fp32_gate=True)
 
     def chain():
@@ -219,7 +220,7 @@ def main():
     # dominant kernel alone (dispatch + int8 on the routing the chain produced)
     chain()
     stages = {}
-    stages["gate_route (gate GEMM + routing, 2 launches + offsets)"] = event_time_us(
+    stages["gate_route entry point (gate GEMM + routing; stand-alone it adds two small launches)"] = event_time_us(
         lambda: ops.gate_route(xd, wd, k, fp32_gate=True), 30, 5)
     stages["dispatch_int8_routed"] = event_time_us(plan.redispatch, 30, 5)
     chain_ev = event_time_us(chain, 30, 5)
@@ -242,7 +243,7 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS,
                      # HBM bytes per launch read from rocprofv3 FETCH_SIZE (x 2.0, the factor a device
                      # copy of known size shows for that counter) + WRITE_SIZE; see profiles/
-                     "traffic": 306.0e6,
+                     "traffic": 307.0e6,
                      "kernel": "dispatch_int8_routed_kernel (last launch of the chain, timed alone)",
                      "algorithmic_bytes": dom_bytes, "avg_us": dom_avg_us},
         "chain": {"algorithmic_bytes": chain_bytes, "device_us_avg": chain_ev[0], "device_us_min": chain_ev[2],
