@@ -26,8 +26,14 @@
 namespace pm {
 
 // tokens per work-group of the gate kernel = tokens per routing group (one lane each in the
-// routing epilogue)
-__host__ __device__ inline int fwd_group_tokens(int) { return 64; }
+// routing epilogue): 64, or 32 on the split-K path (up to 16 experts) when 64 would leave
+// compute units without a work-group
+inline int fwd_group_tokens(int experts, int samples)
+{
+    // measured at 8 experts: 16384 tokens (256 groups of 64) 39 us with 64, 44 us with 32;
+    // 8192 tokens 32 us with 64, 28 us with 32
+    return (experts <= 16 && samples < 64 * 256) ? 32 : 64;
+}
 constexpr int FWD_LOSS_PARTS = 64;
 
 // hist_t / me_t are the transposes of hist / me with the group index running fastest (rows of
@@ -92,7 +98,7 @@ __device__ __forceinline__ uint64_t lanes_below() { return ((uint64_t)1 << lane_
 // CAP: compile-time bound of the expert count held in registers by the routing epilogue
 // NT == 1: split-K over the 4 waves, weights straight from L2 (up to 16 experts);
 // NT > 1: weights shared through LDS, a wave per 16 tokens.
-template <int DT, int SDT, int NT, int CAP, bool SPLITK>
+template <int DT, int SDT, int NT, int CAP, bool SPLITK, int GROUP>
 __global__ __launch_bounds__(256) void gate_route_kernel(
     const void *__restrict__ x, const void *__restrict__ wg, const float *__restrict__ logit_bias,
     int samples, int model_dim, int experts, int k, int normalize_gate,
@@ -101,7 +107,7 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
     float *__restrict__ l_aux, int32_t *__restrict__ counts_out, void *__restrict__ workspace)
 {
     using S = Elem<SDT>;
-    constexpr int GROUP = 64;
+    static_assert(GROUP == 64 || (SPLITK && GROUP == 32), "the LDS-shared variant is built for 64 tokens");
     constexpr int COLS = 16 * NT + 1;
     // split-K: part[4][GROUP][COLS] floats; else the weight buffers / logits[GROUP][COLS]
     __shared__ uint4 smem[SPLITK ? (4 * GROUP * COLS + 3) / 4 : gate_lds_vectors<NT>()];
@@ -114,16 +120,17 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
     const int t0 = blockIdx.x * GROUP;
     constexpr bool STATS = DT == PLANMOE_BF16;
     __shared__ int32_t pstat[SPLITK ? 4 : 1][GROUP][3];
-    if constexpr (SPLITK) gate_tile_partials<DT, NT, 4, 4, STATS>(x, wg, t0, samples, model_dim, experts, part, pstat);
+    if constexpr (SPLITK) gate_tile_partials<DT, NT, GROUP / 16, 4, STATS>(x, wg, t0, samples, model_dim, experts, part, pstat);
     else gate_tile_lds<DT, NT, STATS>(x, wg, t0, samples, model_dim, experts, smem, pstat[0]);
     __syncthreads();
 
-    // ---- routing epilogue, part 1: all four waves, wave w owns tokens [16 w, 16 w + 16).
+    // ---- routing epilogue, part 1: all four waves, wave w owns GROUP / 4 consecutive tokens.
     // LPT lanes share a token, lane el holding the experts el, el + LPT, ...: softmax and the
     // k-fold arg-max are butterflies over those lanes instead of loops over the experts.
     constexpr int LPT = CAP < 16 ? CAP : 16;           // lanes per token
     constexpr int EPL = CAP / LPT;                     // experts per lane
-    constexpr int TPP = WAVE / LPT;                    // tokens per pass of a wave
+    constexpr int TPW4 = GROUP / 4;                    // tokens per wave
+    constexpr int TPP = WAVE / LPT < TPW4 ? WAVE / LPT : TPW4;   // tokens per pass of a wave
     __shared__ uint8_t s_best[64][GROUP];              // [plane][token] chosen expert
     __shared__ float s_me[4][CAP];
     const int wave = tid >> 6, el = lane % LPT, tk = lane / LPT;
@@ -134,10 +141,10 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
     const float eps = SDT == PLANMOE_F32 ? 1.1920928955078125e-07f
                     : SDT == PLANMOE_BF16 ? 0.0078125f : 0.0009765625f;
 
-    for (int p = 0; p < 16 / TPP; ++p) {
-        const int tok = wave * 16 + p * TPP + tk;
+    for (int p = 0; p < TPW4 / TPP; ++p) {
+        const int tok = wave * TPW4 + p * TPP + min(tk, TPP - 1);   // lanes past the pass repeat a token
         const int t = t0 + tok;
-        const bool valid = t < samples;
+        const bool valid = t < samples && tk < TPP;
         float sc[EPL];
         float mx = -INFINITY;
 #pragma unroll
@@ -179,7 +186,7 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
             for (int q = 0; q < EPL; ++q) {
                 float c = (valid && q * LPT + el < experts) ? sc[q] : 0.f;
 #pragma unroll
-                for (int off = LPT; off < WAVE; off <<= 1) c += __shfl_xor(c, off, WAVE);
+                for (int off = LPT; off < WAVE; off <<= 1) c += __shfl_xor(c, off, WAVE);   // lanes past the pass hold 0
                 me_acc[q] += c;
             }
         }
@@ -205,7 +212,7 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
 #pragma unroll
             for (int q = 0; q < EPL; ++q) if (bi == q * LPT + el) taken |= 1u << q;
             denom = (j == 0) ? bv : S::round(denom + bv);
-            if (el == 0) s_best[j][tok] = (uint8_t)bi;
+            if (el == 0 && tk < TPP) s_best[j][tok] = (uint8_t)bi;
             if (j < LPT) {
                 if (el == j) { my_gate = bv; my_idx = bi; }
             } else if (valid && el == j % LPT) {
@@ -240,7 +247,7 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
     // the same choice (wave ballots), the group's histograms, row min / max, score column sums
     if (tid < WAVE) {
         const int t = t0 + tid;
-        const bool valid = t < samples;
+        const bool valid = tid < GROUP && t < samples;
         if constexpr (STATS) {
             if (valid) {
                 // row min / max for the int8 codec of the dispatch launch
@@ -262,7 +269,7 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
             ws.me_t[(int64_t)lane * ws.gstride + blockIdx.x] = v;
         }
         for (int j = 0; j < k; ++j) {
-            const int best = valid ? (int)s_best[j][tid] : -1;
+            const int best = valid ? (int)s_best[j][tid % GROUP] : -1;
             if (lane < CAP) s_hist[lane] = 0;
             __builtin_amdgcn_wave_barrier();
             int rank = 0;
@@ -520,14 +527,16 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
 }
 
 template <int DT, int SDT>
-static void launch_gate_route(int experts, int groups, hipStream_t st, const void *x, const void *wg,
+static void launch_gate_route(int experts, int groups, int group_tokens, hipStream_t st, const void *x, const void *wg,
                               const float *bias, int samples, int model_dim, int k, int normalize,
                               int32_t *indices, int32_t *locations, void *gates, int64_t stride,
                               void *logits_out, void *scores_out, float *l_aux, int32_t *counts, void *ws)
 {
-#define PM_GR(NT, CAP, SPLITK)                                                                           \
-    gate_route_kernel<DT, SDT, NT, CAP, SPLITK><<<groups, 256, 0, st>>>(x, wg, bias, samples, model_dim, experts, \
+#define PM_GR_(NT, CAP, SPLITK, GROUP)                                                                   \
+    gate_route_kernel<DT, SDT, NT, CAP, SPLITK, GROUP><<<groups, 256, 0, st>>>(x, wg, bias, samples, model_dim, experts, \
         k, normalize, indices, locations, gates, stride, logits_out, scores_out, l_aux, counts, ws)
+#define PM_GR(NT, CAP, SPLITK) do { if (SPLITK && group_tokens == 32) PM_GR_(NT, CAP, SPLITK, (SPLITK ? 32 : 64)); \
+                                    else PM_GR_(NT, CAP, SPLITK, 64); } while (0)
     // split-K measured faster than the LDS-shared variant up to 16 experts (30.7 vs 44.4 us at
     // 16384 x 4096 bf16, 8 experts), and the other way round above (168 -> 48 us at 64 experts)
     if (experts <= 8) PM_GR(1, 8, true);
@@ -535,6 +544,7 @@ static void launch_gate_route(int experts, int groups, hipStream_t st, const voi
     else if (experts <= 32) PM_GR(2, 32, false);
     else PM_GR(4, 64, false);
 #undef PM_GR
+#undef PM_GR_
 }
 
 template <int DT>
@@ -586,7 +596,7 @@ struct FwdPlan {
 static void fwd_plan(FwdPlan &plan, void *workspace, int samples, int experts, int top_k)
 {
     plan.k = top_k < experts ? top_k : experts;
-    plan.group_tokens = fwd_group_tokens(experts);
+    plan.group_tokens = fwd_group_tokens(experts, samples);
     plan.groups = (samples + plan.group_tokens - 1) / plan.group_tokens;
     plan.experts_per_block = go_experts_per_block(experts, plan.k);
     plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
@@ -606,14 +616,14 @@ static int run_gate_route(const void *x, const void *wg, int dtype, int fp32_gat
     const int k = plan.k, groups = plan.groups;
     if (fp32_gate || dtype == PLANMOE_F32) {
         PM_DTYPE_SWITCH(dtype, DT, (launch_gate_route<DT, PLANMOE_F32>(
-            experts, groups, st, x, wg, logit_bias, samples, model_dim, k, normalize_gate, indices,
+            experts, groups, plan.group_tokens, st, x, wg, logit_bias, samples, model_dim, k, normalize_gate, indices,
             locations, gates, stride, logits_out, scores_out, l_aux, counts, workspace)));
     } else if (dtype == PLANMOE_BF16) {
-        launch_gate_route<PLANMOE_BF16, PLANMOE_BF16>(experts, groups, st, x, wg, logit_bias, samples,
+        launch_gate_route<PLANMOE_BF16, PLANMOE_BF16>(experts, groups, plan.group_tokens, st, x, wg, logit_bias, samples,
             model_dim, k, normalize_gate, indices, locations, gates, stride, logits_out, scores_out,
             l_aux, counts, workspace);
     } else {
-        launch_gate_route<PLANMOE_F16, PLANMOE_F16>(experts, groups, st, x, wg, logit_bias, samples,
+        launch_gate_route<PLANMOE_F16, PLANMOE_F16>(experts, groups, plan.group_tokens, st, x, wg, logit_bias, samples,
             model_dim, k, normalize_gate, indices, locations, gates, stride, logits_out, scores_out,
             l_aux, counts, workspace);
     }
