@@ -89,6 +89,23 @@ int planmoe_route_topk(const void *input, int dtype, int input_is_logits, const 
                        void *scores_out, float *l_aux, int32_t *expert_counts,
                        void *workspace, size_t workspace_bytes, void *stream);
 
+/* Slot locations for routing decisions that already exist, with the tokens taking their slots in
+ * a given order: compute_sorted_location of batch-prioritised routing (fast_dispatch.py:135-138,
+ * 152-154), and with order == NULL the plain fast_cumsum_sub_one path (:156-168).
+ *   indices       int32 top_k planes (base + j*plane_stride); an index outside [0, experts)
+ *                 takes no slot and gets location -1
+ *   order         optional int32 [samples]: order[p] = token that is p-th to be served (a
+ *                 permutation, e.g. the stable argsort of -max score); NULL = 0, 1, 2, ...
+ *   locations     out int32 planes: all first choices of an expert before all its second
+ *                 choices, inside a plane the served order
+ *   expert_counts optional out int32 [top_k, experts]
+ *   workspace     planmoe_route_workspace_bytes(samples, experts, top_k) bytes
+ * top_k is NOT clamped here: it is the number of planes present. */
+int planmoe_route_locations(const int32_t *indices, int64_t plane_stride, int samples, int experts,
+                            int top_k, const int32_t *order, int32_t *locations,
+                            int32_t *expert_counts, void *workspace, size_t workspace_bytes,
+                            void *stream);
+
 /* Backward of planmoe_route_topk with respect to its input: what autograd derives from the
  * tensor algebra of extract_critical (fast_dispatch.py:148, 170-172: gates are score entries,
  * divided by their clamped sum) and of gshard_loss (losses.py:12-19: me depends on the scores,

@@ -139,6 +139,18 @@ def route_topk(scores, top_k, normalize_gate=True):
     return idx, loc, gates, counts
 
 
+def route_locations(indices, experts, order=None):
+    """indices int32 [k,T]; order int32 [T] or None.  Returns locations[k,T], counts[k,E]."""
+    indices = _c(indices, np.int32)
+    k, T = indices.shape
+    loc = np.empty((k, T), np.int32)
+    counts = np.empty((k, experts), np.int32)
+    o = _c(order, np.int32) if order is not None else None
+    lib().orc_route_locations(_p(indices), ctypes.c_int(T), ctypes.c_int(experts), ctypes.c_int(k),
+                              _p(o) if o is not None else None, _p(loc), _p(counts))
+    return loc, counts
+
+
 def gshard_loss(scores, first_choice):
     is_bf16 = scores.dtype == np.uint16
     scores = np.ascontiguousarray(scores)

@@ -151,6 +151,31 @@ static inline float load_score(const void *scores, int is_bf16, int64_t i)
     return is_bf16 ? bf16_to_f32(((const uint16_t *)scores)[i]) : ((const float *)scores)[i];
 }
 
+/* Locations of existing routing decisions with the tokens served in a given order
+ * (compute_sorted_location, fast_dispatch.py:135-138, applied plane by plane as in :156-168):
+ * location of (plane j, token t) = entries of expert e in planes < j  +  tokens served before t
+ * in plane j with the same expert.  order == NULL: token order.  Indices outside [0, experts)
+ * take no slot (location -1). */
+ORC_API void orc_route_locations(const int32_t *indices, int samples, int experts, int k,
+                                 const int32_t *order, int32_t *locations, int32_t *counts)
+{
+    int64_t *base = (int64_t *)calloc((size_t)experts, sizeof(int64_t));
+    int64_t *seen = (int64_t *)malloc(sizeof(int64_t) * (size_t)experts);
+    memset(counts, 0, sizeof(int32_t) * (size_t)k * experts);
+    for (int j = 0; j < k; ++j) {
+        memset(seen, 0, sizeof(int64_t) * (size_t)experts);
+        for (int p = 0; p < samples; ++p) {
+            int t = order ? order[p] : p;
+            int e = indices[(size_t)j * samples + t];
+            if (e < 0 || e >= experts) { locations[(size_t)j * samples + t] = -1; continue; }
+            locations[(size_t)j * samples + t] = (int32_t)(base[e] + seen[e]);
+            seen[e] += 1;
+        }
+        for (int e = 0; e < experts; ++e) { counts[(size_t)j * experts + e] = (int32_t)seen[e]; base[e] += seen[e]; }
+    }
+    free(base); free(seen);
+}
+
 ORC_API void orc_route_topk(const void *scores, int is_bf16, int samples, int experts, int top_k,
                             int normalize_gate, int32_t *indices, int32_t *locations,
                             void *gates, int32_t *counts)

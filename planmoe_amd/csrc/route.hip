@@ -217,18 +217,64 @@ __global__ __launch_bounds__(TILE) void route_tile_kernel(
     }
 }
 
+// Locations for routing decisions that already exist, with the tokens visited in a given order
+// (batch-prioritised routing, fast_dispatch.py:135-138, 152-154: tokens sorted by importance take
+// their slots first).  Thread p of a tile handles the token order[p] (or p): rank among the
+// tile's tokens with the same choice + per-tile histograms, as in route_tile_kernel.
+__global__ __launch_bounds__(TILE) void locate_tile_kernel(
+    const int32_t *__restrict__ indices, const int32_t *__restrict__ order, int32_t *__restrict__ locations,
+    int64_t stride, int samples, int experts, int k, int32_t *__restrict__ hist)
+{
+    extern __shared__ int32_t wave_cnt[];           // [4][experts]
+    const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
+    const int p = blockIdx.x * TILE + tid;
+    const bool valid = p < samples;
+    const int t = valid ? (order ? order[p] : p) : 0;
+    for (int j = 0; j < k; ++j) {
+        int best = valid ? indices[(int64_t)j * stride + t] : -1;
+        const bool live = valid && best >= 0 && best < experts;     // anything else takes no slot
+        for (int e = tid; e < 4 * experts; e += TILE) wave_cnt[e] = 0;
+        __syncthreads();
+        int rank = 0;
+        uint64_t todo = __ballot(live);
+        while (todo) {
+            const int leader = __ffsll((unsigned long long)todo) - 1;
+            const int le = __builtin_amdgcn_readlane(best, leader);
+            const uint64_t m = __ballot(live && best == le);
+            if (live && best == le) rank = __popcll(m & lanemask_lt());
+            if (lane == leader) wave_cnt[wave * experts + le] = __popcll(m);
+            todo &= ~m;
+        }
+        __syncthreads();
+        if (live) {
+            int before = 0;
+            for (int w = 0; w < wave; ++w) before += wave_cnt[w * experts + best];
+            locations[(int64_t)j * stride + t] = rank + before;
+        } else if (valid) {
+            locations[(int64_t)j * stride + t] = -1;
+        }
+        for (int e = tid; e < experts; e += TILE)
+            hist[((int64_t)blockIdx.x * k + j) * experts + e] =
+                wave_cnt[e] + wave_cnt[experts + e] + wave_cnt[2 * experts + e] + wave_cnt[3 * experts + e];
+        __syncthreads();
+    }
+}
+
 // location = rank in tile + offset of the tile; one thread of the launch finishes the loss
 __global__ __launch_bounds__(TILE) void route_finish_kernel(
     const int32_t *__restrict__ indices, int32_t *__restrict__ locations, int64_t stride,
     int samples, int experts, int k, const int32_t *__restrict__ offs,
-    const float *__restrict__ loss_part, int loss_parts, float *__restrict__ l_aux)
+    const float *__restrict__ loss_part, int loss_parts, float *__restrict__ l_aux,
+    const int32_t *__restrict__ order)
 {
     finish_loss(loss_part, loss_parts, samples, l_aux);
-    const int t = blockIdx.x * TILE + threadIdx.x;
-    if (t >= samples) return;
+    const int p = blockIdx.x * TILE + threadIdx.x;
+    if (p >= samples) return;
+    const int t = order ? order[p] : p;
     for (int j = 0; j < k; ++j) {
         const int64_t o = (int64_t)j * stride + t;
-        locations[o] += offs[((int64_t)blockIdx.x * k + j) * experts + indices[o]];
+        const int e = indices[o];
+        if (e >= 0 && e < experts) locations[o] += offs[((int64_t)blockIdx.x * k + j) * experts + e];
     }
 }
 
@@ -462,7 +508,38 @@ extern "C" int planmoe_route_topk(const void *input, int dtype, int input_is_log
     group_offsets_kernel<<<blocks, 256, 0, st>>>(hist, offs, me, tiles, k, experts, epb, samples, nullptr,
                                                  expert_counts, loss_part, l_aux != nullptr);
     route_finish_kernel<<<tiles, TILE, 0, st>>>(indices, locations, plane_stride, samples, experts, k, offs,
-                                               loss_part, blocks, l_aux);
+                                               loss_part, blocks, l_aux, nullptr);
     PM_LAUNCH_CHECK("planmoe_route_topk");
+    return 0;
+}
+
+extern "C" int planmoe_route_locations(const int32_t *indices, int64_t plane_stride, int samples,
+                                       int experts, int top_k, const int32_t *order,
+                                       int32_t *locations, int32_t *expert_counts, void *workspace,
+                                       size_t workspace_bytes, void *stream)
+{
+    PM_REQUIRE(samples >= 0 && experts >= 1 && top_k >= 1, "planmoe_route_locations: bad shape");
+    PM_REQUIRE(experts <= ROUTE_MAX_E, "planmoe_route_locations: experts %d > supported %d", experts, ROUTE_MAX_E);
+    PM_REQUIRE(plane_stride >= samples, "planmoe_route_locations: plane_stride < samples");
+    hipStream_t st = (hipStream_t)stream;
+    if (samples == 0) {
+        if (expert_counts) fill_u32((uint32_t *)expert_counts, (size_t)top_k * experts, 0u, st);
+        return 0;
+    }
+    PM_REQUIRE(indices && locations, "planmoe_route_locations: NULL argument");
+    PM_REQUIRE(workspace && workspace_bytes >= planmoe_route_workspace_bytes(samples, experts, top_k),
+               "planmoe_route_locations: workspace too small");
+    const int k = top_k;
+    const int tiles = (int)route_tiles(samples);
+    int32_t *hist = (int32_t *)workspace;
+    int32_t *offs = hist + (size_t)tiles * k * experts;
+    locate_tile_kernel<<<tiles, TILE, sizeof(int32_t) * 4 * (size_t)experts, st>>>(
+        indices, order, locations, plane_stride, samples, experts, k, hist);
+    const int epb = go_experts_per_block(experts, k);
+    group_offsets_kernel<<<(experts + epb - 1) / epb, 256, 0, st>>>(hist, offs, nullptr, tiles, k, experts, epb,
+                                                                   samples, nullptr, expert_counts, nullptr, 0);
+    route_finish_kernel<<<tiles, TILE, 0, st>>>(indices, locations, plane_stride, samples, experts, k, offs,
+                                               nullptr, 0, nullptr, order);
+    PM_LAUNCH_CHECK("planmoe_route_locations");
     return 0;
 }

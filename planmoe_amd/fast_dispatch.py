@@ -141,15 +141,19 @@ def extract_critical(scores, top_k, loss_fn=losses.gshard_loss, capacity_factor=
     """fast_dispatch.py:140-195.  Returns ((E, indices_s, locations_s, gates_s, capacity), l_loss).
     gates_s and the GShard l_loss carry gradients back into `scores`.
 
-    Not carried over: batch_prioritized_routing=True (raises)."""
-    if batch_prioritized_routing:
-        raise NotImplementedError("extract_critical: batch_prioritized_routing is not built yet")
+    batch_prioritized_routing (fast_dispatch.py:135-138, 152-154): tokens take their slots in
+    the order of their largest score, highest first.  The reference sorts with an unstable
+    argsort; here tokens with equal importance keep their token order."""
     if not scores.is_cuda:
         raise PlanMoEError("extract_critical: scores must live on the GPU (no CPU path in this build)")
     num_global_experts = int(scores.size(1))
     top_k = min(top_k, num_global_experts)
     want_kernel_loss = loss_fn is losses.gshard_loss
     gates, l_aux, indices, locations, _ = route(scores, top_k, False, normalize_gate, want_kernel_loss)
+    if batch_prioritized_routing:
+        importance_scores = -1 * scores.detach().max(dim=1)[0]
+        order = torch.argsort(importance_scores, dim=0, stable=True).to(torch.int32)
+        locations, _ = ops.route_locations(indices, num_global_experts, order)
     indices_s = [indices[j] for j in range(top_k)]
     locations_s = [locations[j] for j in range(top_k)]
     gates_s = [gates[j] for j in range(top_k)]

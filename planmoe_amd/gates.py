@@ -1,4 +1,6 @@
-"""Linear top-k gate -- mirror of the reference's gates/top.py."""
+"""Gates: the linear top-k gate (gates/top.py) and the cosine gate (gates/cosine_top.py)."""
+import math
+
 import torch
 
 from . import ops
@@ -48,4 +50,36 @@ class LinearTopKGate(torch.nn.Module):
                                  torch.float32 if self.fp32_gate else x.dtype)
 
 
+
+class CosineTopKGate(torch.nn.Module):
+    # gates/cosine_top.py:7-33
+    def __init__(self, model_dim, num_global_experts, k=1, fp32_gate=False, proj_dim=256, init_t=0.5, **options):
+        super().__init__()
+        self.top_k = min(num_global_experts, int(k))
+        self.fp32_gate = fp32_gate
+        self.temperature = torch.nn.Parameter(torch.log(torch.full([1], 1.0 / init_t)), requires_grad=True)
+        self.cosine_projector = torch.nn.Linear(model_dim, proj_dim)
+        self.sim_matrix = torch.nn.Parameter(torch.randn(size=(proj_dim, num_global_experts)), requires_grad=True)
+        torch.nn.init.normal_(self.sim_matrix, 0, 0.01)
+        for opt in options:
+            if opt not in ('capacity_factor', 'gate_noise'):
+                raise Exception('Unrecognized argument provided to Gating module: %s' % opt)
+
+    def forward(self, x):
+        """Cosine similarity of the projected tokens with one vector per expert, scaled by a
+        learnt temperature capped at 1 / 0.01.  The similarity product has the shape of the
+        gate-logits GEMM ([T, proj_dim] x [E, proj_dim]^T) and runs through the same kernel."""
+        w, b, sim = self.cosine_projector.weight, self.cosine_projector.bias, self.sim_matrix
+        if self.fp32_gate:
+            x, w, b, sim = x.float(), w.float(), b.float(), sim.float()
+        elif x.dtype != w.dtype:
+            w, b, sim = w.to(x.dtype), b.to(x.dtype), sim.to(x.dtype)
+        proj = torch.nn.functional.normalize(torch.nn.functional.linear(x, w, b), dim=1)
+        experts = torch.nn.functional.normalize(sim, dim=0).t()
+        logits = _GateLogits.apply(proj.contiguous(), experts.contiguous(), proj.dtype)
+        logit_scale = torch.clamp(self.temperature, max=math.log(1. / 0.01)).exp()
+        return logits * logit_scale.to(logits.dtype)
+
+
 Gate = LinearTopKGate
+GATES = {'top': LinearTopKGate, 'cosine_top': CosineTopKGate}

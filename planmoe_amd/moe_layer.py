@@ -102,10 +102,10 @@ class MOELayer(torch.nn.Module):
                 "Gate type must only include digits, letters and underline characters."
             if seeds is not None and seeds[0] is not None:
                 torch.manual_seed(seeds[0] + gi)
-            if gate_name != 'top':
+            if gate_name not in _gates.GATES:
                 raise Exception("Unrecognized gate_type: %s" % gate_name)
-            gate_module = _gates.Gate(model_dim=self.model_dim, num_global_experts=self.num_global_experts,
-                                      **single_gate_type)
+            gate_module = _gates.GATES[gate_name](model_dim=self.model_dim, num_global_experts=self.num_global_experts,
+                                                  **single_gate_type)
             if not hasattr(gate_module, 'gate_noise'):
                 gate_module.gate_noise = single_gate_type.get('gate_noise', 0.0)
             if not hasattr(gate_module, 'capacity_factor'):

@@ -116,6 +116,28 @@ def route_topk(inp, top_k, is_logits=False, logit_bias=None, normalize_gate=True
     return dict(indices=idx, locations=loc, gates=gates, scores=scores, l_aux=l_aux, counts=counts)
 
 
+def route_locations(indices, experts, order=None, want_counts=False):
+    """Slot locations for existing routing decisions: indices int32 [k, T]; order int32 [T] =
+    token served p-th (batch-prioritised routing), None = token order.
+    Returns (locations [k, T] int32, counts [k, E] int32 | None)."""
+    _need_gpu(indices, "route_locations")
+    if indices.dtype != torch.int32 or indices.dim() != 2:
+        raise PlanMoEError("route_locations: indices must be int32 [top_k, samples]")
+    indices = _contig(indices, "route_locations")
+    k, T = indices.shape
+    dev = indices.device
+    if order is not None:
+        if order.numel() != T:
+            raise PlanMoEError("route_locations: order must hold one entry per token")
+        order = order.to(device=dev, dtype=torch.int32).contiguous()
+    loc = torch.empty((k, T), dtype=torch.int32, device=dev)
+    counts = torch.empty((k, int(experts)), dtype=torch.int32, device=dev) if want_counts else None
+    ws = _ws(lib.planmoe_route_workspace_bytes(T, int(experts), k), dev)
+    check(lib.planmoe_route_locations(_ptr(indices), max(T, 1), T, int(experts), k, _ptr(order), _ptr(loc),
+                                      _ptr(counts), _ptr(ws), ws.numel(), _stream(indices)))
+    return loc, counts
+
+
 def route_bwd(scores, indices, grad_gates, normalize_gate=True, grad_l_aux=None, counts=None,
               through_softmax=False):
     """Gradient of route_topk's gates (and l_aux) with respect to the scores [T, E] (or the

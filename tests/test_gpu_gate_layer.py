@@ -222,3 +222,27 @@ def test_fused_forward_rows_of_one_sign(T, M, E, k):
     assert np.array_equal(raw(out["bias"]), raw(b2)) and np.array_equal(raw(out["scale"]), raw(s2))
     rc, rb, rs = oracle.int8_compress(bf16_bits(ops.dispatch_fwd(x, list(out["indices"]), list(out["locations"]), None, E, C).cpu()))
     assert np.array_equal(c2.cpu().numpy().reshape(rc.shape), rc)
+
+
+def test_cosine_gate_logits_and_layer():
+    """CosineTopKGate against the reference's formula in fp32 torch ops (rtol 1e-5 of the logit
+    scale), then a moe_layer with that gate and batch-prioritised routing trains one step."""
+    import planmoe_amd
+    from planmoe_amd.gates import CosineTopKGate
+    torch.manual_seed(0)
+    gate = CosineTopKGate(96, 12, k=2, fp32_gate=True, proj_dim=64).to(DEV)
+    x = torch.randn(300, 96, device=DEV)
+    got = gate(x)
+    proj = torch.nn.functional.normalize(gate.cosine_projector(x), dim=1)
+    want = (proj @ torch.nn.functional.normalize(gate.sim_matrix, dim=0)) * gate.temperature.exp()
+    assert got.shape == (300, 12) and torch.allclose(got, want, rtol=1e-5, atol=1e-5 * float(gate.temperature.detach().exp()))
+
+    layer = planmoe_amd.moe_layer({'type': 'cosine_top', 'k': 2, 'fp32_gate': True, 'proj_dim': 32}, 64,
+                                  experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 128},
+                                  seeds=(1, 2, 3), compress_name='no', batch_prioritized_routing=True).to(DEV)
+    xin = torch.randn(8, 32, 64, device=DEV, requires_grad=True)
+    y = layer(xin)
+    (y.float().pow(2).mean() + y.l_aux).backward()
+    assert torch.isfinite(xin.grad).all()
+    g = layer.gates[0].sim_matrix.grad
+    assert g is not None and torch.isfinite(g).all() and g.abs().sum() > 0

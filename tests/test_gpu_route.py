@@ -187,3 +187,48 @@ def test_routing_gradients_through_the_fused_softmax():
     ref_g, ref_l = _torch_routing_reference(s64, indices.cpu().numpy(), True, T, E)
     (sum((ref_g[j] * w[j].double()).sum() for j in range(k)) + 2.0 * ref_l).backward()
     assert torch.allclose(l_dev.grad.cpu().double(), l64.grad, rtol=1e-4, atol=1e-7)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,E,k,with_order", [(1000, 8, 2, True), (1000, 8, 2, False), (4097, 64, 1, True),
+                                              (300, 100, 4, True), (77, 3, 3, True), (20000, 16, 2, True)])
+def test_route_locations(T, E, k, with_order):
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(T + E + k)
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)], dim=1).to(torch.int32).contiguous()
+    idx[0, ::17] = -1                                   # dead pairs take no slot
+    idx[k - 1, 5::31] = E + 3
+    order = torch.randperm(T, generator=g).to(torch.int32) if with_order else None
+    loc, counts = ops.route_locations(idx.to(DEV), E, None if order is None else order.to(DEV), want_counts=True)
+    want, wc = oracle.route_locations(idx.numpy(), E, None if order is None else order.numpy())
+    assert np.array_equal(loc.cpu().numpy(), want)
+    assert np.array_equal(counts.cpu().numpy(), wc)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,E,k", [(2048, 8, 2), (555, 16, 1), (16384, 8, 2)])
+def test_batch_prioritized_routing(T, E, k):
+    """extract_critical(batch_prioritized_routing=True): tokens with the larger top score get the
+    lower slots; same indices, gates and loss as without."""
+    import planmoe_amd as moe
+    scores = tie_free_scores(T, E, k, seed=T)
+    sd = scores.to(DEV)
+    (n, idx_s, loc_s, gates_s, cap), l = moe.extract_critical(sd, k, capacity_factor=1.0, batch_prioritized_routing=True)
+    (_, idx0, loc0, gates0, cap0), l0 = moe.extract_critical(sd, k, capacity_factor=1.0)
+    assert cap == cap0 and float(l) == float(l0)
+    for a, b in zip(idx_s, idx0):
+        assert torch.equal(a, b)
+    for a, b in zip(gates_s, gates0):
+        assert torch.equal(a, b)
+    idx = torch.stack(idx_s).cpu().numpy()
+    order = torch.argsort(-scores.max(dim=1)[0], stable=True).numpy().astype(np.int32)
+    want, _ = oracle.route_locations(idx, E, order)
+    got = torch.stack(loc_s).cpu().numpy()
+    assert np.array_equal(got, want)
+    # dropped tokens (location >= capacity) of an expert are its least important ones
+    top = scores.max(dim=1)[0].numpy()
+    for e in range(E):
+        m = idx[0] == e
+        kept, dropped = top[m & (got[0] < cap)], top[m & (got[0] >= cap)]
+        if len(kept) and len(dropped):
+            assert kept.min() >= dropped.max()

@@ -110,3 +110,54 @@ def test_softmax_and_logits_against_torch():
     assert np.allclose(lgb, (xb.double() @ wb.double().t()).numpy(), rtol=1e-12, atol=1e-12)
     sm = oracle.softmax(lg.astype(np.float32))
     assert np.allclose(sm, torch.softmax(torch.from_numpy(lg.astype(np.float32)), 1).numpy(), rtol=1e-6)
+
+
+def _torch_bpr_locations(scores, k):
+    """The reference's tensor algebra for batch-prioritised routing (fast_dispatch.py:135-138,
+    142-168) with torch ops, fast_cumsum_sub_one spelled as cumsum - 1."""
+    T, E = scores.shape
+    topk_indices = torch.topk(scores, k, dim=1).indices
+    indices_s = [x.view(-1) for x in topk_indices.chunk(k, dim=1)]
+    masks_se = [torch.nn.functional.one_hot(x, num_classes=E).to(torch.int64) for x in indices_s]
+    importance = -1 * scores.max(dim=1)[0]
+
+    def compute_location(x):
+        order = importance.argsort(dim=0, stable=True)
+        sorted_x = x[order]
+        sorted_cumsum = (torch.cumsum(sorted_x, dim=0) - 1) * sorted_x
+        return sorted_cumsum[order.argsort(dim=0)]
+
+    locations = [torch.sum(compute_location(masks_se[0]) * masks_se[0], dim=1)]
+    acc_base = None
+    for j in range(1, k):
+        s = torch.sum(masks_se[j - 1], dim=0, keepdim=True)
+        acc_base = s if acc_base is None else acc_base + s
+        loc2 = compute_location(masks_se[j]) + acc_base
+        locations.append(torch.sum(loc2 * masks_se[j], dim=1))
+    return torch.stack(indices_s).numpy().astype(np.int32), torch.stack(locations).numpy().astype(np.int32)
+
+
+@pytest.mark.parametrize("T,E,k", [(257, 8, 2), (1000, 16, 3), (64, 4, 1), (500, 5, 5)])
+def test_route_locations_against_the_torch_chain(T, E, k):
+    """orc_route_locations with the importance order against the reference's own op chain, and
+    without an order against orc_route_topk."""
+    scores = tie_free_scores(T, E, k, seed=T + E)
+    idx, want = _torch_bpr_locations(scores, k)
+    order = torch.argsort(-scores.max(dim=1)[0], stable=True).numpy().astype(np.int32)
+    loc, counts = oracle.route_locations(idx, E, order)
+    assert np.array_equal(loc, want)
+    idx2, loc2, _, counts2 = oracle.route_topk(scores.numpy(), k)
+    assert np.array_equal(idx2, idx)
+    loc3, counts3 = oracle.route_locations(idx, E)
+    assert np.array_equal(loc3, loc2) and np.array_equal(counts3, counts2) and np.array_equal(counts, counts2)
+    # an order only permutes who gets which slot of an expert
+    for j in range(k):
+        for e in range(E):
+            m = idx[j] == e
+            assert sorted(loc[j][m]) == sorted(loc2[j][m])
+
+
+def test_route_locations_ignores_out_of_range_indices():
+    idx = np.array([[0, 5, -1, 1, 0, 7]], np.int32)
+    loc, counts = oracle.route_locations(idx, 2)
+    assert loc.tolist() == [[0, -1, -1, 0, 1, -1]] and counts.tolist() == [[2, 1]]
