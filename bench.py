@@ -174,9 +174,13 @@ def main():
         sys.exit("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
                  "(nothing here uses a second GPU)" % args.gpus)
     if args.kernels:
+        import __graft_entry__
+        __graft_entry__.ensure_built()
         kernel_table()
         return
 
+    import __graft_entry__
+    __graft_entry__.ensure_built()
     import numpy as np
     import torch
     from planmoe_amd import ops

@@ -10,6 +10,10 @@ if ROOT not in sys.path:
 
 GOLDEN = os.path.join(ROOT, "tests", "golden")
 
+# the tests load what is built; only a tree in which nothing is built gets compiled here
+import __graft_entry__  # noqa: E402
+__graft_entry__.ensure_built()
+
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
