@@ -101,15 +101,6 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
         mn = wave_allreduce(mn, [](float a, float b) { return nan_min(a, b); });
         mx = wave_allreduce(mx, [](float a, float b) { return nan_max(a, b); });
     };
-    auto encode = [&](const uint4 &raw, float g, const RowQuant<DT> &rq, uint32_t *w) {
-        float f[V];
-        E::unpack(raw, f);
-#pragma unroll
-        for (int i = 0; i < V; ++i) f[i] = E::round(0.f + g * f[i]);
-#pragma unroll
-        for (int i = 0; i < V / 4; ++i)
-            w[i] = rq(f[4 * i]) | (rq(f[4 * i + 1]) << 8) | (rq(f[4 * i + 2]) << 16) | (rq(f[4 * i + 3]) << 24);
-    };
     auto put = [&](int s, int u, const uint32_t *w) {
         uint8_t *row = codes + (int64_t)s * model_dim;
         if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(row) + u, make_uint2(w[0], w[1]));
@@ -185,18 +176,21 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
                 }
                 const float scale = E::round(mx - mn);
                 if (lane == 0) { E::store(bias_out, s, mn); E::store(scale_out, s, scale); }
-                const RowQuant<DT> rq(mn, scale);
-                auto emit = [&](int u, const uint4 &raw) {
-                    uint32_t w[2];
-                    encode(raw, g, rq, w);
-                    put(s, u, w);
-                };
-                if constexpr (CACHE > 0) {
+                const RowEncoder<DT> enc(mn, scale);
+                auto body = [&](auto mode) {
+                    auto emit = [&](int u, const uint4 &raw) {
+                        uint32_t w[2];
+                        enc.template encode_gated<decltype(mode)::value>(raw, g, w);
+                        put(s, u, w);
+                    };
+                    if constexpr (CACHE > 0) {
 #pragma unroll
-                    for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) emit(c * WAVE + lane, cache[c]);
-                } else {
-                    for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
-                }
+                        for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) emit(c * WAVE + lane, cache[c]);
+                    } else {
+                        for (int u = lane; u < units; u += WAVE) emit(u, src[u]);
+                    }
+                };
+                if (enc.fast()) body(std::true_type{}); else body(std::false_type{});
             }
         }
     }

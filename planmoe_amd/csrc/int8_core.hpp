@@ -119,6 +119,18 @@ struct RowEncoder {
         for (int i = 0; i < E::VEC / 4; ++i)
             w[i] = rq(0.f + f[4 * i]) | (rq(0.f + f[4 * i + 1]) << 8) | (rq(0.f + f[4 * i + 2]) << 16) | (rq(0.f + f[4 * i + 3]) << 24);
     }
+    // the row scaled by its gate first, as the dispatcher stores it: round(0 + g * x)
+    template <bool FAST>
+    __device__ __forceinline__ void encode_gated(const uint4 &raw, float g, uint32_t *w) const
+    {
+        float f[E::VEC];
+        E::unpack(raw, f);
+#pragma unroll
+        for (int i = 0; i < E::VEC; ++i) f[i] = E::round(0.f + g * f[i]);
+#pragma unroll
+        for (int i = 0; i < E::VEC / 4; ++i)
+            w[i] = rq(f[4 * i]) | (rq(f[4 * i + 1]) << 8) | (rq(f[4 * i + 2]) << 16) | (rq(f[4 * i + 3]) << 24);
+    }
 };
 
 // bf16: two elements per 32-bit word all the way.  Min / max run on 16-bit order-preserving
@@ -191,7 +203,12 @@ struct RowEncoder<PLANMOE_BF16> {
     template <bool FAST>
     __device__ __forceinline__ uint32_t pair(uint32_t w) const
     {
-        const float f0 = __uint_as_float(w << 16), f1 = __uint_as_float(w & 0xffff0000u);
+        return pair_values<FAST>(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u));
+    }
+    // two values that are bf16 already -> code0 | code1 << 8
+    template <bool FAST>
+    __device__ __forceinline__ uint32_t pair_values(float f0, float f1) const
+    {
         if constexpr (!FAST) return quantise<PLANMOE_BF16>(0.f + f0, rq.bias, rq.scale) | (quantise<PLANMOE_BF16>(0.f + f1, rq.bias, rq.scale) << 8);
         uint32_t pk = f32x2_to_bf16x2(f0 - rq.bias, f1 - rq.bias);
         const float d0 = __uint_as_float(pk << 16), d1 = __uint_as_float(pk & 0xffff0000u);
@@ -207,6 +224,20 @@ struct RowEncoder<PLANMOE_BF16> {
     {
         w[0] = pair<FAST>(raw.x) | (pair<FAST>(raw.y) << 16);
         w[1] = pair<FAST>(raw.z) | (pair<FAST>(raw.w) << 16);
+    }
+    // the row scaled by its gate first, as the dispatcher stores it: round(0 + g * x)
+    template <bool FAST>
+    __device__ __forceinline__ uint32_t pair_gated(uint32_t w, float g) const
+    {
+        const float x0 = __uint_as_float(w << 16), x1 = __uint_as_float(w & 0xffff0000u);
+        const uint32_t pk = f32x2_to_bf16x2(0.f + g * x0, 0.f + g * x1);
+        return pair_values<FAST>(__uint_as_float(pk << 16), __uint_as_float(pk & 0xffff0000u));
+    }
+    template <bool FAST>
+    __device__ __forceinline__ void encode_gated(const uint4 &raw, float g, uint32_t *w) const
+    {
+        w[0] = pair_gated<FAST>(raw.x, g) | (pair_gated<FAST>(raw.y, g) << 16);
+        w[1] = pair_gated<FAST>(raw.z, g) | (pair_gated<FAST>(raw.w, g) << 16);
     }
 };
 
