@@ -246,3 +246,30 @@ def test_cosine_gate_logits_and_layer():
     assert torch.isfinite(xin.grad).all()
     g = layer.gates[0].sim_matrix.grad
     assert g is not None and torch.isfinite(g).all() and g.abs().sum() > 0
+
+
+@pytest.mark.parametrize("T,M,E,k,cf,use_bias", [(16384, 4096, 8, 2, 1.25, False), (32768, 2048, 64, 1, 1.0, True),
+                                                  (8192, 2048, 2, 2, 1.0, False)])
+def test_forward_entry_point_full_size(T, M, E, k, cf, use_bias):
+    """planmoe_forward_int8 (two launches) at the full size of configs 2, 3 and 1 (bf16 here):
+    routing against the oracle on the scores the kernel reports, codes / bias / scale against the
+    stand-alone dispatch + int8 entry point on that routing, counts and loss against the oracle."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn(T, M, generator=g).bfloat16().to(DEV)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
+    bias = zipf_bias(E) if use_bias else None
+    C = ops.capacity(T, E, k, cf, 4)
+    out = ops.forward_int8(x, wg, k, C, logit_bias=bias, want_scores=True, want_counts=True)
+    scores = out["scores"].cpu().numpy()
+    idx, loc, gates, counts = oracle.route_topk(scores, k)
+    assert np.array_equal(out["indices"].cpu().numpy(), idx)
+    assert np.array_equal(out["locations"].cpu().numpy(), loc)
+    assert np.array_equal(raw(out["gates"]), np_raw(gates))
+    assert np.array_equal(out["counts"].cpu().numpy(), counts)
+    want = oracle.gshard_loss(scores, idx[0])
+    assert abs(float(out["l_aux"]) - want) <= 1e-5 * abs(want)
+    c2, b2, s2 = ops.dispatch_int8(x, list(out["indices"]), list(out["locations"]), None, E, C)
+    assert torch.equal(out["codes"].view(-1), c2.view(-1))
+    assert np.array_equal(raw(out["bias"]).reshape(-1), raw(b2).reshape(-1))
+    assert np.array_equal(raw(out["scale"]).reshape(-1), raw(s2).reshape(-1))
