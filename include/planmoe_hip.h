@@ -198,9 +198,10 @@ int planmoe_combine_bwd_int8(const void *grad_out, const void *expert_out, int d
                              float *grad_gates, void *workspace, size_t workspace_bytes, void *stream);
 
 /* ---------------------------------------------------------------- fused forward chain
- * The layer's forward path up to the all-to-all send buffer in three launches: gate GEMM +
- * routing (gates/top.py:20-26, moe_layer.py:230-256, fast_dispatch.py:140-195), then
- * fast_encode + Int8Compressor::compress (fast_dispatch.py:197-201, int8.cpp:7-44).
+ * The layer's forward path up to the all-to-all send buffer in two launches (three when
+ * top_k > 4): gate GEMM + routing (gates/top.py:20-26, moe_layer.py:230-256,
+ * fast_dispatch.py:140-195), then fast_encode + Int8Compressor::compress
+ * (fast_dispatch.py:197-201, int8.cpp:7-44) with the prefix over the routing groups folded in.
  * Limits: experts <= 64, model_dim a multiple of 8 (bf16/fp16) or 4 (fp32), the all-ones gate
  * helper at encode (is_postscore), capacity_factor > 0 routing.
  *
@@ -208,7 +209,7 @@ int planmoe_combine_bwd_int8(const void *grad_out, const void *expert_out, int d
  * scores and gates are fp32 (top.py:21-23); otherwise they are rounded to `dtype`.
  * gates, logits_out, scores_out are in that score dtype; logits_out / scores_out / l_aux /
  * expert_counts / logit_bias may be NULL.  Other arguments as in planmoe_route_topk.
- * Limits in addition: top_k <= 16.  Calls sharing a workspace must not overlap. */
+ * Calls sharing a workspace must not overlap. */
 size_t planmoe_forward_workspace_bytes(int samples, int experts, int top_k);
 
 /* gate GEMM + routing only (the outputs of planmoe_gate_logits + planmoe_route_topk) */

@@ -1,23 +1,25 @@
-// The forward chain in three launches:
+// The forward chain in two launches (three when top_k > 4):
 //
 //   gate_route_kernel     x is read once: gate-logits GEMM on the matrix cores, then, for the
-//                         work-group's 32 tokens, softmax, k-fold arg-max, gates, the rank of
-//                         every token among the group's tokens with the same choice, and the
-//                         group's expert histogram.
-//   group_offsets_kernel  exclusive prefix of the histograms over groups, choice plane after
-//                         choice plane (all first choices of an expert precede its second
-//                         choices), expert totals and the GShard loss.  Tiny.
-//   dispatch_int8_routed  slot = rank in group + group offset; token rows go to uint8 codes in
-//                         their slots (x read a second time, normally from cache), slots past an
-//                         expert's fill are zero rows.  Or route_offsets_kernel when only the
-//                         routing is wanted.
+//                         work-group's 64 (or 32) tokens = one routing group, softmax, k-fold
+//                         arg-max, gates, the rank of every token among the group's tokens with
+//                         the same choice, and the group's expert histogram.
+//   dispatch_int8_routed  slot = rank in group + entries of earlier groups and planes (all first
+//                         choices of an expert precede its second choices), summed by every wave
+//                         from the transposed histograms; token rows go to uint8 codes in their
+//                         slots (x is read a second time), slots past an expert's fill are zero
+//                         rows; one block finishes the GShard loss and the expert counts.
+//   group_offsets_kernel  only for top_k > 4 and for planmoe_gate_route (routing without
+//                         dispatch, finished by route_offsets_kernel): the prefix over groups as
+//                         a launch of its own.
 //
 // This replaces gates/top.py:20-26 + moe_layer.py:230-256 + fast_dispatch.py:140-195 +
 // fast_encode (fast_dispatch.py:197-201) + Int8Compressor::compress (int8.cpp:7-44).
 //
-// Workspace (32-bit words): totals[E], loss_part[64], hist[groups][k][E], offs[groups][k][E],
-// me[groups][E] (fp32), rank[k][samples] (rank of a token inside its group), row_min[samples],
-// row_max[samples] (fp32; bf16 inputs only: the gate kernel scans the rows it streams anyway).
+// Workspace (32-bit words): hist_t[k][E][groups up to a multiple of 4], me_t[E][same] (fp32),
+// totals[E], loss_part[64], hist[groups][k][E], offs[groups][k][E], me[groups][E] (fp32),
+// rank[k][samples] (rank of a token inside its group), row_min[samples], row_max[samples]
+// (fp32; bf16 inputs only: the gate kernel scans the rows it streams anyway).
 #include "gate_core.hpp"
 #include "rows.hpp"
 #include "int8_core.hpp"

@@ -380,7 +380,7 @@ def forward_int8(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, norma
 
 class ForwardInt8Plan:
     """forward_int8 with every output and the workspace allocated once: `run()` is a single
-    C-ABI call that enqueues the three launches (for serving loops that reuse their buffers)."""
+    C-ABI call that enqueues the two launches (for serving loops that reuse their buffers)."""
 
     def __init__(self, x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
                  want_l_aux=True, want_counts=False):
