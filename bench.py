@@ -105,6 +105,8 @@ def kernel_table():
     add("int8_compress", "2", db + R * M + R * 4, lambda: ops.int8_compress(d))
     codes, b, s_ = ops.int8_compress(d)
     add("int8_decompress", "2", db + R * M + R * 4, lambda: ops.int8_decompress(codes, b, s_))
+    add("combine_int8 (fused)", "2", live * M + R * 4 + xb + plane,
+        lambda: ops.combine_int8(codes, b, s_, idx, loc, gates, T, C))
     add("dispatch_int8 (fused)", "2", xb + R * M + R * 4 + plane, lambda: ops.dispatch_int8(x, idx, loc, None, E, C))
     add("combine_bwd_int8 (fused)", "4", xb + live * M * 2 + R * M + R * 4 + plane + T * k * 4,
         lambda: ops.combine_bwd_int8(x, d, idx, loc, gates, E, C))

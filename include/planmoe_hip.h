@@ -197,6 +197,17 @@ int planmoe_combine_bwd_int8(const void *grad_out, const void *expert_out, int d
                              int experts, int capacity, uint8_t *codes, void *bias, void *scale,
                              float *grad_gates, void *workspace, size_t workspace_bytes, void *stream);
 
+/* Decompress and combine in one pass (Decompress.apply with "int8" followed by fast_decode:
+ * impls/overlap.py:22-29, int8.cpp:46-60, fast_dispatch.py:203-207): what planmoe_combine_fwd
+ * produces from planmoe_int8_decompress's output, without the intermediate
+ * [experts*capacity, model_dim] tensor.  codes / bias / scale as planmoe_int8_compress writes
+ * them; gates fp32 planes or NULL; out [samples, model_dim] in `dtype`.  Needs model_dim a
+ * multiple of 8 (bf16/fp16) or 4 (fp32). */
+int planmoe_combine_int8(const uint8_t *codes, const void *bias, const void *scale, int dtype,
+                         const float *gates, const int32_t *indices, const int32_t *locations,
+                         int64_t plane_stride, int top_k, int samples, int model_dim, int capacity,
+                         void *out, void *stream);
+
 /* ---------------------------------------------------------------- fused forward chain
  * The layer's forward path up to the all-to-all send buffer in two launches (three when
  * top_k > 4): gate GEMM + routing (gates/top.py:20-26, moe_layer.py:230-256,

@@ -196,6 +196,118 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
     }
 }
 
+// Combine fused with the "int8" decode (the receive side: Int8Compressor::decompress,
+// int8.cpp:46-60, followed by fast_decode, fast_dispatch.py:203-207): the token row is the
+// gate-weighted sum of its slots' rows, decoded from the codes on the fly, so the
+// [experts*capacity, model_dim] tensor never exists in memory.  One wavefront owns one token and
+// all its planes; every decoded value is rounded to the tensor's dtype exactly as the stand-alone
+// decoder stores it before it enters the fp32 sum (planes left to right, one rounding at the end).
+template <int DT>
+__global__ __launch_bounds__(256) void combine_int8_kernel(
+    const uint8_t *__restrict__ codes, const void *__restrict__ bias_in, const void *__restrict__ scale_in,
+    const float *__restrict__ gates, const int32_t *__restrict__ indices,
+    const int32_t *__restrict__ locations, int64_t stride, int top_k, int samples, int model_dim,
+    int capacity, void *__restrict__ out)
+{
+    using E = Elem<DT>;
+    constexpr int V = E::VEC;
+    const int wave = threadIdx.x >> 6, lane = lane_id();
+    const int units = model_dim / V;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= samples) return;
+    uint4 *dst = reinterpret_cast<uint4 *>((char *)out + (int64_t)t * model_dim * (int64_t)sizeof(typename E::store_t));
+
+    auto load_codes = [&](int s, int u, uint32_t *w) {
+        const uint8_t *row = codes + (int64_t)s * model_dim;
+        if constexpr (V == 8) { const uint2 c = reinterpret_cast<const uint2 *>(row)[u]; w[0] = c.x; w[1] = c.y; }
+        else { w[0] = reinterpret_cast<const uint32_t *>(row)[u]; w[1] = 0; }
+    };
+    if (top_k <= 4) {
+        // the usual case: all planes of four units are requested before any is decoded
+        constexpr int UB = 4;
+        int slot; float gate;
+        fetch_planes(gates, indices, locations, stride, t, 0, top_k, 0x7fffffff, capacity, slot, gate);
+        float b_l = 0.f, s_l = 0.f;
+        if (lane < top_k && slot >= 0) { b_l = E::load(bias_in, slot); s_l = E::load(scale_in, slot); }
+        for (int u0 = 0; u0 < units; u0 += UB * WAVE) {
+            uint32_t cw[4][UB][2];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int s = j < top_k ? rl_i(slot, j) : -1;
+#pragma unroll
+                for (int b = 0; b < UB; ++b) {
+                    cw[j][b][0] = cw[j][b][1] = 0u;
+                    // clamped, not predicated: straight-line loads (dead planes read slot 0)
+                    load_codes(max(s, 0), min(u0 + b * WAVE + lane, units - 1), cw[j][b]);
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < UB; ++b) {
+                const int u = u0 + b * WAVE + lane;
+                float acc[V];
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[i] = 0.f;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (j < top_k) {
+                        const int s = rl_i(slot, j);
+                        const float g = rl_f(gate, j);
+                        float term[V];
+                        if (s >= 0) {
+                            const RowDecoder<DT> dec(rl_f(b_l, j), rl_f(s_l, j));
+#pragma unroll
+                            for (int q = 0; q < V / 4; ++q) dec.word(cw[j][b][q], term + 4 * q);
+#pragma unroll
+                            for (int i = 0; i < V; ++i) term[i] = g * term[i];
+                        } else {
+#pragma unroll
+                            for (int i = 0; i < V; ++i) term[i] = 0.f;
+                        }
+#pragma unroll
+                        for (int i = 0; i < V; ++i) acc[i] = (j == 0) ? term[i] : acc[i] + term[i];
+                    }
+                }
+                if (u < units) stream_store(dst + u, E::pack(acc));
+            }
+        }
+        return;
+    }
+    for (int u0 = 0; u0 < units; u0 += WAVE) {
+        const int u = u0 + lane;
+        float acc[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc[i] = 0.f;
+        for (int j0 = 0; j0 < top_k; j0 += WAVE) {
+            const int np = min(top_k - j0, WAVE);
+            int slot; float gate;
+            fetch_planes(gates, indices, locations, stride, t, j0, np, 0x7fffffff, capacity, slot, gate);
+            // bias and scale of the lane's own plane, broadcast below
+            float b_l = 0.f, s_l = 0.f;
+            if (lane < np && slot >= 0) { b_l = E::load(bias_in, slot); s_l = E::load(scale_in, slot); }
+            for (int j = 0; j < np; ++j) {
+                const int s = rl_i(slot, j);
+                const float g = rl_f(gate, j);
+                float term[V];
+                if (s >= 0 && u < units) {
+                    const RowDecoder<DT> dec(rl_f(b_l, j), rl_f(s_l, j));
+                    uint32_t w[2];
+                    load_codes(s, u, w);
+#pragma unroll
+                    for (int q = 0; q < V / 4; ++q) dec.word(w[q], term + 4 * q);
+#pragma unroll
+                    for (int i = 0; i < V; ++i) term[i] = g * term[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) term[i] = 0.f;
+                }
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc[i] = (j0 + j == 0) ? term[i] : acc[i] + term[i];
+            }
+        }
+        if (u < units) stream_store(dst + u, E::pack(acc));
+    }
+}
+
 template <int DT>
 static void launch_dispatch_int8(int per_lane, unsigned grid, hipStream_t st, const void *x,
                                  const float *gates, const int32_t *indices, const int32_t *locations,
@@ -286,4 +398,32 @@ extern "C" int planmoe_combine_bwd_int8(const void *grad_out, const void *expert
     return run_dispatch_int8("planmoe_combine_bwd_int8", grad_out, dtype, gates, indices, locations,
                              plane_stride, top_k, samples, model_dim, experts, capacity, codes, bias, scale,
                              workspace, workspace_bytes, expert_out, grad_gates, stream);
+}
+
+extern "C" int planmoe_combine_int8(const uint8_t *codes, const void *bias, const void *scale, int dtype,
+                                    const float *gates, const int32_t *indices, const int32_t *locations,
+                                    int64_t plane_stride, int top_k, int samples, int model_dim,
+                                    int capacity, void *out, void *stream)
+{
+    if (check_planes("planmoe_combine_int8", indices, locations, plane_stride, top_k, samples)) return 1;
+    PM_REQUIRE(dtype_ok(dtype), "planmoe_combine_int8: bad dtype %d", dtype);
+    PM_REQUIRE(model_dim >= 1 && capacity >= 0, "planmoe_combine_int8: bad shape");
+    if (samples == 0) return 0;
+    PM_REQUIRE(out, "planmoe_combine_int8: out is NULL");
+    PM_REQUIRE((codes && bias && scale) || capacity == 0, "planmoe_combine_int8: NULL codec input");
+    const int vec = dtype == PLANMOE_F32 ? 4 : 8;
+    PM_REQUIRE(model_dim % vec == 0 && aligned16(out) && (uintptr_t)codes % 8 == 0,
+               "planmoe_combine_int8: model_dim must be a multiple of %d, out 16-byte and codes 8-byte aligned "
+               "(use planmoe_int8_decompress + planmoe_combine_fwd otherwise)", vec);
+    if (capacity == 0) {
+        // no slot can be live: every token row is zero
+        fill_u32((uint32_t *)out, (size_t)samples * model_dim * (dtype == PLANMOE_F32 ? 4 : 2) / 4, 0u, (hipStream_t)stream);
+        PM_LAUNCH_CHECK("planmoe_combine_int8");
+        return 0;
+    }
+    const int blocks = (samples + 3) / 4;
+    PM_DTYPE_SWITCH(dtype, DT, (combine_int8_kernel<DT><<<blocks, 256, 0, (hipStream_t)stream>>>(
+        codes, bias, scale, gates, indices, locations, plane_stride, top_k, samples, model_dim, capacity, out)));
+    PM_LAUNCH_CHECK("planmoe_combine_int8");
+    return 0;
 }

@@ -79,6 +79,39 @@ struct RowDequant {
     }
 };
 
+// Decoder of one row for callers that consume the values as fp32 right away (combine fused with
+// the decode): four codes of a 32-bit word -> four values, each rounded to the dtype after every
+// step exactly as RowDequant does.  bf16 works on pairs, so that every rounding is one packed
+// conversion for two values.
+template <int DT>
+struct RowDecoder {
+    RowDequant<DT> dq;
+    __device__ __forceinline__ RowDecoder(float b, float s) : dq(b, s) {}
+    __device__ __forceinline__ void word(uint32_t w, float *f) const
+    {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = dq((w >> (8 * i)) & 0xffu);
+    }
+};
+template <>
+struct RowDecoder<PLANMOE_BF16> {
+    float bias, scale;
+    __device__ __forceinline__ RowDecoder(float b, float s) : bias(b), scale(s) {}
+    __device__ __forceinline__ void pair(float c0, float c1, float &o0, float &o1) const
+    {
+        constexpr float inv = 1.0f / 255.0f;
+        uint32_t pk = f32x2_to_bf16x2(c0 * inv, c1 * inv);
+        pk = f32x2_to_bf16x2(__uint_as_float(pk << 16) * scale, __uint_as_float(pk & 0xffff0000u) * scale);
+        pk = f32x2_to_bf16x2(__uint_as_float(pk << 16) + bias, __uint_as_float(pk & 0xffff0000u) + bias);
+        o0 = __uint_as_float(pk << 16); o1 = __uint_as_float(pk & 0xffff0000u);
+    }
+    __device__ __forceinline__ void word(uint32_t w, float *f) const
+    {
+        pair((float)(w & 0xffu), (float)((w >> 8) & 0xffu), f[0], f[1]);
+        pair((float)((w >> 16) & 0xffu), (float)(w >> 24), f[2], f[3]);
+    }
+};
+
 // ---------------------------------------------------------------- row-level building blocks
 // RowStats<DT, CANON>: running min / max of a row, NaN-propagating like torch.min / torch.max.
 // CANON: the row as the dispatcher would store it (0 + x, so -0 reads as +0).  RowEncoder<DT>: one 16-byte vector of

@@ -14,7 +14,7 @@ from . import experts as _experts
 from . import gates as _gates
 from . import losses, ops
 from .fast_dispatch import extract_critical, fast_decode, fast_encode, route
-from .overlap import a2a_ffn_overlap_forward
+from .overlap import a2a_ffn_overlap_forward, fused_int8_eligible, fused_int8_forward
 
 
 class MOELayer(torch.nn.Module):
@@ -184,6 +184,18 @@ class MOELayer(torch.nn.Module):
                                            batch_prioritized_routing=self.batch_prioritized_routing,
                                            normalize_gate=self.normalize_gate, group=self.group,
                                            alignment=alignment)
+
+        if fused_int8_eligible(x, self.compress_name, degree, self.is_postscore):
+            # encode + compress and decompress + decode in one pass each (bit-identical to the steps)
+            if self.training:
+                self.save_count = self.save_count + 1
+
+            def expert_fn(expert_input):
+                return self.expert_local(expert_input, original_shape[-reserve_dims:])
+            y = fused_int8_forward(x, crit, expert_fn)
+            y = y.view(list(original_shape)).to(original_dtype)
+            self.l_aux = y.l_aux = l_aux
+            return self.result_func(y) if self.result_func is not None else y
 
         # the reference casts x to the logits dtype around fast_encode / fast_decode
         # (moe_layer.py:265, 306); the kernels do that fp32 arithmetic in registers

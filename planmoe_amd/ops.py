@@ -265,6 +265,20 @@ def int8_decompress(codes, bias, scale):
     return out
 
 
+def combine_int8(codes, bias, scale, indices, locations, gates, samples, capacity_):
+    """The int8 decompressor followed by fast_decode, in one pass: codes [experts*capacity, M]
+    uint8 with their bias / scale -> [T, M] in bias.dtype."""
+    _need_gpu(codes, "combine_int8")
+    codes = _contig(codes, "combine_int8")
+    M = codes.shape[-1]
+    idx, loc, g, stride = _plane_args(indices, locations, gates, "combine_int8")
+    out = torch.empty((samples, M), dtype=bias.dtype, device=codes.device)
+    check(lib.planmoe_combine_int8(_ptr(codes), _ptr(bias.contiguous()), _ptr(scale.contiguous()),
+                                   _dt(bias, "combine_int8"), _ptr(g), _ptr(idx), _ptr(loc), stride,
+                                   len(indices), samples, M, capacity_, _ptr(out), _stream(codes)))
+    return out
+
+
 def dispatch_int8(x, indices, locations, gates, experts, capacity_):
     """fast_encode followed by the int8 compressor, in one pass.
     Returns codes [experts*capacity, M] uint8, bias, scale [experts*capacity, 1]."""

@@ -5,6 +5,7 @@ stream (no comm streams to overlap with)."""
 import torch
 
 from . import compressor as _ck
+from . import ops
 
 MAX_NUM_SPLIT = 32     # AllToAllStatus.max_num_split of the reference (communicate.py)
 
@@ -71,3 +72,73 @@ def a2a_ffn_overlap_forward(input, expert_fn, a2a_ffn_overlap_degree, use_2dh, g
     for i in range(a2a_ffn_overlap_degree):
         input_split[i] = Decompress.apply(input_split[i], compress_name, comm_name)
     return torch.cat(input_split, dim=split_dim).contiguous()
+
+
+# ------------------------------------------------------------------------------ fused int8 path
+# With the "int8" compressor and one chunk, the steps either side of the all-to-all collapse:
+#   send side     fast_encode + Compress      -> one pass (planmoe_dispatch_int8)
+#   receive side  Decompress + fast_decode    -> one pass (planmoe_combine_int8)
+# and the same two fusions serve the backward pass (Decompress.backward compresses the gradient,
+# Compress.backward decompresses it, overlap.py:19-21, 32-34).  Results are bit-identical to the
+# step-by-step pipeline; FUSE_INT8 = False keeps the reference's structure.
+FUSE_INT8 = True
+
+
+class _EncodeInt8(torch.autograd.Function):
+    """Decompress(Comm(Compress(fast_encode(x)))) for the all-ones gate helper (is_postscore)."""
+
+    @staticmethod
+    def forward(ctx, x, indices, locations, experts, capacity):
+        codes, bias, scale = ops.dispatch_int8(x, list(indices), list(locations), None, experts, capacity)
+        ctx.save_for_backward(indices, locations)
+        ctx.samples, ctx.capacity = x.shape[0], capacity
+        return ops.int8_decompress(codes, bias, scale)
+
+    @staticmethod
+    def backward(ctx, grad):
+        indices, locations = ctx.saved_tensors
+        codes, bias, scale = ops.int8_compress(grad.contiguous())
+        dx = ops.combine_int8(codes, bias, scale, list(indices), list(locations), None, ctx.samples, ctx.capacity)
+        return dx, None, None, None, None
+
+
+class _DecodeInt8(torch.autograd.Function):
+    """fast_decode(Decompress(Comm(Compress(y)))) with the gates applied at decode."""
+
+    @staticmethod
+    def forward(ctx, y, indices, locations, experts, capacity, samples, *gates):
+        codes, bias, scale = ops.int8_compress(y.contiguous())
+        out = ops.combine_int8(codes, bias, scale, list(indices), list(locations), list(gates), samples, capacity)
+        ctx.save_for_backward(codes, bias, scale, indices, locations, *gates)
+        ctx.experts, ctx.capacity = experts, capacity
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        codes, bias, scale, indices, locations, *gates = ctx.saved_tensors
+        seen = ops.int8_decompress(codes, bias, scale)          # the tensor fast_decode consumed
+        gcodes, gbias, gscale, grad_gates = ops.combine_bwd_int8(
+            grad_out.contiguous(), seen, list(indices), list(locations), list(gates), ctx.experts, ctx.capacity)
+        grad_y = ops.int8_decompress(gcodes, gbias, gscale)
+        return (grad_y, None, None, None, None, None,
+                *[grad_gates[j].to(g.dtype) for j, g in enumerate(gates)])
+
+
+def fused_int8_eligible(x, compress_name, degree, is_postscore):
+    vec = 4 if x.dtype == torch.float32 else 8
+    return (FUSE_INT8 and compress_name == 'int8' and degree == 1 and is_postscore and x.is_cuda and
+            x.dtype in (torch.float32, torch.bfloat16, torch.float16) and x.shape[-1] % vec == 0)
+
+
+def fused_int8_forward(x, crit, expert_fn):
+    """encode -> [codec, comm, codec] -> experts -> [codec, comm, codec] -> decode for one chunk
+    and the int8 compressor.  crit = (experts, indices_s, locations_s, gates_s, capacity)."""
+    experts, indices_s, locations_s, gates_s, capacity = crit
+    indices = torch.stack([t.reshape(-1) for t in indices_s]).to(torch.int32).contiguous()     # [k, T]
+    locations = torch.stack([t.reshape(-1) for t in locations_s]).to(torch.int32).contiguous()
+    y = _EncodeInt8.apply(x.contiguous(), indices, locations, experts, capacity)
+    y = expert_fn(y.view(experts, capacity, x.shape[-1]))
+    y = y.reshape(experts * capacity, -1).to(x.dtype)
+    gates = [g.float() for g in gates_s]
+    return _DecodeInt8.apply(y, indices, locations, experts, capacity, x.shape[0], *gates)
+

@@ -258,3 +258,31 @@ def test_combine_bwd_int8_equals_the_unfused_backward(T, M, E, k, cf, dtype):
         assert (np.abs(got - want) <= rtol * np.abs(want) + 1e-6 * mag).all()
         assert (got[loc[j] >= C] == 0).all()
         assert np.allclose(got, g2[j].cpu().numpy(), rtol=1e-5, atol=1e-6 * mag.max())
+
+
+@pytest.mark.parametrize("T,M,E,k,dtype,gated", [(1000, 512, 8, 2, torch.bfloat16, True), (300, 264, 5, 3, torch.bfloat16, False),
+                                                  (257, 128, 4, 2, torch.float32, True), (64, 72, 3, 1, torch.float16, True),
+                                                  (16384, 4096, 8, 2, torch.bfloat16, True)])
+def test_combine_int8_equals_decompress_then_combine(T, M, E, k, dtype, gated):
+    """planmoe_combine_int8 against planmoe_int8_decompress + planmoe_combine_fwd (bit for bit),
+    and, for bf16 / fp32, that pair against the oracle."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(T + M)
+    scores = torch.softmax(torch.randn(T, E, generator=g), 1)
+    r = ops.route_topk(scores.to(DEV), k)
+    C = ops.capacity(T, E, k, 1.0, 4)
+    idx, loc = list(r["indices"]), list(r["locations"])
+    gates = [x.float() for x in r["gates"]] if gated else None
+    y = torch.randn(E * C, M, generator=g).to(dtype).to(DEV)          # expert outputs
+    codes, bias, scale = ops.int8_compress(y)
+    want = ops.combine_fwd(ops.int8_decompress(codes, bias, scale), idx, loc, gates, T, C)
+    got = ops.combine_int8(codes, bias, scale, idx, loc, gates, T, C)
+    assert np.array_equal(raw(got), raw(want))
+    if dtype != torch.float16 and T <= 1000:
+        rc, rb, rs = oracle.int8_compress(bf16_bits(y.cpu()) if dtype == torch.bfloat16 else y.cpu().numpy())
+        dec = oracle.int8_decompress(rc, rb, rs)
+        dec32 = from_bf16_bits(dec).float().numpy() if dtype == torch.bfloat16 else dec
+        ref = oracle.decode(dec32, [a.cpu().numpy() for a in idx], [a.cpu().numpy() for a in loc],
+                            [a.cpu().numpy() for a in gates] if gated else None, T, C)
+        ref_t = torch.from_numpy(ref).to(dtype)
+        assert np.array_equal(raw(got), raw(ref_t))

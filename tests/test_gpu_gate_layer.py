@@ -273,3 +273,28 @@ def test_forward_entry_point_full_size(T, M, E, k, cf, use_bias):
     assert torch.equal(out["codes"].view(-1), c2.view(-1))
     assert np.array_equal(raw(out["bias"]).reshape(-1), raw(b2).reshape(-1))
     assert np.array_equal(raw(out["scale"]).reshape(-1), raw(s2).reshape(-1))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_moe_layer_fused_int8_path_equals_the_stepwise_pipeline(dtype):
+    """moe_layer with compress_name='int8': the fused send / receive sides (dispatch+compress,
+    decompress+combine) against the step-by-step pipeline, outputs and every gradient bit for bit."""
+    import planmoe_amd
+    from planmoe_amd import overlap
+    results = []
+    for fuse in (True, False):
+        overlap.FUSE_INT8 = fuse
+        try:
+            layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 1.25}, 128,
+                                          experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 64},
+                                          seeds=(1, 2, 3), compress_name='int8').to(DEV).to(dtype)
+            x = torch.randn(6, 50, 128, generator=torch.Generator().manual_seed(5)).to(dtype).to(DEV).requires_grad_(True)
+            y = layer(x)
+            (y.float().pow(2).mean() + y.l_aux.float()).backward()
+            results.append((y.detach(), x.grad.detach(), layer.gates[0].wg.weight.grad.detach(),
+                            layer.experts.batched_fc1_w.grad.detach()))
+        finally:
+            overlap.FUSE_INT8 = True
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    assert results[0][1].abs().sum() > 0 and results[0][2].abs().sum() > 0
