@@ -298,3 +298,20 @@ def test_moe_layer_fused_int8_path_equals_the_stepwise_pipeline(dtype):
     for a, b in zip(*results):
         assert torch.equal(a, b)
     assert results[0][1].abs().sum() > 0 and results[0][2].abs().sum() > 0
+
+
+def test_moe_layer_prescore_noise_and_load_importance_loss():
+    """The remaining layer options run end to end: gates applied at encode (is_postscore=False),
+    gate noise with the load-importance loss, a data-dependent capacity (capacity_factor = 0)."""
+    import planmoe_amd
+    layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'gate_noise': 1.0, 'capacity_factor': 0.0},
+                                  64, experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 96},
+                                  seeds=(1, 2, 3), compress_name='int8', is_postscore=False,
+                                  is_gshard_loss=False).to(DEV).train()
+    x = torch.randn(4, 40, 64, device=DEV, requires_grad=True)
+    y = layer(x)
+    assert y.shape == x.shape and torch.isfinite(y).all() and torch.isfinite(y.l_aux)
+    (y.pow(2).mean() + y.l_aux).backward()
+    assert torch.isfinite(x.grad).all()
+    wg = layer.gates[0].wg.weight.grad
+    assert wg is not None and torch.isfinite(wg).all() and wg.abs().sum() > 0

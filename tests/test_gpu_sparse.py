@@ -183,3 +183,28 @@ def test_autograd_wiring_matches_the_reference_functions():
     for j in range(k):
         want = oracle.bwd_gate(idx[j], loc[j], dOut.cpu().double().numpy(), eo.detach().cpu().view(E * C, M).double().numpy(), C)
         assert np.allclose(crit[3][j].grad.cpu().numpy(), want, rtol=1e-5, atol=1e-4)
+
+
+def test_prescore_mode_gates_at_encode():
+    """is_postscore=False (fast_dispatch.py:40-45, 120-131): the gates scale the rows at encode,
+    decode uses all-ones, and the gate gradient comes out of the encoder's backward."""
+    import planmoe_amd
+    T, M, E, k = 160, 48, 4, 2
+    idx, loc, gates, C = _routing(T, E, k, 1.0, seed=9)
+    gs = [t.requires_grad_() for t in _dev(gates)]
+    crit = (E, _dev(idx), _dev(loc), gs, C)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(T, M, generator=g).to(DEV).requires_grad_()
+    y = planmoe_amd.fast_encode(x, crit, is_postscore=False)
+    want = oracle.encode(x.detach().cpu().numpy(), list(idx), list(loc), list(gates), E, C)
+    assert np.array_equal(raw(y.view(E * C, M)), want.view(np.int32))
+    dY = torch.randn(E, C, M, generator=g).to(DEV)
+    y.backward(dY)
+    want_dx = oracle.decode(dY.cpu().view(E * C, M).numpy(), list(idx), list(loc), list(gates), T, C)
+    assert np.array_equal(raw(x.grad), want_dx.view(np.int32))
+    for j in range(k):
+        wg = oracle.bwd_gate(idx[j], loc[j], x.detach().cpu().double().numpy(), dY.cpu().view(E * C, M).double().numpy(), C)
+        assert np.allclose(gs[j].grad.cpu().numpy(), wg, rtol=1e-5, atol=1e-4)
+    out = planmoe_amd.fast_decode(y.detach(), crit, is_postscore=False)
+    want_out = oracle.decode(want, list(idx), list(loc), None, T, C)
+    assert np.array_equal(raw(out), want_out.view(np.int32))
