@@ -41,31 +41,49 @@ struct BitWriter {
     }
 };
 
+// The decoder looks at the stream by bit position: the block's words sit in LDS (NW + 1 words per
+// thread, the last one zero) and a look is two neighbouring words funnel-shifted, so there is no
+// refill state to carry and no branch in the reader.  Streams of one or two words stay in a
+// register pair that is shifted as bits are consumed.
 template <int NW>
 struct BitReader {
-    uint32_t w[NW];
-    uint64_t acc;
-    int avail, wi;
-    __device__ __forceinline__ void init()
+    const uint32_t *words;      // this thread's NW + 1 words in LDS
+    int pos;
+    uint64_t small;             // NW <= 2: the whole stream in a register pair instead
+    __device__ __forceinline__ void init(uint32_t *lds, const uint32_t *w)
     {
-        acc = w[0];
-        avail = 32; wi = 1;
-        if constexpr (NW > 1) { acc |= (uint64_t)w[1] << 32; avail = 64; wi = 2; }
-    }
-    __device__ __forceinline__ void skip(int n)
-    {
-        acc >>= n; avail -= n;
-        if (avail <= 32 && wi < NW) {
-            uint32_t x = 0;
+        pos = 0;
+        if constexpr (NW <= 2) {
+            small = w[0];
+            if constexpr (NW == 2) small |= (uint64_t)w[1] << 32;
+            words = nullptr;
+        } else {
+            uint32_t *mine = lds + threadIdx.x * (NW + 1);
 #pragma unroll
-            for (int i = 0; i < NW; ++i) if (i == wi) x = w[i];
-            acc |= (uint64_t)x << avail;
-            avail += 32; ++wi;
+            for (int i = 0; i < NW; ++i) mine[i] = w[i];
+            mine[NW] = 0u;
+            words = mine;
+            small = 0;
         }
+    }
+    // the next 32 bits of the stream (zeros past its end)
+    __device__ __forceinline__ uint32_t peek() const
+    {
+        if constexpr (NW <= 2) {
+            return (uint32_t)small;                 // skip() keeps the register pair shifted
+        } else {
+            const int i = pos >> 5;
+            return __builtin_amdgcn_alignbit(words[i + 1], words[i], pos & 31);
+        }
+    }
+    __device__ __forceinline__ void skip(int n)      // n <= 32
+    {
+        if constexpr (NW <= 2) small >>= n;
+        else pos += n;
     }
     __device__ __forceinline__ uint32_t get(int n)   // n <= 31
     {
-        const uint32_t v = (uint32_t)acc & ((1u << n) - 1u);
+        const uint32_t v = peek() & ((1u << n) - 1u);
         skip(n);
         return v;
     }
@@ -247,7 +265,6 @@ __device__ __forceinline__ void encode_block(const float *f, BitWriter<NW> &bw, 
 template <int N, int NW>
 __device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f)
 {
-    br.init();
     if (!br.get(1)) {
 #pragma unroll
         for (int i = 0; i < N; ++i) f[i] = 0.f;
@@ -264,16 +281,28 @@ __device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f)
         bits -= mm;
         uint32_t x = br.get(mm);
         while (nsig < N && bits > 0) {
-            --bits;
-            if (!br.get(1)) break;
-            const int lim = min(N - 1 - nsig, bits);
-            const uint32_t win = (uint32_t)br.acc & ((1u << lim) - 1u);
-            if (win != 0u) {
-                const int z = __builtin_ctz(win);
-                br.skip(z + 1); bits -= z + 1; nsig += z;
-            } else {
-                br.skip(lim); bits -= lim; nsig += lim;
+            if constexpr (N == 4) {
+                // tiny blocks: test bit and run are read separately (measured faster here)
+                --bits;
+                if (!br.get(1)) break;
+                const int lim = min(N - 1 - nsig, bits);
+                const uint32_t win = br.peek() & ((1u << lim) - 1u);
+                const int z = win != 0u ? __builtin_ctz(win) : lim;
+                const int used = win != 0u ? z + 1 : lim;
+                br.skip(used); bits -= used; nsig += z;
+                x |= 1u << nsig;
+                ++nsig;
+                continue;
             }
+            // one look per segment: the test bit, then the zeros up to the next one bit (cut short
+            // by the budget or by the block's last value, whose one is implied)
+            const uint32_t look = br.peek();
+            if (!(look & 1u)) { br.skip(1); --bits; break; }
+            const int lim = min(N - 1 - nsig, bits - 1);
+            const uint32_t win = (look >> 1) & ((1u << lim) - 1u);
+            const int z = win != 0u ? __builtin_ctz(win) : lim;       // zeros read
+            const int used = 1 + (win != 0u ? z + 1 : lim);
+            br.skip(used); bits -= used; nsig += z;
             x |= 1u << nsig;
             ++nsig;
         }
@@ -372,8 +401,11 @@ __global__ __launch_bounds__(256) void zfp_decode1_kernel(const uint32_t *__rest
 {
     const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (b >= blocks) return;
+    __shared__ uint32_t lds[NW <= 2 ? 1 : (NW + 1) * 256];
+    uint32_t w[NW];
+    load_words<NW>(in + b * NW, w);
     BitReader<NW> br;
-    load_words<NW>(in + b * NW, br.w);
+    br.init(lds, w);
     float f[4];
     decode_block<4, NW>(br, f);
     reinterpret_cast<float4 *>(field)[b] = make_float4(f[0], f[1], f[2], f[3]);
@@ -411,8 +443,11 @@ __global__ __launch_bounds__(256) void zfp_decode2_kernel(const uint32_t *__rest
 {
     const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (b >= blocks) return;
+    __shared__ uint32_t lds[NW <= 2 ? 1 : (NW + 1) * 256];
+    uint32_t w[NW];
+    load_words<NW>(in + b * NW, w);
     BitReader<NW> br;
-    load_words<NW>(in + b * NW, br.w);
+    br.init(lds, w);
     float f[16];
     decode_block<16, NW>(br, f);
     const int64_t by = b / nbx, bx = b - by * nbx;
