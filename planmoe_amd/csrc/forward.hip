@@ -713,7 +713,7 @@ extern "C" int planmoe_forward_int8(const void *x, const void *wg, int dtype, in
     PM_REQUIRE(capacity >= 0 && (int64_t)experts * capacity < (1ll << 31), "planmoe_forward_int8: bad capacity");
     if (fused_check("planmoe_forward_int8", x, wg, dtype, samples, model_dim, experts, top_k, plane_stride)) return 1;
     PM_REQUIRE(indices && locations && gates, "planmoe_forward_int8: NULL routing output");
-    PM_REQUIRE(codes && bias && scale, "planmoe_forward_int8: NULL codec output");
+    PM_REQUIRE((codes && bias && scale) || capacity == 0, "planmoe_forward_int8: NULL codec output");
     PM_REQUIRE((uintptr_t)codes % 8 == 0, "planmoe_forward_int8: codes must be 8-byte aligned");
     PM_REQUIRE(workspace && workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
                "planmoe_forward_int8: workspace too small");
@@ -738,7 +738,7 @@ extern "C" int planmoe_forward_int8_redispatch(const void *x, int dtype, int sam
 {
     PM_REQUIRE(dtype_ok(dtype) && samples >= 1 && experts >= 1 && experts <= 64 && top_k >= 1 && capacity >= 0,
                "planmoe_forward_int8_redispatch: bad arguments");
-    PM_REQUIRE(x && indices && locations && codes && bias && scale && workspace,
+    PM_REQUIRE(x && indices && locations && workspace && ((codes && bias && scale) || capacity == 0),
                "planmoe_forward_int8_redispatch: NULL argument");
     PM_REQUIRE(workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
                "planmoe_forward_int8_redispatch: workspace too small");
