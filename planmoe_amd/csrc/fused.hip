@@ -351,7 +351,14 @@ static int run_dispatch_int8(const char *who, const void *x, int dtype, const fl
     PM_REQUIRE((int64_t)experts * capacity < (1ll << 31), "%s: experts*capacity overflows int32", who);
     PM_REQUIRE((int64_t)samples * top_k < (1ll << 31), "%s: samples*top_k overflows int32", who);
     const int slots = experts * capacity;
-    if (slots == 0) return 0;
+    if (slots == 0) {
+        // every token is dropped: nothing to encode, and no gate receives a gradient
+        if (grad_gates && samples > 0) {
+            fill_u32((uint32_t *)grad_gates, (size_t)(top_k - 1) * plane_stride + samples, 0u, (hipStream_t)stream);
+            PM_LAUNCH_CHECK(who);
+        }
+        return 0;
+    }
     PM_REQUIRE(x || samples == 0, "%s: x is NULL", who);
     PM_REQUIRE(codes && bias && scale, "%s: NULL output", who);
     PM_REQUIRE(workspace && workspace_bytes >= planmoe_dispatch_workspace_bytes(experts, capacity),
@@ -393,7 +400,7 @@ extern "C" int planmoe_combine_bwd_int8(const void *grad_out, const void *expert
                                         uint8_t *codes, void *bias, void *scale, float *grad_gates,
                                         void *workspace, size_t workspace_bytes, void *stream)
 {
-    PM_REQUIRE(gates && expert_out && grad_gates,
+    PM_REQUIRE(gates && grad_gates && (expert_out || (int64_t)experts * capacity == 0),
                "planmoe_combine_bwd_int8: gates, expert_out and grad_gates must not be NULL");
     return run_dispatch_int8("planmoe_combine_bwd_int8", grad_out, dtype, gates, indices, locations,
                              plane_stride, top_k, samples, model_dim, experts, capacity, codes, bias, scale,

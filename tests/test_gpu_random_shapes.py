@@ -96,3 +96,36 @@ def test_zfp_random_fields(nx, ny, dims):
     assert len(want) == n and np.array_equal(stream.cpu().numpy()[:n], want)
     dec = ops.zfp_decompress(stream, nx, ny, dims)
     assert np.array_equal(raw(dec), np_raw(oracle.zfp_decompress(want, ny, nx, dims, 8.0)))
+
+
+@pytest.mark.parametrize("T,M,E,k,cf", _shapes(16, 3))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gated_and_backward_pieces(T, M, E, k, cf, dtype):
+    """Gated dispatch, the gate gradient and the config-4 fusion on random shapes: fp32 results
+    bit for bit against the oracle, bf16 against the stage-by-stage entry points."""
+    from planmoe_amd import ops
+    scores = tie_free_scores(T, E, k, seed=T * 17 + E)
+    idx, loc, gates, _ = oracle.route_topk(scores.numpy(), k, normalize_gate=False)
+    r = ops.route_topk(scores.to(DEV), k, normalize_gate=False)
+    assert np.array_equal(r["locations"].cpu().numpy(), loc) and np.array_equal(raw(r["gates"]), np_raw(gates))
+    C = ops.capacity(T, E, k, cf, 4)
+    g = torch.Generator().manual_seed(M * 3 + T)
+    x = torch.randn(T, M, generator=g).to(dtype)
+    eo = torch.randn(E * C, M, generator=g).to(dtype)
+    xd, eod = x.to(DEV), eo.to(DEV)
+    i, l = list(r["indices"]), list(r["locations"])
+    gt = [t.float() for t in r["gates"]]
+    d = ops.dispatch_fwd(xd, i, l, gt, E, C)                      # gates applied at encode
+    gg = ops.bwd_gate(xd, eod, i, l, C)
+    if dtype == torch.float32:
+        want = oracle.encode(x.numpy(), list(idx), list(loc), [a.astype(np.float32) for a in gates], E, C)
+        assert np.array_equal(raw(d), want.view(np.int32))
+        for j in range(k):
+            w = oracle.bwd_gate(idx[j], loc[j], x.double().numpy(), eo.double().numpy(), C)
+            scale = np.abs(x.double().numpy()).sum(1) * (np.abs(eo.numpy()).max() if eo.numel() else 0) + 1e-30
+            assert (np.abs(gg[j].cpu().numpy() - w) <= 1e-5 * scale).all()
+    # config-4 fusion == gated dispatch -> int8 compress, and its gate gradient == bwd_gate
+    codes, bias, scale_, gg2 = ops.combine_bwd_int8(xd, eod, i, l, gt, E, C)
+    c2, b2, s2 = ops.int8_compress(d)
+    assert torch.equal(codes, c2) and np.array_equal(raw(bias), raw(b2)) and np.array_equal(raw(scale_), raw(s2))
+    assert torch.equal(gg2, gg)
