@@ -269,6 +269,33 @@ int planmoe_zfp_compress(const float *field, int dims, int64_t nx, int64_t ny, d
 int planmoe_zfp_decompress(const void *stream_in, int dims, int64_t nx, int64_t ny, double rate,
                            float *field, void *stream);
 
+/* ---------------------------------------------------------------- GPULZ ("lz") lossless codec
+ * Replaces lz_compress / lz_decompress (custom/compressor/gpulz.cu:408-535), the codec behind
+ * LzCompressor (custom/compressor/lz.cpp:3-60).  The input is taken as 32-bit symbols in blocks
+ * of 2048 bytes (512 symbols); a block holds one flag bit per token (least significant bit
+ * first, 1 = match) and the token bytes: 4 for a literal symbol, 2 (length, offset) for a match
+ * into the 32 symbols before it.  Symbols are compared as floats (gpulz.cu:62): +0 equals -0, a
+ * NaN equals nothing.  Streams are byte-identical to the reference's four tensors:
+ *   flag_offsets, data_offsets   int32 [blocks + 1]   exclusive prefix sums of the per-block sizes
+ *   flags                        uint8 [blocks * 64]  zero beyond flag_offsets[blocks]
+ *   data                         uint8 [blocks * 2048] zero beyond data_offsets[blocks]
+ * with blocks = planmoe_lz_blocks(nbytes).  nbytes must be a multiple of 4 and below 2^31; a
+ * last partial block is coded as if padded with zero symbols (the reference reads past the end
+ * of its input there, gpulz.cu:36-39), and decoding writes only the first nbytes.
+ * Compression runs as one pass with a chained prefix over the blocks (no staging copy of the
+ * token bytes, unlike gpulz.cu:148-211 + 220-258), plus a launch that zeroes the slack. */
+int64_t planmoe_lz_blocks(int64_t nbytes);
+size_t planmoe_lz_workspace_bytes(int64_t nbytes);
+int planmoe_lz_compress(const void *input, int64_t nbytes, int32_t *flag_offsets, int32_t *data_offsets,
+                        uint8_t *flags, uint8_t *data, void *workspace, size_t workspace_bytes,
+                        void *stream);
+/* Streams that this coder cannot have written (offsets out of order, a match that reaches
+ * before its block) never make the kernel read or write out of bounds; the symbols they cover
+ * decode as zero. */
+int planmoe_lz_decompress(void *output, int64_t nbytes, const int32_t *flag_offsets,
+                          const int32_t *data_offsets, const uint8_t *flags, const uint8_t *data,
+                          void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -248,3 +248,32 @@ def zfp_encode_block(block, dims=2, rate=8.0):
         lib().orc_zfp_encode_block_float(_p(_c(block, np.float32)), ctypes.c_int(dims),
                                          ctypes.c_double(rate), _p(out))
     return out
+
+
+# --------------------------------------------------------------------------- GPULZ ("lz") codec
+LZ_BLOCK_BYTES = 2048
+
+
+def lz_compress(x):
+    """x: float32, size a multiple of 512.  Returns (flag_offsets int32 [B+1], data_offsets int32
+    [B+1], flags uint8 [B*64], data uint8 [B*2048]); both byte arrays zero beyond their totals."""
+    x = _c(x, np.float32).reshape(-1)
+    assert x.size % 512 == 0
+    B = x.size // 512
+    fo = np.zeros((B + 1,), np.int32)
+    do = np.zeros((B + 1,), np.int32)
+    flags = np.zeros((B * 64,), np.uint8)
+    data = np.zeros((B * 2048,), np.uint8)
+    lib().orc_lz_compress(_p(x), ctypes.c_int64(B), _p(fo), _p(do), _p(flags), _p(data))
+    return fo, do, flags, data
+
+
+def lz_decompress(flag_offsets, data_offsets, flags, data):
+    fo = _c(flag_offsets, np.int32)
+    B = fo.size - 1
+    out = np.zeros((B * 512,), np.float32)
+    rc = lib().orc_lz_decompress(_p(out), ctypes.c_int64(B), _p(fo), _p(_c(data_offsets, np.int32)),
+                                 _p(_c(flags, np.uint8)), _p(_c(data, np.uint8)))
+    if rc != 0:
+        raise ValueError("lz stream is inconsistent")
+    return out

@@ -622,3 +622,102 @@ ORC_API int orc_zfp_decompress(const uint8_t *in, int dims, int64_t nx, int64_t 
     }
     return 0;
 }
+
+/* ------------------------------------------------------------------ GPULZ ("lz") codec
+ * The lossless codec behind compress_name="lz" (custom/compressor/gpulz.cu).  The input is
+ * cut into blocks of 2048 bytes = 512 float symbols (gpulz.cu:6-14); every block is coded
+ * on its own:
+ *   1. for every position p the matcher of gpulz.cu:46-85 runs over the (at most) 32
+ *      symbols before p and yields one (length, offset) pair;
+ *   2. a greedy left-to-right parse (gpulz.cu:98-127, minEncodeLength = 1 for floats,
+ *      gpulz.cu:448) turns them into tokens: length 0 -> literal (4 bytes), otherwise a
+ *      match (2 bytes: length, offset) that skips `length` symbols; one flag bit per token,
+ *      least significant bit first, 1 = match;
+ *   3. the per-block flag bytes and token bytes are packed back to back in block order, with
+ *      exclusive prefix sums of the per-block sizes as offset tables of blocks+1 entries
+ *      (gpulz.cu:460-494, 220-258).
+ * Symbols are compared as floats (gpulz.cu:62): +0 equals -0 and a NaN equals nothing.
+ */
+enum { LZ_SYMS = 512, LZ_WINDOW = 32 };
+
+static void lz_match_at(const float *blk, int p, int *best_len, int *best_off)
+{
+    int w = p > LZ_WINDOW ? p - LZ_WINDOW : 0;
+    int ahead = p, run = 0, run_off = 0, len = 0, off = 0;
+    while (w < p && ahead < LZ_SYMS) {
+        if (blk[ahead] == blk[w]) {
+            if (run == 0) run_off = ahead - w;
+            ++run;
+            ++ahead;
+        } else {
+            if (run > len) { len = run; off = run_off; }
+            run = 0;
+            ahead = p;
+        }
+        ++w;                                 /* a window symbol is never looked at twice */
+    }
+    if (run > len) { len = run; off = run_off; }
+    *best_len = len;
+    *best_off = off;
+}
+
+/* in: blocks*512 floats.  flag_off, data_off: blocks+1 entries.  flags (blocks*64 bytes) and
+ * data (blocks*2048 bytes) must be zero-initialised; the reference allocates them with
+ * at::zeros (gpulz.cu:425-436) and sends them whole. */
+ORC_API int orc_lz_compress(const float *in, int64_t blocks, int32_t *flag_off, int32_t *data_off,
+                            uint8_t *flags, uint8_t *data)
+{
+    int64_t nf = 0, nd = 0;
+    for (int64_t b = 0; b < blocks; ++b) {
+        const float *blk = in + b * LZ_SYMS;
+        flag_off[b] = (int32_t)nf;
+        data_off[b] = (int32_t)nd;
+        int tokens = 0;
+        for (int p = 0; p < LZ_SYMS;) {
+            int len, off;
+            lz_match_at(blk, p, &len, &off);
+            if (len == 0) {
+                memcpy(data + nd, blk + p, 4);
+                nd += 4;
+                p += 1;
+            } else {
+                data[nd] = (uint8_t)len;
+                data[nd + 1] = (uint8_t)off;
+                nd += 2;
+                flags[nf + tokens / 8] |= (uint8_t)(1u << (tokens % 8));
+                p += len;
+            }
+            ++tokens;
+        }
+        nf += (tokens + 7) / 8;
+    }
+    flag_off[blocks] = (int32_t)nf;
+    data_off[blocks] = (int32_t)nd;
+    return 0;
+}
+
+/* gpulz.cu:263-318: one block at a time, tokens in flag order; a match copies `length`
+ * symbols from `offset` symbols before the position the token starts at. */
+ORC_API int orc_lz_decompress(float *out, int64_t blocks, const int32_t *flag_off,
+                              const int32_t *data_off, const uint8_t *flags, const uint8_t *data)
+{
+    for (int64_t b = 0; b < blocks; ++b) {
+        float *blk = out + b * LZ_SYMS;
+        const uint8_t *d = data + data_off[b];
+        int nflag = flag_off[b + 1] - flag_off[b];
+        int p = 0;
+        for (int t = 0; t < 8 * nflag && p < LZ_SYMS; ++t) {
+            if ((flags[flag_off[b] + t / 8] >> (t % 8)) & 1) {
+                int len = d[0], off = d[1], start = p;
+                d += 2;
+                if (off > start || start + len > LZ_SYMS) return -1;   /* not a stream of this coder */
+                for (int i = 0; i < len; ++i) blk[p++] = blk[start - off + i];
+            } else {
+                memcpy(blk + p, d, 4);
+                d += 4;
+                ++p;
+            }
+        }
+    }
+    return 0;
+}

@@ -222,7 +222,6 @@ __device__ __forceinline__ void gate_tile_lds(const void *__restrict__ x, const 
     const int tid = threadIdx.x, w = tid >> 6, l = lane_id();
     const int m = l & 15, g = l >> 4;
     const int nv = model_dim / V;                    // 16-byte vectors per row
-    const int chunks = (nv + 15) / 16;
 
     RowStats<PLANMOE_BF16, true> st;
     if constexpr (STATS) st.init();

@@ -451,3 +451,43 @@ def zfp_decompress(stream, nx, ny, dims=2, rate=8.0):
     out = torch.empty((ny, nx), dtype=torch.float32, device=stream.device)
     check(lib.planmoe_zfp_decompress(_ptr(stream), dims, nx, ny, float(rate), _ptr(out), _stream(stream)))
     return out
+
+
+# ------------------------------------------------------------------------------ GPULZ ("lz") codec
+LZ_BLOCK_BYTES = 2048
+
+
+def lz_compress(x, workspace=None):
+    """x: any contiguous GPU tensor whose byte size is a multiple of 4 (the reference takes fp32).
+    Returns the reference's four tensors (gpulz.cu:502-507): flag_offsets, data_offsets int32
+    [blocks + 1], flags uint8 [blocks * 64], data uint8 [blocks * 2048]; the byte tensors are zero
+    beyond flag_offsets[-1] / data_offsets[-1].  `workspace` (uint8, lz_workspace_bytes) is
+    allocated when not given; after the call its second 32-bit word is non-zero if the chained
+    prefix gave up waiting (never expected)."""
+    _need_gpu(x, "lz_compress")
+    x = _contig(x, "lz_compress")
+    nbytes = x.numel() * x.element_size()
+    blocks = int(lib.planmoe_lz_blocks(nbytes))
+    dev = x.device
+    flag_offsets = torch.empty((blocks + 1,), dtype=torch.int32, device=dev)
+    data_offsets = torch.empty((blocks + 1,), dtype=torch.int32, device=dev)
+    flags = torch.empty((blocks * 64,), dtype=torch.uint8, device=dev)
+    data = torch.empty((blocks * LZ_BLOCK_BYTES,), dtype=torch.uint8, device=dev)
+    if workspace is None:
+        workspace = _ws(lib.planmoe_lz_workspace_bytes(nbytes), dev)
+    check(lib.planmoe_lz_compress(_ptr(x), nbytes, _ptr(flag_offsets), _ptr(data_offsets), _ptr(flags),
+                                  _ptr(data), _ptr(workspace), workspace.numel(), _stream(x)))
+    return flag_offsets, data_offsets, flags, data
+
+
+def lz_decompress(out, flag_offsets, data_offsets, flags, data):
+    """Decodes into `out` (the reference's lz_decompress writes its first argument, gpulz.cu:510-523)."""
+    _need_gpu(out, "lz_decompress")
+    if not out.is_contiguous():
+        raise PlanMoEError("lz_decompress: out must be contiguous")
+    nbytes = out.numel() * out.element_size()
+    check(lib.planmoe_lz_decompress(_ptr(out), nbytes, _ptr(_contig(flag_offsets, "lz_decompress")),
+                                    _ptr(_contig(data_offsets, "lz_decompress")),
+                                    _ptr(_contig(flags, "lz_decompress")),
+                                    _ptr(_contig(data, "lz_decompress")), _stream(out)))
+    return out

@@ -1,0 +1,154 @@
+"""GPULZ ("lz") codec on the GPU against the CPU oracle: the four stream tensors byte for byte,
+decoding of the oracle's streams, round trips, a ragged tail, and streams no coder wrote."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from planmoe_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def gpu_compress(x_np):
+    x = torch.from_numpy(x_np).to(DEV)
+    ws = torch.empty((max(int(_lib.lib.planmoe_lz_workspace_bytes(x_np.nbytes)), 16),), dtype=torch.uint8, device=DEV)
+    fo, do, flags, data = ops.lz_compress(x, workspace=ws)
+    torch.cuda.synchronize()
+    assert int(ws[:8].view(torch.int32)[1]) == 0, "the chained prefix gave up waiting"
+    return fo, do, flags, data
+
+
+def same_streams(got, want):
+    for g, w, name in zip(got, want, ("flag_offsets", "data_offsets", "flags", "data")):
+        g = g.cpu().numpy()
+        assert g.shape == w.shape, name
+        if not np.array_equal(g, w):
+            bad = int(np.flatnonzero(g != w)[0])
+            raise AssertionError("%s differs first at %d: %d != %d" % (name, bad, g[bad], w[bad]))
+
+
+def check(x_np):
+    x_np = np.ascontiguousarray(x_np, np.float32).reshape(-1)
+    want = oracle.lz_compress(x_np)
+    got = gpu_compress(x_np)
+    same_streams(got, want)
+    out = torch.full((x_np.size,), 7.0, dtype=torch.float32, device=DEV)
+    ops.lz_decompress(out, *got)
+    ref = oracle.lz_decompress(*want)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+    return got
+
+
+def distinct(n, start=1000.0):
+    return (start + np.arange(n)).astype(np.float32)
+
+
+def test_hand_worked_blocks():
+    blocks = [np.full(512, 3.5, np.float32), distinct(512)]
+    for prefix in ([1, 1, 2, 1, 2], [1, 2, 1, 3, 1, 4], [1, 2, 4, 1, 2, 3, 5, 1, 2, 3, 6],
+                   [0.0, -0.0, float('nan'), float('nan')]):
+        b = distinct(512)
+        b[:len(prefix)] = prefix
+        blocks.append(b)
+    tail = distinct(512)
+    tail[510:] = tail[508:510]
+    blocks.append(tail)
+    for b in blocks:
+        check(b)
+    check(np.concatenate(blocks))
+
+
+@pytest.mark.parametrize("alphabet,nblocks,seed", [(2, 9, 0), (3, 64, 1), (8, 200, 2), (64, 1000, 3),
+                                                   (100000, 777, 4)])
+def test_random_alphabets(alphabet, nblocks, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.integers(0, alphabet, size=nblocks * 512).astype(np.float32)
+    check(x)
+
+
+def test_dispatched_buffer_with_empty_slots():
+    # what the codec sees in the layer: rows of activations, some capacity slots all zero
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((4096, 1024)).astype(np.float32)
+    x[rng.random(4096) < 0.3] = 0.0
+    x[100, 17:900] = -0.0
+    x[200, 5] = np.nan
+    x[201, :] = np.inf
+    fo, do, flags, data = check(x)
+    assert int(do[-1]) < x.nbytes                        # the empty slots shrink
+
+
+def test_many_groups_chain():
+    # 40 000 blocks = 5 000 work-groups: the sums travel through many published words
+    rng = np.random.default_rng(6)
+    x = rng.integers(0, 5, size=40000 * 512).astype(np.float32)
+    x[::3] += rng.standard_normal(x[::3].size).astype(np.float32)
+    check(x)
+
+
+@pytest.mark.parametrize("nsym", [1, 8, 511, 513, 512 * 3 + 100, 512 * 17 - 1])
+def test_ragged_tail(nsym):
+    rng = np.random.default_rng(nsym)
+    x = rng.integers(0, 4, size=nsym).astype(np.float32)
+    padded = np.zeros((-(-nsym // 512) * 512,), np.float32)
+    padded[:nsym] = x
+    want = oracle.lz_compress(padded)                    # the tail block is coded as if zero-padded
+    got = gpu_compress(x)
+    same_streams(got, want)
+    out = torch.full((nsym + 8,), 7.0, dtype=torch.float32, device=DEV)
+    ops.lz_decompress(out[:nsym], *got)
+    assert np.array_equal(out[:nsym].cpu().numpy(), x)
+    assert np.all(out[nsym:].cpu().numpy() == 7.0)       # nothing written past the end
+
+
+def test_empty():
+    x = torch.empty((0,), dtype=torch.float32, device=DEV)
+    fo, do, flags, data = ops.lz_compress(x)
+    assert fo.tolist() == [0] and do.tolist() == [0] and flags.numel() == 0 and data.numel() == 0
+    ops.lz_decompress(x, fo, do, flags, data)
+
+
+def test_other_dtypes_are_taken_as_words():
+    rng = np.random.default_rng(8)
+    x = torch.from_numpy(rng.integers(0, 3, size=(64, 1024)).astype(np.float32)).to(DEV).bfloat16()
+    got = ops.lz_compress(x)
+    words = x.cpu().view(torch.int32).numpy().view(np.float32)
+    same_streams(got, oracle.lz_compress(words))
+    out = torch.empty_like(x)
+    ops.lz_decompress(out, *got)
+    assert torch.equal(out.view(torch.int16), x.view(torch.int16))
+
+
+def test_foreign_streams_stay_in_bounds():
+    # nothing a coder wrote: the decoder must neither fault nor touch memory outside `out`
+    rng = np.random.default_rng(9)
+    B = 300
+    for kind in range(3):
+        fo = rng.integers(-50, B * 64 + 50, size=B + 1).astype(np.int32)
+        do = rng.integers(-50, B * 2048 + 50, size=B + 1).astype(np.int32)
+        if kind == 1:
+            fo, do = np.sort(fo), np.sort(do)
+        if kind == 2:
+            fo = (np.arange(B + 1) * 64).astype(np.int32)
+            do = (np.arange(B + 1) * 1500).astype(np.int32)
+        flags = rng.integers(0, 256, size=B * 64).astype(np.uint8)
+        data = rng.integers(0, 256, size=B * 2048).astype(np.uint8)
+        guard = torch.full((B * 512 + 1024,), 7.0, dtype=torch.float32, device=DEV)
+        out = guard[512:512 + B * 512]
+        ops.lz_decompress(out, *[torch.from_numpy(a).to(DEV) for a in (fo, do, flags, data)])
+        torch.cuda.synchronize()
+        g = guard.cpu().numpy()
+        assert np.all(g[:512] == 7.0) and np.all(g[512 + B * 512:] == 7.0)
+    check(np.full(1024, 2.0, np.float32))                # and the device still answers
+
+
+def test_argument_errors():
+    x = torch.zeros((1024,), dtype=torch.float32, device=DEV)
+    with pytest.raises(_lib.PlanMoEError):
+        ops.lz_compress(x, workspace=torch.empty((8,), dtype=torch.uint8, device=DEV))
+    with pytest.raises(_lib.PlanMoEError):
+        ops.lz_compress(torch.zeros((3,), dtype=torch.bfloat16, device=DEV))       # 6 bytes
+    with pytest.raises(_lib.PlanMoEError):
+        ops.lz_compress(torch.zeros((4,), dtype=torch.float32))                    # CPU tensor
