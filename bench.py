@@ -61,7 +61,7 @@ def cpu_baseline(T_sample, M, E, k, cf, x_bits, wg_bits, min_seconds):
     return T_sample * reps / dt, dt, reps
 
 
-def kernel_table():
+def kernel_table(only=None):
     """Every entry point at the full size of its workload (BASELINE configs 1-5): device time over
     back-to-back launches (HIP events) against the algorithmic bytes = inputs read once + outputs
     written once.  One line per entry point; an entry point may be several launches."""
@@ -72,6 +72,8 @@ def kernel_table():
     rows = []
 
     def add(name, cfg, nbytes, fn, iters=20):
+        if only and only not in name:
+            return
         # the calls are recorded into a HIP graph once and the graph is replayed: the Python
         # wrappers (output allocation + ctypes call) are slower than the short kernels
         for _ in range(3):
@@ -152,6 +154,17 @@ def kernel_table():
         st = ops.zfp_compress(f, nx, ny, dims)
         add("zfp_decompress %d-D" % dims, "5", zb, lambda: ops.zfp_decompress(st, nx, ny, dims), iters=5)
 
+    # the same buffer through the lossless codec: as it is (no symbol repeats, nothing shrinks) and
+    # with 30 % of the capacity slots empty (zero rows shrink to 44 bytes per 2048)
+    for label, buf in (("dense", f), ("30% empty", f * (torch.rand(f.shape[0], 1, device=dev) >= 0.3))):
+        buf = buf.contiguous()
+        fo, do, fl, da = ops.lz_compress(buf)
+        used = int(fo[-1]) + int(do[-1]) + 2 * fo.numel() * 4
+        lws = torch.empty((ops.lib.planmoe_lz_workspace_bytes(buf.numel() * 4),), dtype=torch.uint8, device=dev)
+        add("lz_compress %s" % label, "5", buf.numel() * 4 + used, lambda: ops.lz_compress(buf, workspace=lws), iters=5)
+        out = torch.empty_like(buf)
+        add("lz_decompress %s" % label, "5", buf.numel() * 4 + used, lambda: ops.lz_decompress(out, fo, do, fl, da), iters=5)
+
     print("%-30s %-4s %10s %9s %9s %8s %6s" % ("entry point", "cfg", "alg MB", "avg us", "best us", "GB/s", "frac"))
     for name, cfg, nbytes, avg, best in rows:
         gbs = nbytes / avg / 1e3
@@ -171,6 +184,7 @@ def main():
     ap.add_argument("--kernels", action="store_true",
                     help="instead of the JSON line, print a table of every entry point at full size "
                          "(device time, algorithmic bytes, fraction of the HBM peak)")
+    ap.add_argument("--only", default=None, help="with --kernels: only the entry points whose name contains this")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
@@ -178,7 +192,7 @@ def main():
     if args.kernels:
         import __graft_entry__
         __graft_entry__.ensure_built()
-        kernel_table()
+        kernel_table(args.only)
         return
 
     import __graft_entry__

@@ -282,8 +282,9 @@ int planmoe_zfp_decompress(const void *stream_in, int dims, int64_t nx, int64_t 
  * with blocks = planmoe_lz_blocks(nbytes).  nbytes must be a multiple of 4 and below 2^31; a
  * last partial block is coded as if padded with zero symbols (the reference reads past the end
  * of its input there, gpulz.cu:36-39), and decoding writes only the first nbytes.
- * Compression runs as one pass with a chained prefix over the blocks (no staging copy of the
- * token bytes, unlike gpulz.cu:148-211 + 220-258), plus a launch that zeroes the slack. */
+ * Compression sizes every block, scans the sizes in place in the offset tables and then packs
+ * every block at its final offset; there is no full-size staging buffer (gpulz.cu:148-211,
+ * 220-258 have two).  All five pointers must be 16-byte aligned. */
 int64_t planmoe_lz_blocks(int64_t nbytes);
 size_t planmoe_lz_workspace_bytes(int64_t nbytes);
 int planmoe_lz_compress(const void *input, int64_t nbytes, int32_t *flag_offsets, int32_t *data_offsets,

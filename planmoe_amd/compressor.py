@@ -123,14 +123,47 @@ class ZfpCompressor(AbstractCompressor):
         self.comm_ptr.all_to_all(input, output, self.length)
 
 
+class LzCompressor(AbstractCompressor):
+    """compressor/lz.cpp:3-73: GPULZ lossless codec.  compress keeps the four stream tensors and
+    returns its input; all_to_all ships the four tensors whole; decompress decodes into the
+    tensor it is handed (g_output, a zeroed twin of the input).  float32 only, as the
+    reference's data_ptr<float>() (gpulz.cu:15,451)."""
+
+    def compress(self, input):
+        if input.dtype != torch.float32:
+            raise PlanMoEError("LzCompressor: expected scalar type Float but found %s" % input.dtype)
+        x = input.contiguous()
+        (self.flagArrOffsetGlobal, self.compressedDataOffsetGlobal, self.flagArrGlobal,
+         self.compressedDataGlobal) = ops.lz_compress(x)
+        self.g_flagArrOffsetGlobal = torch.empty_like(self.flagArrOffsetGlobal)
+        self.g_compressedDataOffsetGlobal = torch.empty_like(self.compressedDataOffsetGlobal)
+        self.g_flagArrGlobal = torch.empty_like(self.flagArrGlobal)
+        self.g_compressedDataGlobal = torch.empty_like(self.compressedDataGlobal)
+        self.g_output = torch.zeros_like(x)
+        return input
+
+    def decompress(self, input):
+        if input.dtype != torch.float32:
+            raise PlanMoEError("LzCompressor: expected scalar type Float but found %s" % input.dtype)
+        return ops.lz_decompress(input, self.g_flagArrOffsetGlobal, self.g_compressedDataOffsetGlobal,
+                                 self.g_flagArrGlobal, self.g_compressedDataGlobal)
+
+    def all_to_all(self, input, output):
+        for src, dst in ((self.flagArrOffsetGlobal, self.g_flagArrOffsetGlobal),
+                         (self.compressedDataOffsetGlobal, self.g_compressedDataOffsetGlobal),
+                         (self.flagArrGlobal, self.g_flagArrGlobal),
+                         (self.compressedDataGlobal, self.g_compressedDataGlobal)):
+            self.comm_ptr.all_to_all(src, dst, src.numel() * src.element_size())
+
+
 def get_compressor(name, comm_ptr):
-    # custom_kernel.cpp:194-207; "lz" is not part of this build
+    # custom_kernel.cpp:194-207
     if name == "int8":
         return Int8Compressor(comm_ptr)
     if name == "zfp":
         return ZfpCompressor(comm_ptr)
     if name == "lz":
-        raise PlanMoEError("the 'lz' compressor is not part of this build")
+        return LzCompressor(comm_ptr)
     return NoCompressor(comm_ptr)
 
 

@@ -6,6 +6,7 @@
 // One GPU: the comm step copies into g_output on the current stream.
 #include "planmoe/compressor/abstract.h"
 #include "planmoe/compressor/int8.h"
+#include "planmoe/compressor/lz.h"
 #include "planmoe/compressor/no.h"
 #include "planmoe/compressor/zfpc.h"
 #include "planmoe_hip.h"
@@ -145,6 +146,50 @@ void ZfpCompressor::all_to_all(const torch::Tensor &input, const torch::Tensor &
     comm_ptr->all_to_all(input, output, length);
 }
 
+LzCompressor::LzCompressor(std::shared_ptr<AbstractComm> comm_ptr) : AbstractCompressor(comm_ptr) {}
+torch::Tensor LzCompressor::compress(const torch::Tensor &input)
+{
+    CHECK_GPU(input);
+    AT_ASSERTM(input.scalar_type() == at::kFloat, "lz: expected scalar type Float");
+    AT_ASSERTM(comm_ptr->g_world_size == 1, "lz: one slice per rank, and this build runs one rank");
+    const torch::Tensor x = input.contiguous();
+    const int64_t nbytes = (int64_t)x.nbytes();
+    const int64_t blocks = planmoe_lz_blocks(nbytes);
+    const auto i32 = x.options().dtype(at::kInt), u8 = x.options().dtype(at::kByte);
+    flagArrOffsetGlobal        = at::empty({blocks + 1}, i32);
+    compressedDataOffsetGlobal = at::empty({blocks + 1}, i32);
+    flagArrGlobal              = at::empty({blocks * 64}, u8);          // the codec zeroes the slack itself
+    compressedDataGlobal       = at::empty({blocks * 2048}, u8);
+    workspace                  = at::empty({(int64_t)planmoe_lz_workspace_bytes(nbytes)}, u8);
+    PM_CALL(planmoe_lz_compress(x.data_ptr(), nbytes, flagArrOffsetGlobal.data_ptr<int>(),
+                                compressedDataOffsetGlobal.data_ptr<int>(), flagArrGlobal.data_ptr<uint8_t>(),
+                                compressedDataGlobal.data_ptr<uint8_t>(), workspace.data_ptr(),
+                                (size_t)workspace.nbytes(), current_stream()));
+    g_flagArrOffsetGlobal        = at::empty_like(flagArrOffsetGlobal);
+    g_compressedDataOffsetGlobal = at::empty_like(compressedDataOffsetGlobal);
+    g_flagArrGlobal              = at::empty_like(flagArrGlobal);
+    g_compressedDataGlobal       = at::empty_like(compressedDataGlobal);
+    g_output                     = at::zeros_like(x);
+    return input;
+}
+torch::Tensor LzCompressor::decompress(const torch::Tensor &input)
+{
+    CHECK_GPU(input);
+    AT_ASSERTM(input.is_contiguous() && input.scalar_type() == at::kFloat, "lz: expected a contiguous Float tensor");
+    PM_CALL(planmoe_lz_decompress(input.data_ptr(), (int64_t)input.nbytes(), g_flagArrOffsetGlobal.data_ptr<int>(),
+                                  g_compressedDataOffsetGlobal.data_ptr<int>(), g_flagArrGlobal.data_ptr<uint8_t>(),
+                                  g_compressedDataGlobal.data_ptr<uint8_t>(), current_stream()));
+    return input;
+}
+void LzCompressor::all_to_all(const torch::Tensor &, const torch::Tensor &)
+{
+    // lz.cpp:67-73: the four stream tensors travel whole; input / output are not touched
+    comm_ptr->all_to_all(flagArrOffsetGlobal, g_flagArrOffsetGlobal, flagArrOffsetGlobal.nbytes());
+    comm_ptr->all_to_all(compressedDataOffsetGlobal, g_compressedDataOffsetGlobal, compressedDataOffsetGlobal.nbytes());
+    comm_ptr->all_to_all(flagArrGlobal, g_flagArrGlobal, flagArrGlobal.nbytes());
+    comm_ptr->all_to_all(compressedDataGlobal, g_compressedDataGlobal, compressedDataGlobal.nbytes());
+}
+
 // ---------------------------------------------------------------- registry (custom_kernel.cpp:194-288)
 static std::vector<PlanMoEStream> g_streams;          // no comm streams on one GPU
 
@@ -152,7 +197,7 @@ static AbstractCompressor *get_compressor(const std::string &name, std::shared_p
 {
     if (name == "int8") return new Int8Compressor(comm_ptr);
     if (name == "zfp") return new ZfpCompressor(comm_ptr);
-    AT_ASSERTM(name != "lz", "the 'lz' compressor is not part of this build");
+    if (name == "lz") return new LzCompressor(comm_ptr);
     return new NoCompressor(comm_ptr);
 }
 static std::shared_ptr<AbstractComm> get_comm(const std::string &)

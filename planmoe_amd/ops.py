@@ -462,8 +462,7 @@ def lz_compress(x, workspace=None):
     Returns the reference's four tensors (gpulz.cu:502-507): flag_offsets, data_offsets int32
     [blocks + 1], flags uint8 [blocks * 64], data uint8 [blocks * 2048]; the byte tensors are zero
     beyond flag_offsets[-1] / data_offsets[-1].  `workspace` (uint8, lz_workspace_bytes) is
-    allocated when not given; after the call its second 32-bit word is non-zero if the chained
-    prefix gave up waiting (never expected)."""
+    allocated when not given."""
     _need_gpu(x, "lz_compress")
     x = _contig(x, "lz_compress")
     nbytes = x.numel() * x.element_size()

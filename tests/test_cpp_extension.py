@@ -29,7 +29,7 @@ def test_module_surface_and_host_side_errors():
     ck.clear_ptr_lst()
     with pytest.raises(RuntimeError, match="no CPU kernels"):
         ck.invoke_cpu_fp32([torch.zeros(1)], [1, 1, 1], 0)
-    with pytest.raises(RuntimeError, match="lz"):
+    with pytest.raises(RuntimeError, match="GPU tensor"):
         ck.compress_operation(torch.zeros(4, 4, 8), "lz", "naive")
     ck.clear_ptr_lst()
 
@@ -72,6 +72,28 @@ def test_pipeline_through_the_cpp_registry():
     d = ck.decompress_operation(ck.comm_operation(ck.compress_operation(bx, "int8", "pipe")))
     rc, rb, rs = oracle.int8_compress(bf16_bits(bx))
     assert d.dtype == torch.bfloat16 and np.array_equal(raw(d), np_raw(oracle.int8_decompress(rc, rb, rs)))
+
+
+@pytest.mark.gpu
+def test_lz_through_the_cpp_registry():
+    from planmoe_amd import ext
+    ck = ext.load()
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(4, 64, 256, generator=g)
+    x[1] = 0.0                                           # empty capacity slots
+    x = x.to(DEV)
+    ck.clear_ptr_lst()
+    sent = ck.compress_operation(x, "lz", "naive")
+    assert sent.data_ptr() == x.data_ptr()               # lz.cpp:40 returns its input
+    recv = ck.comm_operation(sent)
+    assert recv.data_ptr() != x.data_ptr() and not recv.any()     # g_output = zeros_like (lz.cpp:25)
+    dec = ck.decompress_operation(recv)
+    assert dec.data_ptr() == recv.data_ptr()             # decoded in place (lz.cpp:52-59)
+    assert torch.equal(dec, x)
+    ck.clear_ptr_lst()
+    with pytest.raises(RuntimeError, match="Float"):
+        ck.compress_operation(x.bfloat16(), "lz", "naive")
+    ck.clear_ptr_lst()
 
 
 @pytest.mark.gpu

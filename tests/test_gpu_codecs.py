@@ -218,6 +218,19 @@ def test_compressor_registry_round_trips():
     assert np.array_equal(raw(dec[1]), oracle.int8_decompress(rc, rb, rs).view(np.int32))
     st = oracle.zfp_compress(x.cpu().numpy().reshape(-1, 256), 2)
     assert np.array_equal(raw(dec[2]), oracle.zfp_decompress(st, 256, 256, 2).reshape(4, 64, 256).view(np.int32))
+    # 'lz': the input comes back untouched, the streams travel, the decode fills g_output
+    x[2] = 0.0
+    c = compressor.compress_operation(x, "lz", "naive")
+    assert c is x
+    lz = compressor._compress_ptr_lst[-1]
+    want = oracle.lz_compress(x.cpu().numpy())
+    for got, ref in zip((lz.flagArrOffsetGlobal, lz.compressedDataOffsetGlobal, lz.flagArrGlobal,
+                         lz.compressedDataGlobal), want):
+        assert np.array_equal(got.cpu().numpy(), ref)
+    r = compressor.comm_operation(c)
+    assert r is not x and not r.any()
+    d = compressor.decompress_operation(r)
+    assert d is r and torch.equal(d, x)
     bx = x.bfloat16()
     c = compressor.compress_operation(bx, "int8", "naive")
     d = compressor.decompress_operation(compressor.comm_operation(c))

@@ -154,6 +154,23 @@ def test_moe_layer_trains_with_builtin_ffn():
     assert wg_grad is not None and torch.isfinite(wg_grad).all() and wg_grad.abs().sum() > 0
 
 
+def test_moe_layer_with_the_lossless_codec_equals_no_codec():
+    """compress_name='lz' changes nothing but the sign of a zero: output and gradients equal
+    those of compress_name='no', forward and backward, with two chunks per pass."""
+    import planmoe_amd
+    res = {}
+    for compress in ("no", "lz"):
+        layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 2.0}, 64,
+                                      experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 128},
+                                      seeds=(1, 2, 3), compress_name=compress, a2a_ffn_overlap_degree=2).to(DEV)
+        x = torch.randn(8, 32, 64, generator=torch.Generator().manual_seed(5)).to(DEV).requires_grad_(True)
+        y = layer(x)
+        (y.float().pow(2).mean() + y.l_aux).backward()
+        res[compress] = (y.detach(), x.grad, layer.experts.batched_fc1_w.grad, layer.gates[0].wg.weight.grad)
+    for a, b in zip(res["no"], res["lz"]):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("T,M,E,k,cf,dtype,fp32_gate,use_bias", [
     (1000, 512, 8, 2, 1.25, torch.bfloat16, True, False), (33, 256, 4, 2, 1.0, torch.bfloat16, True, False),
     (4096, 1024, 64, 1, 1.0, torch.bfloat16, True, True), (500, 2048, 2, 2, 1.0, torch.float32, True, False),

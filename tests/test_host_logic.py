@@ -61,8 +61,12 @@ def test_registry_protocol_errors():
     with pytest.raises(PlanMoEError):
         compressor.decompress_operation(ra)
     compressor.clear_ptr_lst()
-    with pytest.raises(PlanMoEError):
-        compressor.get_compressor("lz", compressor.get_comm("naive"))
+    lz = compressor.get_compressor("lz", compressor.get_comm("naive"))
+    assert isinstance(lz, compressor.LzCompressor)
+    with pytest.raises(PlanMoEError, match="GPU"):
+        lz.compress(torch.zeros(4, 4, 8))                # no CPU path
+    with pytest.raises(PlanMoEError, match="Float"):
+        lz.compress(torch.zeros(4, 4, 8, dtype=torch.bfloat16))
 
 
 def test_zfp_compressor_shape_check():
