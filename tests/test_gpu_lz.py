@@ -91,6 +91,27 @@ def test_many_blocks_and_scan_chunks():
     check(x)
 
 
+def test_config5_full_size():
+    """The [16, 8192, 1024] fp32 buffer of config 5 (512 MiB, 262 144 blocks): a quarter of the
+    capacity slots empty, some rows thinned out like an activation after a ReLU, the rest dense.
+    All four stream tensors against the oracle, the decode against the input."""
+    rng = np.random.default_rng(11)
+    R, M = 16 * 8192, 1024
+    x = rng.standard_normal((R, M), dtype=np.float32)
+    kind = rng.random(R)
+    x[kind < 0.25] = 0.0
+    thin = (kind >= 0.25) & (kind < 0.35)
+    x[thin] = np.maximum(x[thin], 0.0)
+    want = oracle.lz_compress(x)
+    xd = torch.from_numpy(x).to(DEV)
+    got = ops.lz_compress(xd)
+    same_streams(got, want)
+    out = torch.empty_like(xd)
+    ops.lz_decompress(out, *got)
+    assert torch.equal(out.view(torch.int32), xd.view(torch.int32))      # no -0 and no NaN in this input
+    assert int(got[1][-1]) < 0.8 * x.nbytes
+
+
 @pytest.mark.parametrize("nsym", [1, 8, 511, 513, 512 * 3 + 100, 512 * 17 - 1])
 def test_ragged_tail(nsym):
     rng = np.random.default_rng(nsym)

@@ -129,3 +129,30 @@ def test_gated_and_backward_pieces(T, M, E, k, cf, dtype):
     c2, b2, s2 = ops.int8_compress(d)
     assert torch.equal(codes, c2) and np.array_equal(raw(bias), raw(b2)) and np.array_equal(raw(scale_), raw(s2))
     assert torch.equal(gg2, gg)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_lz_random_buffers(seed):
+    """GPULZ streams against the oracle on buffers of random size and texture: small alphabets
+    (many matches of every length), runs, dense values, zeros of both signs, a ragged tail."""
+    from planmoe_amd import ops
+    rng = np.random.default_rng(100 + seed)
+    nsym = int(rng.integers(1, 40 * 512))
+    alphabet = int(rng.choice([1, 2, 3, 5, 17, 1000, 10 ** 6]))
+    x = rng.integers(0, alphabet, size=nsym).astype(np.float32)
+    for _ in range(int(rng.integers(0, 6))):                       # runs of one value
+        a = int(rng.integers(0, nsym)); n = int(rng.integers(1, 700))
+        x[a:a + n] = float(rng.choice([0.0, -0.0, 1.5, np.inf]))
+    if seed % 3 == 0:
+        x[rng.integers(0, nsym, size=5)] = np.nan
+    padded = np.zeros((-(-nsym // 512) * 512,), np.float32)
+    padded[:nsym] = x
+    want = oracle.lz_compress(padded)
+    xd = torch.from_numpy(x).to(DEV)
+    got = ops.lz_compress(xd)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w)
+    out = torch.empty_like(xd)
+    ops.lz_decompress(out, *got)
+    ref = oracle.lz_decompress(*want)[:nsym]
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), ref.view(np.uint32))
