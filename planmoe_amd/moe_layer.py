@@ -14,7 +14,9 @@ from . import experts as _experts
 from . import gates as _gates
 from . import losses, ops
 from .fast_dispatch import extract_critical, fast_decode, fast_encode, route
-from .overlap import a2a_ffn_overlap_forward, fused_int8_eligible, fused_int8_forward
+from . import overlap as _overlap
+from .overlap import (a2a_ffn_overlap_forward, fused_gate_eligible, fused_gate_forward, fused_int8_eligible,
+                      fused_int8_forward)
 
 
 class MOELayer(torch.nn.Module):
@@ -154,14 +156,31 @@ class MOELayer(torch.nn.Module):
         cf = gctx.capacity_factor if capacity_factor is None else capacity_factor
         alignment = 4 * self.sharded_count * degree
 
+        noisy = self.training and gctx.gate_noise > 0
+        plain = (self.is_gshard_loss and not self.batch_prioritized_routing and cf > 0)
+        if (plain and not noisy and _overlap.FUSE_GATE and
+                fused_gate_eligible(x, gctx, self.num_global_experts, self.compress_name, degree, self.is_postscore)):
+            # gate GEMM, routing, encode and compress as one two-launch call; decompress + decode
+            # in one pass (same routing and the same bits per stage as the steps below)
+            kk = min(k, self.num_global_experts)
+            cap = ops.capacity(x.size(0), self.num_global_experts, kk, cf, alignment)
+            if self.training:
+                self.save_count = self.save_count + 1
+
+            def expert_fn(expert_input):
+                return self.expert_local(expert_input, original_shape[-reserve_dims:])
+            y, l_aux = fused_gate_forward(x, gctx, kk, cap, self.normalize_gate, expert_fn)
+            l_aux = l_aux.to(torch.float32 if gctx.fp32_gate else x.dtype)
+            y = y.view(list(original_shape)).to(original_dtype)
+            self.l_aux = y.l_aux = l_aux
+            return self.result_func(y) if self.result_func is not None else y
+
         # routing (moe_layer.py:230-256)
         logits = gctx(x)
-        noisy = self.training and gctx.gate_noise > 0
         if noisy:
             logits_w_noise = logits + gctx.gate_noise * torch.randn_like(logits) / self.num_global_experts
         else:
             logits_w_noise = logits
-        plain = (self.is_gshard_loss and not self.batch_prioritized_routing and cf > 0)
         if plain:
             # softmax, top-k, slots, gates and the GShard loss in one routing call
             kk = min(k, self.num_global_experts)

@@ -82,6 +82,8 @@ def a2a_ffn_overlap_forward(input, expert_fn, a2a_ffn_overlap_degree, use_2dh, g
 # Compress.backward decompresses it, overlap.py:19-21, 32-34).  Results are bit-identical to the
 # step-by-step pipeline; FUSE_INT8 = False keeps the reference's structure.
 FUSE_INT8 = True
+# one step further: the gate GEMM and the routing join the send side (planmoe_forward_int8)
+FUSE_GATE = True
 
 
 class _EncodeInt8(torch.autograd.Function):
@@ -122,6 +124,65 @@ class _DecodeInt8(torch.autograd.Function):
         grad_y = ops.int8_decompress(gcodes, gbias, gscale)
         return (grad_y, None, None, None, None, None,
                 *[grad_gates[j].to(g.dtype) for j, g in enumerate(gates)])
+
+
+class _GateRouteEncodeInt8(torch.autograd.Function):
+    """Gate GEMM + softmax / top-k / capacity slots + fast_encode + Compress in the two launches
+    of planmoe_forward_int8, then Decompress.  Outputs: the [E*C, M] tensor the experts see, the
+    gates [k, T] and l_aux (all three differentiable), indices and locations [k, T].
+    Backward: the dispatch gradient as in _EncodeInt8; gates and l_aux go back through
+    planmoe_route_bwd to the logits and from there into x and the gate weight (library GEMMs)."""
+
+    @staticmethod
+    def forward(ctx, x, w, top_k, capacity, fp32_gate, normalize_gate):
+        out = ops.forward_int8(x, w, top_k, capacity, fp32_gate=fp32_gate, normalize_gate=normalize_gate,
+                               want_scores=True, want_counts=True)
+        ctx.save_for_backward(x, w, out["scores"], out["indices"], out["locations"], out["counts"])
+        ctx.capacity, ctx.normalize_gate = capacity, normalize_gate
+        ctx.mark_non_differentiable(out["indices"], out["locations"])
+        y = ops.int8_decompress(out["codes"], out["bias"], out["scale"])
+        return y, out["gates"], out["l_aux"], out["indices"], out["locations"]
+
+    @staticmethod
+    def backward(ctx, grad_y, grad_gates, grad_l_aux, *unused):
+        x, w, scores, indices, locations, counts = ctx.saved_tensors
+        dx = dw = None
+        if grad_y is not None:
+            codes, bias, scale = ops.int8_compress(grad_y.contiguous())
+            dx = ops.combine_int8(codes, bias, scale, list(indices), list(locations), None, x.shape[0], ctx.capacity)
+        if grad_gates is not None or grad_l_aux is not None:
+            if grad_gates is None:
+                grad_gates = torch.zeros((indices.shape[0], x.shape[0]), dtype=scores.dtype, device=x.device)
+            grad_logits = ops.route_bwd(scores, indices, grad_gates.contiguous(), ctx.normalize_gate, grad_l_aux,
+                                        counts if grad_l_aux is not None else None, through_softmax=True)
+            g = grad_logits.to(x.dtype)
+            dw = g.t() @ x
+            dx = g @ w if dx is None else dx + g @ w
+        return dx, dw, None, None, None, None
+
+
+def fused_gate_eligible(x, gate, experts, compress_name, degree, is_postscore):
+    """The whole send side (gate, routing, encode, compress) as planmoe_forward_int8."""
+    from .gates import LinearTopKGate
+    return (fused_int8_eligible(x, compress_name, degree, is_postscore) and type(gate) is LinearTopKGate and
+            experts <= 64 and x.shape[0] >= 1)
+
+
+def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn):
+    """moe_layer's forward from the gate to the combine for the int8 compressor, one chunk, the
+    GShard loss and plain routing.  Returns (output [T, M], l_aux)."""
+    w = gate.wg.weight
+    if w.dtype != x.dtype:
+        w = w.to(x.dtype)
+    experts = w.shape[0]
+    x = x.contiguous()
+    y, gates, l_aux, indices, locations = _GateRouteEncodeInt8.apply(x, w.contiguous(), top_k, capacity,
+                                                                     bool(gate.fp32_gate), bool(normalize_gate))
+    y = expert_fn(y.view(experts, capacity, x.shape[-1]))
+    y = y.reshape(experts * capacity, -1).to(x.dtype)
+    k = indices.shape[0]
+    out = _DecodeInt8.apply(y, indices, locations, experts, capacity, x.shape[0], *[gates[j].float() for j in range(k)])
+    return out, l_aux
 
 
 def fused_int8_eligible(x, compress_name, degree, is_postscore):

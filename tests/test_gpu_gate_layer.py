@@ -300,21 +300,48 @@ def test_moe_layer_fused_int8_path_equals_the_stepwise_pipeline(dtype):
     from planmoe_amd import overlap
     results = []
     for fuse in (True, False):
-        overlap.FUSE_INT8 = fuse
+        overlap.FUSE_INT8, overlap.FUSE_GATE = fuse, False
         try:
-            layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 1.25}, 128,
-                                          experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 64},
-                                          seeds=(1, 2, 3), compress_name='int8').to(DEV).to(dtype)
-            x = torch.randn(6, 50, 128, generator=torch.Generator().manual_seed(5)).to(dtype).to(DEV).requires_grad_(True)
-            y = layer(x)
-            (y.float().pow(2).mean() + y.l_aux.float()).backward()
-            results.append((y.detach(), x.grad.detach(), layer.gates[0].wg.weight.grad.detach(),
-                            layer.experts.batched_fc1_w.grad.detach()))
+            results.append(_layer_pass(planmoe_amd, dtype))
         finally:
-            overlap.FUSE_INT8 = True
+            overlap.FUSE_INT8 = overlap.FUSE_GATE = True
     for a, b in zip(*results):
         assert torch.equal(a, b)
     assert results[0][1].abs().sum() > 0 and results[0][2].abs().sum() > 0
+
+
+def _layer_pass(planmoe_amd, dtype):
+    layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 1.25}, 128,
+                                  experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 64},
+                                  seeds=(1, 2, 3), compress_name='int8').to(DEV).to(dtype)
+    x = torch.randn(6, 50, 128, generator=torch.Generator().manual_seed(5)).to(dtype).to(DEV).requires_grad_(True)
+    y = layer(x)
+    (y.float().pow(2).mean() + y.l_aux.float()).backward()
+    return (y.detach(), x.grad.detach(), layer.gates[0].wg.weight.grad.detach(),
+            layer.experts.batched_fc1_w.grad.detach(), y.l_aux.detach())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_moe_layer_with_the_gate_in_the_fused_send_side(dtype):
+    """The layer's default for compress_name='int8': gate GEMM + routing + encode + compress as
+    planmoe_forward_int8.  Its softmax sums in another order than the stand-alone routing, so
+    the comparison with the staged pipeline is to rounding, forward and backward."""
+    import planmoe_amd
+    from planmoe_amd import overlap
+    assert overlap.FUSE_GATE and overlap.FUSE_INT8
+    fused = _layer_pass(planmoe_amd, dtype)
+    overlap.FUSE_GATE = False
+    try:
+        staged = _layer_pass(planmoe_amd, dtype)
+    finally:
+        overlap.FUSE_GATE = True
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-4
+    for name, a, b in zip(("y", "dx", "dwg", "dfc1", "l_aux"), fused, staged):
+        a, b = a.float(), b.float()
+        assert a.shape == b.shape
+        err = (a - b).abs().max().item()
+        assert err <= tol * max(b.abs().max().item(), 1e-6), (name, err)
+    assert fused[2].abs().sum() > 0
 
 
 def test_moe_layer_prescore_noise_and_load_importance_loss():
