@@ -408,7 +408,7 @@ __global__ __launch_bounds__(LZ_WAVES * WAVE) void lz_place_kernel(
         if (lane == 0) flagw[0] = 0x001ffffeu;
     } else {
         LzBlock b;
-        lz_analyse(raw, sh.keys[wave], lane, b);
+        if (lz_analyse(raw, sh.keys[wave], lane, b) != LZ_GENERAL) return;   // the input changed between the launches
         flag_bytes = b.flag_bytes;
         data_bytes = b.data_bytes;
         if (lane < 16) flagw[lane] = 0;
