@@ -20,6 +20,16 @@
  *        input dtype, exhaustive bf16 sweep, min->0 / max->255 invariants
  *   orc_zfp_*                                        golden bitstreams and decoded fields
  *        from stock libzfp 0.5.5 (serial), cross-decode both ways
+ *   orc_lz_*                                         streams worked out by hand for inputs where
+ *        each rule of the matcher decides the outcome, closed forms for constant and
+ *        all-distinct blocks, round trips through a decoder written from the stream layout
+ *
+ * Parity unpinned (nothing available here fixes it; the tests say so where they touch it):
+ *   the order torch.topk gives equal scores on a GPU (this file: lower expert id first);
+ *   CUDA's multiply-by-reciprocal in the int8 decompress (tolerance-level only);
+ *   equality of the reference's patched CUDA zfp with serial zfp 0.5.5;
+ *   what the reference's lz kernels read past an input whose size is not a multiple of 2048
+ *   bytes (callers of orc_lz_* pad with zeros).
  *
  * Build: gcc -O2 -fPIC -shared -ffp-contract=off -fno-fast-math (see oracle/Makefile).
  */
