@@ -72,7 +72,7 @@ def kernel_table(only=None):
     rows = []
 
     def add(name, cfg, nbytes, fn, iters=20):
-        if only and only not in name:
+        if only and only not in "%s [%s]" % (name, cfg):
             return
         # the calls are recorded into a HIP graph once and the graph is replayed: the Python
         # wrappers (output allocation + ctypes call) are slower than the short kernels
@@ -154,6 +154,16 @@ def kernel_table(only=None):
         st = ops.zfp_compress(f, nx, ny, dims)
         add("zfp_decompress %d-D" % dims, "5", zb, lambda: ops.zfp_decompress(st, nx, ny, dims), iters=5)
 
+    # config 5's send side: 65536 tokens x 1024 fp32, 16 experts, top-2, capacity 8192, into the zfp stream
+    T5, M5, E5, k5 = 65536, 1024, 16, 2
+    C5 = ops.capacity(T5, E5, k5, 1.0, 4)
+    x5 = torch.randn(T5, M5, generator=g).to(dev)
+    r5 = ops.route_topk(torch.softmax(torch.randn(T5, E5, generator=g), 1).to(dev), k5)
+    i5, l5 = list(r5["indices"]), list(r5["locations"])
+    zs = ops.dispatch_zfp(x5, i5, l5, None, E5, C5)
+    add("dispatch_fwd", "5", T5 * M5 * 4 + E5 * C5 * M5 * 4, lambda: ops.dispatch_fwd(x5, i5, l5, None, E5, C5), iters=5)
+    add("dispatch_zfp (fused)", "5", T5 * M5 * 4 + E5 * C5 * M5, lambda: ops.dispatch_zfp(x5, i5, l5, None, E5, C5, out=zs), iters=5)
+
     # the same buffer through the lossless codec: as it is (no symbol repeats, nothing shrinks) and
     # with 30 % of the capacity slots empty (zero rows shrink to 44 bytes per 2048)
     for label, buf in (("dense", f), ("30% empty", f * (torch.rand(f.shape[0], 1, device=dev) >= 0.3))):
@@ -184,7 +194,7 @@ def main():
     ap.add_argument("--kernels", action="store_true",
                     help="instead of the JSON line, print a table of every entry point at full size "
                          "(device time, algorithmic bytes, fraction of the HBM peak)")
-    ap.add_argument("--only", default=None, help="with --kernels: only the entry points whose name contains this")
+    ap.add_argument("--only", default=None, help="with --kernels: only the lines whose 'name [config]' contains this, e.g. lz_ or [5]")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "

@@ -269,6 +269,19 @@ int planmoe_zfp_compress(const float *field, int dims, int64_t nx, int64_t ny, d
 int planmoe_zfp_decompress(const void *stream_in, int dims, int64_t nx, int64_t ny, double rate,
                            float *field, void *stream);
 
+/* fast_encode followed by ZfpCompressor::compress in one pass (GatingEncoder.forward,
+ * fast_dispatch.py:26-29, then zfpc.cpp:23-51; with `gates` also GatingDecoder.backward's scatter,
+ * fast_dispatch.py:69-71, followed by Decompress.backward's compress, overlap.py:32-34): the
+ * stream is that of planmoe_zfp_compress(dims = 2, nx = model_dim, ny = experts * capacity) on
+ * the buffer planmoe_dispatch_fwd would have written, and that buffer never exists.  fp32 only (the
+ * codec reads its field as fp32, zfpc.cpp:31); model_dim and experts * capacity multiples of 4;
+ * gates may be NULL (gate = 1). */
+size_t planmoe_dispatch_zfp_workspace_bytes(int experts, int capacity);
+int planmoe_dispatch_zfp(const float *x, const float *gates, const int32_t *indices,
+                         const int32_t *locations, int64_t plane_stride, int top_k, int samples,
+                         int model_dim, int experts, int capacity, double rate, void *stream_out,
+                         size_t stream_capacity, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------- GPULZ ("lz") lossless codec
  * Replaces lz_compress / lz_decompress (custom/compressor/gpulz.cu:408-535), the codec behind
  * LzCompressor (custom/compressor/lz.cpp:3-60).  The input is taken as 32-bit symbols in blocks

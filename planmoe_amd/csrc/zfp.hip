@@ -457,6 +457,69 @@ __global__ __launch_bounds__(256) void zfp_decode2_kernel(const uint32_t *__rest
         *reinterpret_cast<float4 *>(p + j * nx) = make_float4(f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]);
 }
 
+// ---------------------------------------------------------------- dispatch fused with the 2-D encoder
+// fast_encode followed by ZfpCompressor::compress (fast_dispatch.py:26-29 + zfpc.cpp:23-51) without
+// the [experts * capacity, model_dim] buffer in between: a block of the field is 4 consecutive
+// slot rows x 4 columns, so the encoder fetches its 4 rows from the tokens that fill those slots.
+
+// slot -> token that fills it (-1 = empty: pre-filled) and, for the gated variant, its gate
+__global__ __launch_bounds__(256) void slot_source_mark(int32_t *__restrict__ src, float *__restrict__ sgate,
+                                                       const float *__restrict__ gates,
+                                                       const int32_t *__restrict__ indices,
+                                                       const int32_t *__restrict__ locations, int64_t stride,
+                                                       int top_k, int samples, int experts, int capacity)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= samples * top_k) return;
+    const int j = i / samples, t = i - j * samples;
+    const int64_t o = (int64_t)j * stride + t;
+    const int e = indices[o], l = locations[o];
+    if (e < 0 || e >= experts || l < 0 || l >= capacity) return;
+    const int slot = e * capacity + l;
+    src[slot] = t;
+    if (gates) sgate[slot] = gates[o];
+}
+
+template <int NW, bool GATED>
+__global__ __launch_bounds__(256) void dispatch_zfp2_kernel(const float *__restrict__ x,
+                                                           const int32_t *__restrict__ src,
+                                                           const float *__restrict__ sgate, int64_t model_dim,
+                                                           int64_t nbx, int64_t blocks,
+                                                           uint32_t *__restrict__ out)
+{
+    __shared__ uint32_t lds[NW * 256];
+    __shared__ uint32_t tab[512];
+    group_code_table(tab);
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    const int64_t by = b / nbx, bx = b - by * nbx;
+    const int4 tok = *reinterpret_cast<const int4 *>(src + 4 * by);
+    const int t[4] = {tok.x, tok.y, tok.z, tok.w};
+    float g[4] = {1.f, 1.f, 1.f, 1.f};
+    if constexpr (GATED) {
+        const float4 gv = *reinterpret_cast<const float4 *>(sgate + 4 * by);
+        g[0] = gv.x; g[1] = gv.y; g[2] = gv.z; g[3] = gv.w;
+    }
+    float f[16];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        // straight-line load at a clamped row; an empty slot is a row of zeros
+        const float4 v = *reinterpret_cast<const float4 *>(x + (int64_t)max(t[j], 0) * model_dim + 4 * bx);
+        const bool live = t[j] >= 0;
+        // the dispatch kernel stores 0 + g * x (x itself without gates); the sign of a zero does not
+        // reach the stream
+        f[4 * j] = live ? (GATED ? g[j] * v.x : v.x) : 0.f;
+        f[4 * j + 1] = live ? (GATED ? g[j] * v.y : v.y) : 0.f;
+        f[4 * j + 2] = live ? (GATED ? g[j] * v.z : v.z) : 0.f;
+        f[4 * j + 3] = live ? (GATED ? g[j] * v.w : v.w) : 0.f;
+    }
+    BitWriter<NW> bw;
+    encode_block<16, NW>(f, bw, lds, tab);
+    uint32_t w[NW];
+    bw.words(lds, w);
+    store_words<NW>(out + b * NW, w);
+}
+
 static int zfp_maxbits(int dims, double rate)
 {
     const int n = dims == 1 ? 4 : 16;
@@ -547,5 +610,56 @@ extern "C" int planmoe_zfp_decompress(const void *stream_in, int dims, int64_t n
         else zfp_decode2_kernel<NW><<<grid, 256, 0, st>>>((const uint32_t *)stream_in, nx, nx / 4, blocks, field);
     });
     PM_LAUNCH_CHECK("planmoe_zfp_decompress");
+    return 0;
+}
+
+extern "C" size_t planmoe_dispatch_zfp_workspace_bytes(int experts, int capacity)
+{
+    if (experts <= 0 || capacity <= 0) return 16;
+    return round_up((size_t)experts * (size_t)capacity * 8u, 256);        // slot -> token, slot -> gate
+}
+
+extern "C" int planmoe_dispatch_zfp(const float *x, const float *gates, const int32_t *indices,
+                                    const int32_t *locations, int64_t plane_stride, int top_k, int samples,
+                                    int model_dim, int experts, int capacity, double rate, void *stream_out,
+                                    size_t stream_capacity, void *workspace, size_t workspace_bytes, void *stream)
+{
+    const char *who = "planmoe_dispatch_zfp";
+    PM_REQUIRE((indices && locations) || samples == 0, "%s: indices/locations must not be NULL", who);
+    PM_REQUIRE(top_k >= 1 && samples >= 0 && plane_stride >= samples, "%s: bad routing planes", who);
+    PM_REQUIRE(model_dim >= 1 && experts >= 1 && capacity >= 0, "%s: bad shape", who);
+    PM_REQUIRE((int64_t)experts * capacity < (1ll << 31) && (int64_t)samples * top_k < (1ll << 31),
+               "%s: experts*capacity or samples*top_k overflows int32", who);
+    const int64_t rows = (int64_t)experts * capacity;
+    int nw; int64_t blocks;
+    if (zfp_check(who, 2, model_dim, rows, rate, nw, blocks)) return 1;
+    if (blocks == 0) return 0;
+    PM_REQUIRE((x || samples == 0) && stream_out, "%s: NULL argument", who);
+    PM_REQUIRE(aligned16(x) && aligned16(stream_out), "%s: buffers must be 16-byte aligned", who);
+    const size_t need = planmoe_zfp_stream_bytes(2, model_dim, rows, rate);
+    PM_REQUIRE(stream_capacity >= need, "%s: stream buffer too small (%zu < %zu)", who, stream_capacity, need);
+    hipStream_t st = (hipStream_t)stream;
+    if (samples == 0) {
+        // every slot is empty, and a field of zeros codes as a stream of zeros
+        fill_u32((uint32_t *)stream_out, need / 4, 0u, st);
+        PM_LAUNCH_CHECK(who);
+        return 0;
+    }
+    PM_REQUIRE(workspace && aligned16(workspace) &&
+               workspace_bytes >= planmoe_dispatch_zfp_workspace_bytes(experts, capacity),
+               "%s: workspace too small or not 16-byte aligned", who);
+    int32_t *src = (int32_t *)workspace;
+    float *sgate = (float *)(src + rows);
+    fill_u32((uint32_t *)src, (size_t)rows, 0xffffffffu, st);
+    slot_source_mark<<<(unsigned)(((int64_t)samples * top_k + 255) / 256), 256, 0, st>>>(
+        src, sgate, gates, indices, locations, plane_stride, top_k, samples, experts, capacity);
+    const unsigned grid = (unsigned)((blocks + 255) / 256);
+    PM_NW_SWITCH(nw, NW, {
+        if (gates) dispatch_zfp2_kernel<NW, true><<<grid, 256, 0, st>>>(x, src, sgate, model_dim, model_dim / 4, blocks,
+                                                                       (uint32_t *)stream_out);
+        else dispatch_zfp2_kernel<NW, false><<<grid, 256, 0, st>>>(x, src, sgate, model_dim, model_dim / 4, blocks,
+                                                                  (uint32_t *)stream_out);
+    });
+    PM_LAUNCH_CHECK(who);
     return 0;
 }

@@ -16,7 +16,7 @@ from . import losses, ops
 from .fast_dispatch import extract_critical, fast_decode, fast_encode, route
 from . import overlap as _overlap
 from .overlap import (a2a_ffn_overlap_forward, fused_gate_eligible, fused_gate_forward, fused_int8_eligible,
-                      fused_int8_forward)
+                      fused_int8_forward, fused_zfp_eligible, fused_zfp_forward)
 
 
 class MOELayer(torch.nn.Module):
@@ -212,6 +212,18 @@ class MOELayer(torch.nn.Module):
             def expert_fn(expert_input):
                 return self.expert_local(expert_input, original_shape[-reserve_dims:])
             y = fused_int8_forward(x, crit, expert_fn)
+            y = y.view(list(original_shape)).to(original_dtype)
+            self.l_aux = y.l_aux = l_aux
+            return self.result_func(y) if self.result_func is not None else y
+
+        if fused_zfp_eligible(x, self.compress_name, degree, self.is_postscore, crit[0], crit[4]):
+            # encode + compress in one pass, forward and (with the gates) backward
+            if self.training:
+                self.save_count = self.save_count + 1
+
+            def expert_fn(expert_input):
+                return self.expert_local(expert_input, original_shape[-reserve_dims:])
+            y = fused_zfp_forward(x, crit, expert_fn)
             y = y.view(list(original_shape)).to(original_dtype)
             self.l_aux = y.l_aux = l_aux
             return self.result_func(y) if self.result_func is not None else y

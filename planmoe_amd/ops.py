@@ -453,6 +453,25 @@ def zfp_decompress(stream, nx, ny, dims=2, rate=8.0):
     return out
 
 
+def dispatch_zfp(x, indices, locations, gates, experts, capacity_, rate=8.0, out=None):
+    """fast_encode + zfp_compress (2-D, nx = M, ny = experts * capacity) in one pass: the stream of
+    the dispatched buffer without the buffer.  x: fp32 [T, M].  Returns what zfp_compress returns."""
+    _need_gpu(x, "dispatch_zfp")
+    x = _contig(x, "dispatch_zfp")
+    if x.dtype != torch.float32:
+        raise PlanMoEError("dispatch_zfp: the codec reads its field as fp32; pass a float32 tensor")
+    T, M = x.shape
+    idx, loc, g, stride = _plane_args(indices, locations, gates, "dispatch_zfp")
+    R = experts * capacity_
+    if out is None:
+        out = torch.empty((zfp_max_bytes(2, M, R, rate),), dtype=torch.uint8, device=x.device)
+        out[zfp_stream_bytes(2, M, R, rate):].zero_()
+    ws = _ws(lib.planmoe_dispatch_zfp_workspace_bytes(experts, capacity_), x.device)
+    check(lib.planmoe_dispatch_zfp(_ptr(x), _ptr(g), _ptr(idx), _ptr(loc), stride, len(indices), T, M, experts,
+                                   capacity_, float(rate), _ptr(out), out.numel(), _ptr(ws), ws.numel(), _stream(x)))
+    return out
+
+
 # ------------------------------------------------------------------------------ GPULZ ("lz") codec
 LZ_BLOCK_BYTES = 2048
 

@@ -185,6 +185,75 @@ def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn):
     return out, l_aux
 
 
+# ------------------------------------------------------------------------------ fused zfp send side
+# With the "zfp" compressor (fp32 data) the send side collapses as well: fast_encode + Compress ->
+# planmoe_dispatch_zfp, in the forward pass and, with the gates, in the backward pass of
+# fast_decode.  Decompress and fast_decode stay separate launches.
+class _EncodeZfp(torch.autograd.Function):
+    """Decompress(Comm(Compress(fast_encode(x)))) for the all-ones gate helper (is_postscore)."""
+
+    @staticmethod
+    def forward(ctx, x, indices, locations, experts, capacity):
+        R, M = experts * capacity, x.shape[1]
+        stream = ops.dispatch_zfp(x, list(indices), list(locations), None, experts, capacity)
+        ctx.save_for_backward(indices, locations)
+        ctx.samples, ctx.capacity = x.shape[0], capacity
+        return ops.zfp_decompress(stream, M, R, 2)
+
+    @staticmethod
+    def backward(ctx, grad):
+        indices, locations = ctx.saved_tensors
+        R, M = grad.shape
+        seen = ops.zfp_decompress(ops.zfp_compress(grad.contiguous(), M, R, 2), M, R, 2)
+        dx = ops.combine_fwd(seen, list(indices), list(locations), None, ctx.samples, ctx.capacity)
+        return dx, None, None, None, None
+
+
+class _DecodeZfp(torch.autograd.Function):
+    """fast_decode(Decompress(Comm(Compress(y)))) with the gates applied at decode."""
+
+    @staticmethod
+    def forward(ctx, y, indices, locations, experts, capacity, samples, *gates):
+        R, M = y.shape
+        seen = ops.zfp_decompress(ops.zfp_compress(y.contiguous(), M, R, 2), M, R, 2)
+        ctx.save_for_backward(seen, indices, locations, *gates)
+        ctx.experts, ctx.capacity = experts, capacity
+        return ops.combine_fwd(seen, list(indices), list(locations), list(gates), samples, capacity)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        seen, indices, locations, *gates = ctx.saved_tensors
+        R, M = seen.shape
+        grad_out = grad_out.contiguous()
+        stream = ops.dispatch_zfp(grad_out, list(indices), list(locations), list(gates), ctx.experts, ctx.capacity)
+        grad_y = ops.zfp_decompress(stream, M, R, 2)
+        gg = ops.bwd_gate(grad_out, seen, list(indices), list(locations), ctx.capacity)
+        return (grad_y, None, None, None, None, None, *[gg[j].to(g.dtype) for j, g in enumerate(gates)])
+
+
+FUSE_ZFP = True
+
+
+def fused_zfp_eligible(x, compress_name, degree, is_postscore, experts, capacity):
+    # the conditions under which ZfpCompressor.compress accepts the [E, C, M] buffer (zfpc.cpp:24-31)
+    return (FUSE_ZFP and compress_name == 'zfp' and degree == 1 and is_postscore and x.is_cuda and
+            x.dtype == torch.float32 and x.shape[-1] % 4 == 0 and experts % 4 == 0 and capacity % 4 == 0 and
+            capacity > 0)
+
+
+def fused_zfp_forward(x, crit, expert_fn):
+    """encode -> [codec, comm, codec] -> experts -> [codec, comm, codec] -> decode for one chunk
+    and the zfp compressor.  crit = (experts, indices_s, locations_s, gates_s, capacity)."""
+    experts, indices_s, locations_s, gates_s, capacity = crit
+    indices = torch.stack([t.reshape(-1) for t in indices_s]).to(torch.int32).contiguous()     # [k, T]
+    locations = torch.stack([t.reshape(-1) for t in locations_s]).to(torch.int32).contiguous()
+    y = _EncodeZfp.apply(x.contiguous(), indices, locations, experts, capacity)
+    y = expert_fn(y.view(experts, capacity, x.shape[-1]))
+    y = y.reshape(experts * capacity, -1).to(x.dtype)
+    gates = [g.float() for g in gates_s]
+    return _DecodeZfp.apply(y, indices, locations, experts, capacity, x.shape[0], *gates)
+
+
 def fused_int8_eligible(x, compress_name, degree, is_postscore):
     vec = 4 if x.dtype == torch.float32 else 8
     return (FUSE_INT8 and compress_name == 'int8' and degree == 1 and is_postscore and x.is_cuda and

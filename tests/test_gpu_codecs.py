@@ -299,3 +299,47 @@ def test_combine_int8_equals_decompress_then_combine(T, M, E, k, dtype, gated):
                             [a.cpu().numpy() for a in gates] if gated else None, T, C)
         ref_t = torch.from_numpy(ref).to(dtype)
         assert np.array_equal(raw(got), raw(ref_t))
+
+
+@pytest.mark.parametrize("T,M,E,k,cf,gated", [(1000, 256, 8, 2, 1.25, False), (333, 1024, 16, 2, 0.5, True),
+                                              (64, 4, 4, 4, 1.0, True), (5000, 132, 12, 1, 1.0, False),
+                                              (7, 64, 4, 2, 4.0, True)])
+def test_dispatch_zfp_equals_dispatch_then_compress(T, M, E, k, cf, gated):
+    """planmoe_dispatch_zfp: the stream of the dispatched buffer without the buffer, against the
+    two stages and against the oracle."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(T + M)
+    x = torch.randn(T, M, generator=g)
+    scores = torch.softmax(torch.randn(T, E, generator=g), dim=1)
+    r = ops.route_topk(scores.to(DEV), k)
+    C = ops.capacity(T, E, k, cf, 4)
+    idx, loc = list(r["indices"]), list(r["locations"])
+    gates = list(r["gates"]) if gated else None
+    xd = x.to(DEV)
+    got = ops.dispatch_zfp(xd, idx, loc, gates, E, C)
+    staged = ops.zfp_compress(ops.dispatch_fwd(xd, idx, loc, gates, E, C), M, E * C, 2)
+    assert torch.equal(got, staged)
+    n = ops.zfp_stream_bytes(2, M, E * C)
+    d = oracle.encode(x.numpy(), list(r["indices"].cpu().numpy()), list(r["locations"].cpu().numpy()),
+                      list(r["gates"].cpu().numpy()) if gated else None, E, C)
+    assert np.array_equal(got.cpu().numpy()[:n], oracle.zfp_compress(d.reshape(E * C, M), 2))
+
+
+def test_dispatch_zfp_edge_cases():
+    from planmoe_amd import ops
+    from planmoe_amd._lib import PlanMoEError
+    x = torch.randn(16, 64, device=DEV)
+    idx = [torch.zeros(16, dtype=torch.int32, device=DEV)]
+    loc = [torch.arange(16, dtype=torch.int32, device=DEV)]
+    # every token dropped (capacity 0): nothing to code
+    assert ops.dispatch_zfp(x, idx, loc, None, 4, 0).numel() == ops.zfp_max_bytes(2, 64, 0)
+    # no token at all: a field of zeros
+    e = torch.empty((0, 64), device=DEV)
+    none = [torch.empty((0,), dtype=torch.int32, device=DEV)]
+    out = ops.dispatch_zfp(e, none, none, None, 4, 8)
+    assert not out.any()
+    assert torch.equal(out, ops.zfp_compress(torch.zeros(32, 64, device=DEV), 64, 32, 2))
+    with pytest.raises(PlanMoEError, match="zfp fails."):
+        ops.dispatch_zfp(x, idx, loc, None, 3, 2)                      # 6 slot rows
+    with pytest.raises(PlanMoEError):
+        ops.dispatch_zfp(x.bfloat16(), idx, loc, None, 4, 8)

@@ -310,6 +310,30 @@ def test_moe_layer_fused_int8_path_equals_the_stepwise_pipeline(dtype):
     assert results[0][1].abs().sum() > 0 and results[0][2].abs().sum() > 0
 
 
+def test_moe_layer_fused_zfp_send_side_equals_the_stepwise_pipeline():
+    """compress_name='zfp' (fp32): fast_encode + compress as planmoe_dispatch_zfp in forward and in
+    the backward of fast_decode -- outputs and every gradient bit for bit against the steps."""
+    import planmoe_amd
+    from planmoe_amd import overlap
+    results = []
+    for fuse in (True, False):
+        overlap.FUSE_ZFP = fuse
+        try:
+            layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 1.25}, 128,
+                                          experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 64},
+                                          seeds=(1, 2, 3), compress_name='zfp').to(DEV)
+            x = torch.randn(6, 50, 128, generator=torch.Generator().manual_seed(5)).to(DEV).requires_grad_(True)
+            y = layer(x)
+            (y.pow(2).mean() + y.l_aux).backward()
+            results.append((y.detach(), x.grad.detach(), layer.gates[0].wg.weight.grad.detach(),
+                            layer.experts.batched_fc1_w.grad.detach()))
+        finally:
+            overlap.FUSE_ZFP = True
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    assert results[0][1].abs().sum() > 0 and results[0][2].abs().sum() > 0
+
+
 def _layer_pass(planmoe_amd, dtype):
     layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 1.25}, 128,
                                   experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 64},
