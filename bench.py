@@ -161,7 +161,12 @@ def kernel_table(only=None):
     r5 = ops.route_topk(torch.softmax(torch.randn(T5, E5, generator=g), 1).to(dev), k5)
     i5, l5 = list(r5["indices"]), list(r5["locations"])
     zs = ops.dispatch_zfp(x5, i5, l5, None, E5, C5)
+    g5 = [t.float() for t in r5["gates"]]
+    d5 = ops.zfp_decompress(zs, M5, E5 * C5, 2)
     add("dispatch_fwd", "5", T5 * M5 * 4 + E5 * C5 * M5 * 4, lambda: ops.dispatch_fwd(x5, i5, l5, None, E5, C5), iters=5)
+    add("combine_fwd", "5", 3 * T5 * M5 * 4, lambda: ops.combine_fwd(d5, i5, l5, g5, T5, C5), iters=5)
+    add("combine_zfp (fused)", "5", E5 * C5 * M5 + T5 * M5 * 4,
+        lambda: ops.combine_zfp(zs, i5, l5, g5, T5, E5, C5, M5), iters=5)
     add("dispatch_zfp (fused)", "5", T5 * M5 * 4 + E5 * C5 * M5, lambda: ops.dispatch_zfp(x5, i5, l5, None, E5, C5, out=zs), iters=5)
 
     # the same buffer through the lossless codec: as it is (no symbol repeats, nothing shrinks) and

@@ -282,6 +282,18 @@ int planmoe_dispatch_zfp(const float *x, const float *gates, const int32_t *indi
                          int model_dim, int experts, int capacity, double rate, void *stream_out,
                          size_t stream_capacity, void *workspace, size_t workspace_bytes, void *stream);
 
+/* ZfpCompressor::decompress followed by fast_decode in one pass (zfpc.cpp:66-86, then
+ * GatingDecoder.forward, fast_dispatch.py:59-64; without gates GatingEncoder.backward's gather,
+ * fast_dispatch.py:33-38): out[t] = sum over the choices of token t, left to right, of
+ * gate * (decoded slot row), bit for bit what planmoe_zfp_decompress + planmoe_combine_fwd give,
+ * and the decoded buffer never exists (empty slots are not even decoded).  fp32, 2-D stream with
+ * nx = model_dim, ny = experts * capacity; gates may be NULL (gate = 1).  2 + 2 * top_k launches. */
+size_t planmoe_combine_zfp_workspace_bytes(int experts, int capacity);
+int planmoe_combine_zfp(const void *stream_in, double rate, const float *gates, const int32_t *indices,
+                        const int32_t *locations, int64_t plane_stride, int top_k, int samples,
+                        int model_dim, int experts, int capacity, float *out, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------- GPULZ ("lz") lossless codec
  * Replaces lz_compress / lz_decompress (custom/compressor/gpulz.cu:408-535), the codec behind
  * LzCompressor (custom/compressor/lz.cpp:3-60).  The input is taken as 32-bit symbols in blocks

@@ -464,6 +464,7 @@ __global__ __launch_bounds__(256) void zfp_decode2_kernel(const uint32_t *__rest
 
 // slot -> token that fills it (-1 = empty: pre-filled) and, for the gated variant, its gate
 __global__ __launch_bounds__(256) void slot_source_mark(int32_t *__restrict__ src, float *__restrict__ sgate,
+                                                       int32_t *__restrict__ splane,
                                                        const float *__restrict__ gates,
                                                        const int32_t *__restrict__ indices,
                                                        const int32_t *__restrict__ locations, int64_t stride,
@@ -478,6 +479,7 @@ __global__ __launch_bounds__(256) void slot_source_mark(int32_t *__restrict__ sr
     const int slot = e * capacity + l;
     src[slot] = t;
     if (gates) sgate[slot] = gates[o];
+    if (splane) splane[slot] = j;
 }
 
 template <int NW, bool GATED>
@@ -518,6 +520,83 @@ __global__ __launch_bounds__(256) void dispatch_zfp2_kernel(const float *__restr
     uint32_t w[NW];
     bw.words(lds, w);
     store_words<NW>(out + b * NW, w);
+}
+
+// ---------------------------------------------------------------- 2-D decoder fused with combine
+// ZfpCompressor::decompress followed by fast_decode (zfpc.cpp:66-86 + fast_dispatch.py:59-64)
+// without the decoded [experts * capacity, model_dim] buffer: a decoded block holds 4 slot rows,
+// and every row goes to the token that owns the slot.  The reference adds the choices of a token
+// left to right, so one launch per choice plane: plane 0 stores gate * row, plane j adds to what
+// is there; blocks without a row of the plane leave before decoding (the slots of an expert are
+// filled plane after plane, so almost every block belongs to one plane), and empty slots are
+// never decoded.  A small launch per plane gives the tokens whose choice was dropped the
+// reference's "+ 0" (a zero row for plane 0).
+template <int NW>
+__global__ __launch_bounds__(256) void combine_zfp2_kernel(const uint32_t *__restrict__ in,
+                                                          const int32_t *__restrict__ src,
+                                                          const float *__restrict__ sgate,
+                                                          const int32_t *__restrict__ splane, int plane,
+                                                          int64_t model_dim, int64_t nbx, int64_t blocks,
+                                                          float *__restrict__ out)
+{
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    __shared__ uint32_t lds[NW <= 2 ? 1 : (NW + 1) * 256];
+    const int64_t by = b / nbx, bx = b - by * nbx;
+    const int4 tok = *reinterpret_cast<const int4 *>(src + 4 * by);
+    const int4 pl = *reinterpret_cast<const int4 *>(splane + 4 * by);
+    const int t[4] = {tok.x, tok.y, tok.z, tok.w};
+    const bool mine[4] = {tok.x >= 0 && pl.x == plane, tok.y >= 0 && pl.y == plane,
+                          tok.z >= 0 && pl.z == plane, tok.w >= 0 && pl.w == plane};
+    if (!(mine[0] || mine[1] || mine[2] || mine[3])) return;
+    float g[4] = {1.f, 1.f, 1.f, 1.f};
+    if (sgate) {
+        const float4 gv = *reinterpret_cast<const float4 *>(sgate + 4 * by);
+        g[0] = gv.x; g[1] = gv.y; g[2] = gv.z; g[3] = gv.w;
+    }
+    // what is there so far, requested before the decode (straight-line loads at clamped rows)
+    float4 acc[4];
+    if (plane > 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            acc[j] = *reinterpret_cast<const float4 *>(out + (int64_t)max(t[j], 0) * model_dim + 4 * bx);
+    }
+    uint32_t w[NW];
+    load_words<NW>(in + b * NW, w);
+    BitReader<NW> br;
+    br.init(lds, w);
+    float f[16];
+    decode_block<16, NW>(br, f);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (!mine[j]) continue;
+        float4 v = make_float4(g[j] * f[4 * j], g[j] * f[4 * j + 1], g[j] * f[4 * j + 2], g[j] * f[4 * j + 3]);
+        if (plane > 0) v = make_float4(acc[j].x + v.x, acc[j].y + v.y, acc[j].z + v.z, acc[j].w + v.w);
+        *reinterpret_cast<float4 *>(out + (int64_t)t[j] * model_dim + 4 * bx) = v;
+    }
+}
+
+// tokens whose choice `plane` takes no slot: a zero row (plane 0) or row + 0 (later planes)
+__global__ __launch_bounds__(256) void combine_dropped_kernel(const int32_t *__restrict__ indices,
+                                                             const int32_t *__restrict__ locations,
+                                                             int64_t stride, int plane, int samples,
+                                                             int model_dim, int experts, int capacity,
+                                                             float *__restrict__ out)
+{
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= samples) return;
+    const int64_t o = (int64_t)plane * stride + t;
+    const int e = indices[o], l = locations[o];
+    if (e >= 0 && e < experts && l >= 0 && l < capacity) return;
+    float4 *row = reinterpret_cast<float4 *>(out + (int64_t)t * model_dim);
+    for (int u = lane_id(); u < model_dim / 4; u += WAVE) {
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (plane > 0) {
+            v = row[u];
+            v = make_float4(v.x + 0.f, v.y + 0.f, v.z + 0.f, v.w + 0.f);
+        }
+        row[u] = v;
+    }
 }
 
 static int zfp_maxbits(int dims, double rate)
@@ -652,7 +731,7 @@ extern "C" int planmoe_dispatch_zfp(const float *x, const float *gates, const in
     float *sgate = (float *)(src + rows);
     fill_u32((uint32_t *)src, (size_t)rows, 0xffffffffu, st);
     slot_source_mark<<<(unsigned)(((int64_t)samples * top_k + 255) / 256), 256, 0, st>>>(
-        src, sgate, gates, indices, locations, plane_stride, top_k, samples, experts, capacity);
+        src, sgate, nullptr, gates, indices, locations, plane_stride, top_k, samples, experts, capacity);
     const unsigned grid = (unsigned)((blocks + 255) / 256);
     PM_NW_SWITCH(nw, NW, {
         if (gates) dispatch_zfp2_kernel<NW, true><<<grid, 256, 0, st>>>(x, src, sgate, model_dim, model_dim / 4, blocks,
@@ -660,6 +739,57 @@ extern "C" int planmoe_dispatch_zfp(const float *x, const float *gates, const in
         else dispatch_zfp2_kernel<NW, false><<<grid, 256, 0, st>>>(x, src, sgate, model_dim, model_dim / 4, blocks,
                                                                   (uint32_t *)stream_out);
     });
+    PM_LAUNCH_CHECK(who);
+    return 0;
+}
+
+extern "C" size_t planmoe_combine_zfp_workspace_bytes(int experts, int capacity)
+{
+    if (experts <= 0 || capacity <= 0) return 16;
+    return round_up((size_t)experts * (size_t)capacity * 12u, 256);       // slot -> token, gate, plane
+}
+
+extern "C" int planmoe_combine_zfp(const void *stream_in, double rate, const float *gates,
+                                   const int32_t *indices, const int32_t *locations, int64_t plane_stride,
+                                   int top_k, int samples, int model_dim, int experts, int capacity,
+                                   float *out, void *workspace, size_t workspace_bytes, void *stream)
+{
+    const char *who = "planmoe_combine_zfp";
+    PM_REQUIRE((indices && locations) || samples == 0, "%s: indices/locations must not be NULL", who);
+    PM_REQUIRE(top_k >= 1 && samples >= 0 && plane_stride >= samples, "%s: bad routing planes", who);
+    PM_REQUIRE(model_dim >= 1 && experts >= 1 && capacity >= 0, "%s: bad shape", who);
+    PM_REQUIRE((int64_t)experts * capacity < (1ll << 31) && (int64_t)samples * top_k < (1ll << 31),
+               "%s: experts*capacity or samples*top_k overflows int32", who);
+    const int64_t rows = (int64_t)experts * capacity;
+    int nw; int64_t blocks;
+    if (zfp_check(who, 2, model_dim, rows, rate, nw, blocks)) return 1;
+    if (samples == 0) return 0;
+    PM_REQUIRE(out && aligned16(out), "%s: out must be a 16-byte aligned buffer", who);
+    hipStream_t st = (hipStream_t)stream;
+    if (blocks == 0) {                                  // no slot at all: every token row is zero
+        fill_u32((uint32_t *)out, (size_t)samples * model_dim, 0u, st);
+        PM_LAUNCH_CHECK(who);
+        return 0;
+    }
+    PM_REQUIRE(stream_in && aligned16(stream_in), "%s: the stream must be a 16-byte aligned buffer", who);
+    PM_REQUIRE(workspace && aligned16(workspace) &&
+               workspace_bytes >= planmoe_combine_zfp_workspace_bytes(experts, capacity),
+               "%s: workspace too small or not 16-byte aligned", who);
+    int32_t *src = (int32_t *)workspace;
+    float *sgate = (float *)(src + rows);
+    int32_t *splane = (int32_t *)(sgate + rows);
+    fill_u32((uint32_t *)src, (size_t)rows, 0xffffffffu, st);
+    slot_source_mark<<<(unsigned)(((int64_t)samples * top_k + 255) / 256), 256, 0, st>>>(
+        src, sgate, splane, gates, indices, locations, plane_stride, top_k, samples, experts, capacity);
+    const unsigned grid = (unsigned)((blocks + 255) / 256);
+    for (int j = 0; j < top_k; ++j) {
+        PM_NW_SWITCH(nw, NW, {
+            combine_zfp2_kernel<NW><<<grid, 256, 0, st>>>((const uint32_t *)stream_in, src, gates ? sgate : nullptr,
+                                                         splane, j, model_dim, model_dim / 4, blocks, out);
+        });
+        combine_dropped_kernel<<<(unsigned)((samples + 3) / 4), 256, 0, st>>>(indices, locations, plane_stride, j,
+                                                                            samples, model_dim, experts, capacity, out);
+    }
     PM_LAUNCH_CHECK(who);
     return 0;
 }

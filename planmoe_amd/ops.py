@@ -472,6 +472,20 @@ def dispatch_zfp(x, indices, locations, gates, experts, capacity_, rate=8.0, out
     return out
 
 
+def combine_zfp(stream, indices, locations, gates, samples, experts, capacity_, model_dim, rate=8.0):
+    """zfp_decompress (2-D, nx = model_dim, ny = experts * capacity) + fast_decode in one pass:
+    [T, model_dim] fp32 straight from the stream."""
+    _need_gpu(stream, "combine_zfp")
+    stream = _contig(stream, "combine_zfp")
+    idx, loc, g, stride = _plane_args(indices, locations, gates, "combine_zfp")
+    out = torch.empty((samples, model_dim), dtype=torch.float32, device=stream.device)
+    ws = _ws(lib.planmoe_combine_zfp_workspace_bytes(experts, capacity_), stream.device)
+    check(lib.planmoe_combine_zfp(_ptr(stream), float(rate), _ptr(g), _ptr(idx), _ptr(loc), stride, len(indices),
+                                  samples, model_dim, experts, capacity_, _ptr(out), _ptr(ws), ws.numel(),
+                                  _stream(stream)))
+    return out
+
+
 # ------------------------------------------------------------------------------ GPULZ ("lz") codec
 LZ_BLOCK_BYTES = 2048
 

@@ -185,10 +185,11 @@ def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn):
     return out, l_aux
 
 
-# ------------------------------------------------------------------------------ fused zfp send side
-# With the "zfp" compressor (fp32 data) the send side collapses as well: fast_encode + Compress ->
-# planmoe_dispatch_zfp, in the forward pass and, with the gates, in the backward pass of
-# fast_decode.  Decompress and fast_decode stay separate launches.
+# ------------------------------------------------------------------------------ fused zfp path
+# With the "zfp" compressor (fp32 data) both sides collapse as well: fast_encode + Compress ->
+# planmoe_dispatch_zfp (forward pass and, with the gates, the backward pass of fast_decode);
+# Decompress + fast_decode -> planmoe_combine_zfp (forward pass and the backward pass of
+# fast_encode).  Bit-identical to the steps.
 class _EncodeZfp(torch.autograd.Function):
     """Decompress(Comm(Compress(fast_encode(x)))) for the all-ones gate helper (is_postscore)."""
 
@@ -197,36 +198,38 @@ class _EncodeZfp(torch.autograd.Function):
         R, M = experts * capacity, x.shape[1]
         stream = ops.dispatch_zfp(x, list(indices), list(locations), None, experts, capacity)
         ctx.save_for_backward(indices, locations)
-        ctx.samples, ctx.capacity = x.shape[0], capacity
+        ctx.samples, ctx.experts, ctx.capacity = x.shape[0], experts, capacity
         return ops.zfp_decompress(stream, M, R, 2)
 
     @staticmethod
     def backward(ctx, grad):
         indices, locations = ctx.saved_tensors
         R, M = grad.shape
-        seen = ops.zfp_decompress(ops.zfp_compress(grad.contiguous(), M, R, 2), M, R, 2)
-        dx = ops.combine_fwd(seen, list(indices), list(locations), None, ctx.samples, ctx.capacity)
+        stream = ops.zfp_compress(grad.contiguous(), M, R, 2)
+        dx = ops.combine_zfp(stream, list(indices), list(locations), None, ctx.samples, ctx.experts, ctx.capacity, M)
         return dx, None, None, None, None
 
 
 class _DecodeZfp(torch.autograd.Function):
-    """fast_decode(Decompress(Comm(Compress(y)))) with the gates applied at decode."""
+    """fast_decode(Decompress(Comm(Compress(y)))) with the gates applied at decode.  The decoded
+    buffer is not kept: the backward pass decodes the saved stream (a quarter of its size) again."""
 
     @staticmethod
     def forward(ctx, y, indices, locations, experts, capacity, samples, *gates):
         R, M = y.shape
-        seen = ops.zfp_decompress(ops.zfp_compress(y.contiguous(), M, R, 2), M, R, 2)
-        ctx.save_for_backward(seen, indices, locations, *gates)
-        ctx.experts, ctx.capacity = experts, capacity
-        return ops.combine_fwd(seen, list(indices), list(locations), list(gates), samples, capacity)
+        stream = ops.zfp_compress(y.contiguous(), M, R, 2)
+        ctx.save_for_backward(stream, indices, locations, *gates)
+        ctx.experts, ctx.capacity, ctx.shape = experts, capacity, (R, M)
+        return ops.combine_zfp(stream, list(indices), list(locations), list(gates), samples, experts, capacity, M)
 
     @staticmethod
     def backward(ctx, grad_out):
-        seen, indices, locations, *gates = ctx.saved_tensors
-        R, M = seen.shape
+        stream, indices, locations, *gates = ctx.saved_tensors
+        R, M = ctx.shape
         grad_out = grad_out.contiguous()
-        stream = ops.dispatch_zfp(grad_out, list(indices), list(locations), list(gates), ctx.experts, ctx.capacity)
-        grad_y = ops.zfp_decompress(stream, M, R, 2)
+        seen = ops.zfp_decompress(stream, M, R, 2)              # the tensor fast_decode consumed
+        gstream = ops.dispatch_zfp(grad_out, list(indices), list(locations), list(gates), ctx.experts, ctx.capacity)
+        grad_y = ops.zfp_decompress(gstream, M, R, 2)
         gg = ops.bwd_gate(grad_out, seen, list(indices), list(locations), ctx.capacity)
         return (grad_y, None, None, None, None, None, *[gg[j].to(g.dtype) for j, g in enumerate(gates)])
 

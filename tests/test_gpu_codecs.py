@@ -343,3 +343,44 @@ def test_dispatch_zfp_edge_cases():
         ops.dispatch_zfp(x, idx, loc, None, 3, 2)                      # 6 slot rows
     with pytest.raises(PlanMoEError):
         ops.dispatch_zfp(x.bfloat16(), idx, loc, None, 4, 8)
+
+
+@pytest.mark.parametrize("T,M,E,k,cf,gated", [(1000, 256, 8, 2, 1.25, True), (333, 1024, 16, 2, 0.5, True),
+                                              (64, 4, 4, 4, 1.0, True), (5000, 132, 12, 1, 1.0, False),
+                                              (7, 64, 4, 2, 4.0, False), (900, 64, 4, 3, 0.25, True)])
+def test_combine_zfp_equals_decompress_then_combine(T, M, E, k, cf, gated):
+    """planmoe_combine_zfp: the token rows straight from the stream, bit for bit what the two
+    stages give (dropped choices, empty slots, gates of both signs, zero rows)."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(T * 3 + M)
+    scores = torch.softmax(torch.randn(T, E, generator=g), dim=1)
+    r = ops.route_topk(scores.to(DEV), k)
+    C = ops.capacity(T, E, k, cf, 4)
+    idx, loc = list(r["indices"]), list(r["locations"])
+    gates = None
+    if gated:
+        gates = [(torch.randn(T, generator=g) * (torch.rand(T, generator=g) > 0.1)).to(DEV) for _ in range(k)]
+    y = torch.randn(E * C, M, generator=g)
+    y[::7] = 0.0
+    stream = ops.zfp_compress(y.to(DEV), M, E * C, 2)
+    got = ops.combine_zfp(stream, idx, loc, gates, T, E, C, M)
+    dec = ops.zfp_decompress(stream, M, E * C, 2)
+    want = ops.combine_fwd(dec, idx, loc, gates, T, C)
+    assert np.array_equal(raw(got), raw(want))
+    ref = oracle.decode(oracle.zfp_decompress(stream.cpu().numpy()[:ops.zfp_stream_bytes(2, M, E * C)], E * C, M, 2),
+                        list(r["indices"].cpu().numpy()), list(r["locations"].cpu().numpy()),
+                        [t.cpu().numpy() for t in gates] if gated else None, T, C)
+    assert np.array_equal(raw(got), ref.view(np.int32))
+
+
+def test_combine_zfp_edge_cases():
+    from planmoe_amd import ops
+    idx = [torch.zeros(16, dtype=torch.int32, device=DEV)]
+    loc = [torch.arange(16, dtype=torch.int32, device=DEV)]
+    none = torch.empty((0,), dtype=torch.uint8, device=DEV)
+    out = ops.combine_zfp(ops.zfp_compress(torch.empty((0, 64), device=DEV), 64, 0, 2), idx, loc, None, 16, 4, 0, 64)
+    assert out.shape == (16, 64) and not out.any()                        # capacity 0: every token dropped
+    e = [torch.empty((0,), dtype=torch.int32, device=DEV)]
+    stream = ops.zfp_compress(torch.randn(32, 64, device=DEV), 64, 32, 2)
+    assert ops.combine_zfp(stream, e, e, None, 0, 4, 8, 64).shape == (0, 64)
+    del none
