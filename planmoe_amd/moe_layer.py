@@ -169,7 +169,7 @@ class MOELayer(torch.nn.Module):
 
             def expert_fn(expert_input):
                 return self.expert_local(expert_input, original_shape[-reserve_dims:])
-            y, l_aux = fused_gate_forward(x, gctx, kk, cap, self.normalize_gate, expert_fn)
+            y, l_aux = fused_gate_forward(x, gctx, kk, cap, self.normalize_gate, expert_fn, degree)
             l_aux = l_aux.to(torch.float32 if gctx.fp32_gate else x.dtype)
             y = y.view(list(original_shape)).to(original_dtype)
             self.l_aux = y.l_aux = l_aux
@@ -211,7 +211,7 @@ class MOELayer(torch.nn.Module):
 
             def expert_fn(expert_input):
                 return self.expert_local(expert_input, original_shape[-reserve_dims:])
-            y = fused_int8_forward(x, crit, expert_fn)
+            y = fused_int8_forward(x, crit, expert_fn, degree)
             y = y.view(list(original_shape)).to(original_dtype)
             self.l_aux = y.l_aux = l_aux
             return self.result_func(y) if self.result_func is not None else y
@@ -223,7 +223,7 @@ class MOELayer(torch.nn.Module):
 
             def expert_fn(expert_input):
                 return self.expert_local(expert_input, original_shape[-reserve_dims:])
-            y = fused_zfp_forward(x, crit, expert_fn)
+            y = fused_zfp_forward(x, crit, expert_fn, degree)
             y = y.view(list(original_shape)).to(original_dtype)
             self.l_aux = y.l_aux = l_aux
             return self.result_func(y) if self.result_func is not None else y

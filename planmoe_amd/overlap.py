@@ -74,8 +74,23 @@ def a2a_ffn_overlap_forward(input, expert_fn, a2a_ffn_overlap_degree, use_2dh, g
     return torch.cat(input_split, dim=split_dim).contiguous()
 
 
+def _experts_in_chunks(expert_fn, buf, degree):
+    """The experts see the [E, C, M] buffer in a2a_ffn_overlap_degree slices along the capacity, as in
+    a2a_ffn_overlap_forward.  The codecs work row by row (int8) or on 4-row blocks that never
+    straddle a slice (zfp, capacity aligned to 4 * degree), so coding the whole buffer at once
+    gives each slice the values it would get on its own."""
+    if degree == 1:
+        return expert_fn(buf)
+    assert degree <= MAX_NUM_SPLIT, \
+        "Excepting a2a_ffn_overlap_degree (%d) <= AllToAllStatus.max_num_split (%d)." % (degree, MAX_NUM_SPLIT)
+    assert buf.shape[1] % degree == 0, \
+        "Excepting input.shape[%d] (%d) be multiple of a2a_ffn_overlap_degree (%d)." % (1, buf.shape[1], degree)
+    return torch.cat([expert_fn(c.contiguous()) for c in buf.split(buf.shape[1] // degree, dim=1)], dim=1)
+
+
 # ------------------------------------------------------------------------------ fused int8 path
-# With the "int8" compressor and one chunk, the steps either side of the all-to-all collapse:
+# With the "int8" compressor the steps either side of the all-to-all collapse (for any
+# a2a_ffn_overlap_degree: only the expert call is sliced, see _experts_in_chunks):
 #   send side     fast_encode + Compress      -> one pass (planmoe_dispatch_int8)
 #   receive side  Decompress + fast_decode    -> one pass (planmoe_combine_int8)
 # and the same two fusions serve the backward pass (Decompress.backward compresses the gradient,
@@ -168,9 +183,9 @@ def fused_gate_eligible(x, gate, experts, compress_name, degree, is_postscore):
             experts <= 64 and x.shape[0] >= 1)
 
 
-def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn):
-    """moe_layer's forward from the gate to the combine for the int8 compressor, one chunk, the
-    GShard loss and plain routing.  Returns (output [T, M], l_aux)."""
+def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn, degree=1):
+    """moe_layer's forward from the gate to the combine for the int8 compressor, the GShard loss
+    and plain routing.  Returns (output [T, M], l_aux)."""
     w = gate.wg.weight
     if w.dtype != x.dtype:
         w = w.to(x.dtype)
@@ -178,7 +193,7 @@ def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn):
     x = x.contiguous()
     y, gates, l_aux, indices, locations = _GateRouteEncodeInt8.apply(x, w.contiguous(), top_k, capacity,
                                                                      bool(gate.fp32_gate), bool(normalize_gate))
-    y = expert_fn(y.view(experts, capacity, x.shape[-1]))
+    y = _experts_in_chunks(expert_fn, y.view(experts, capacity, x.shape[-1]), degree)
     y = y.reshape(experts * capacity, -1).to(x.dtype)
     k = indices.shape[0]
     out = _DecodeInt8.apply(y, indices, locations, experts, capacity, x.shape[0], *[gates[j].float() for j in range(k)])
@@ -239,19 +254,19 @@ FUSE_ZFP = True
 
 def fused_zfp_eligible(x, compress_name, degree, is_postscore, experts, capacity):
     # the conditions under which ZfpCompressor.compress accepts the [E, C, M] buffer (zfpc.cpp:24-31)
-    return (FUSE_ZFP and compress_name == 'zfp' and degree == 1 and is_postscore and x.is_cuda and
+    return (FUSE_ZFP and compress_name == 'zfp' and is_postscore and x.is_cuda and
             x.dtype == torch.float32 and x.shape[-1] % 4 == 0 and experts % 4 == 0 and capacity % 4 == 0 and
             capacity > 0)
 
 
-def fused_zfp_forward(x, crit, expert_fn):
-    """encode -> [codec, comm, codec] -> experts -> [codec, comm, codec] -> decode for one chunk
-    and the zfp compressor.  crit = (experts, indices_s, locations_s, gates_s, capacity)."""
+def fused_zfp_forward(x, crit, expert_fn, degree=1):
+    """encode -> [codec, comm, codec] -> experts -> [codec, comm, codec] -> decode for the
+    zfp compressor.  crit = (experts, indices_s, locations_s, gates_s, capacity)."""
     experts, indices_s, locations_s, gates_s, capacity = crit
     indices = torch.stack([t.reshape(-1) for t in indices_s]).to(torch.int32).contiguous()     # [k, T]
     locations = torch.stack([t.reshape(-1) for t in locations_s]).to(torch.int32).contiguous()
     y = _EncodeZfp.apply(x.contiguous(), indices, locations, experts, capacity)
-    y = expert_fn(y.view(experts, capacity, x.shape[-1]))
+    y = _experts_in_chunks(expert_fn, y.view(experts, capacity, x.shape[-1]), degree)
     y = y.reshape(experts * capacity, -1).to(x.dtype)
     gates = [g.float() for g in gates_s]
     return _DecodeZfp.apply(y, indices, locations, experts, capacity, x.shape[0], *gates)
@@ -259,18 +274,18 @@ def fused_zfp_forward(x, crit, expert_fn):
 
 def fused_int8_eligible(x, compress_name, degree, is_postscore):
     vec = 4 if x.dtype == torch.float32 else 8
-    return (FUSE_INT8 and compress_name == 'int8' and degree == 1 and is_postscore and x.is_cuda and
+    return (FUSE_INT8 and compress_name == 'int8' and is_postscore and x.is_cuda and
             x.dtype in (torch.float32, torch.bfloat16, torch.float16) and x.shape[-1] % vec == 0)
 
 
-def fused_int8_forward(x, crit, expert_fn):
-    """encode -> [codec, comm, codec] -> experts -> [codec, comm, codec] -> decode for one chunk
-    and the int8 compressor.  crit = (experts, indices_s, locations_s, gates_s, capacity)."""
+def fused_int8_forward(x, crit, expert_fn, degree=1):
+    """encode -> [codec, comm, codec] -> experts -> [codec, comm, codec] -> decode for the
+    int8 compressor.  crit = (experts, indices_s, locations_s, gates_s, capacity)."""
     experts, indices_s, locations_s, gates_s, capacity = crit
     indices = torch.stack([t.reshape(-1) for t in indices_s]).to(torch.int32).contiguous()     # [k, T]
     locations = torch.stack([t.reshape(-1) for t in locations_s]).to(torch.int32).contiguous()
     y = _EncodeInt8.apply(x.contiguous(), indices, locations, experts, capacity)
-    y = expert_fn(y.view(experts, capacity, x.shape[-1]))
+    y = _experts_in_chunks(expert_fn, y.view(experts, capacity, x.shape[-1]), degree)
     y = y.reshape(experts * capacity, -1).to(x.dtype)
     gates = [g.float() for g in gates_s]
     return _DecodeInt8.apply(y, indices, locations, experts, capacity, x.shape[0], *gates)

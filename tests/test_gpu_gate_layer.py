@@ -334,6 +334,31 @@ def test_moe_layer_fused_zfp_send_side_equals_the_stepwise_pipeline():
     assert results[0][1].abs().sum() > 0 and results[0][2].abs().sum() > 0
 
 
+@pytest.mark.parametrize("compress,dtype", [("int8", torch.bfloat16), ("int8", torch.float32), ("zfp", torch.float32)])
+def test_fused_paths_with_two_chunks_equal_the_stepwise_pipeline(compress, dtype):
+    """a2a_ffn_overlap_degree = 2: the fused kernels code the whole buffer and only the expert call
+    is sliced; the step-by-step pipeline codes slice by slice.  Same bits, forward and backward."""
+    import planmoe_amd
+    from planmoe_amd import overlap
+    results = []
+    for fuse in (True, False):
+        overlap.FUSE_INT8 = overlap.FUSE_ZFP = fuse
+        overlap.FUSE_GATE = False
+        try:
+            layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 1.25}, 128,
+                                          experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 64},
+                                          seeds=(1, 2, 3), compress_name=compress, a2a_ffn_overlap_degree=2).to(DEV).to(dtype)
+            x = torch.randn(6, 50, 128, generator=torch.Generator().manual_seed(5)).to(dtype).to(DEV).requires_grad_(True)
+            y = layer(x)
+            (y.float().pow(2).mean() + y.l_aux.float()).backward()
+            results.append((y.detach(), x.grad.detach(), layer.gates[0].wg.weight.grad.detach(),
+                            layer.experts.batched_fc1_w.grad.detach()))
+        finally:
+            overlap.FUSE_INT8 = overlap.FUSE_ZFP = overlap.FUSE_GATE = True
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+
+
 def _layer_pass(planmoe_amd, dtype):
     layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 1.25}, 128,
                                   experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 64},
