@@ -19,7 +19,11 @@
 
 namespace pm {
 
-constexpr int TILE = 256;         // tokens per tile = threads per block
+#ifndef PM_ROUTE_TILE
+#define PM_ROUTE_TILE 256
+#endif
+constexpr int TILE = PM_ROUTE_TILE;   // tokens per tile = threads per block
+constexpr int TILE_WAVES = TILE / WAVE;
 constexpr int ROUTE_MAX_E = 2048; // LDS table is 4 waves x experts counters
 
 __device__ __forceinline__ uint64_t lanemask_lt()
@@ -70,7 +74,7 @@ __global__ __launch_bounds__(TILE) void route_tile_kernel(
     float *__restrict__ me_part)
 {
     using E = Elem<DT>;
-    extern __shared__ int32_t wave_cnt[];           // [4][experts]
+    extern __shared__ int32_t wave_cnt[];           // [TILE_WAVES][experts]
     const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
     const int t = blockIdx.x * TILE + tid;
     const bool valid = t < samples;
@@ -83,15 +87,27 @@ __global__ __launch_bounds__(TILE) void route_tile_kernel(
     if constexpr (CAP > 0) {
         // the tile's rows come in with coalesced loads, half a tile at a time, and every thread
         // picks its row out of LDS (row length + 1 keeps the banks apart)
-        float *stage = reinterpret_cast<float *>(wave_cnt + 4 * experts);       // [TILE / 2][experts + 1]
+        float *stage = reinterpret_cast<float *>(wave_cnt + TILE_WAVES * experts);       // [TILE / 2][experts + 1]
         const int64_t tile_base = (int64_t)blockIdx.x * TILE * experts;
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
             const int r0 = half * (TILE / 2);
             const int nrows = max(0, min(TILE / 2, samples - (int)blockIdx.x * TILE - r0));
-            for (int i = tid; i < nrows * experts; i += TILE) {
-                const int r = i / experts, e = i - r * experts;
-                stage[r * (experts + 1) + e] = E::load(input, tile_base + (int64_t)r0 * experts + i);
+            // 8 loads in flight per thread (clamped index: straight-line loads, one wait per batch)
+            const int n = nrows * experts;
+            const int64_t half_base = tile_base + (int64_t)r0 * experts;
+            for (int i0 = tid; i0 < n; i0 += 8 * TILE) {
+                float v[8];
+#pragma unroll
+                for (int q = 0; q < 8; ++q) v[q] = E::load(input, half_base + min(i0 + q * TILE, n - 1));
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const int i = i0 + q * TILE;
+                    if (i < n) {
+                        const int r = i / experts, e = i - r * experts;
+                        stage[r * (experts + 1) + e] = v[q];
+                    }
+                }
             }
             __syncthreads();
             if (valid && tid / (TILE / 2) == half) {
@@ -148,8 +164,11 @@ __global__ __launch_bounds__(TILE) void route_tile_kernel(
         }
         __syncthreads();
         for (int e = tid; e < experts; e += TILE)
-            me_part[(int64_t)blockIdx.x * experts + e] =
-                ((wsum[e] + wsum[experts + e]) + wsum[2 * experts + e]) + wsum[3 * experts + e];
+        {
+            float a = wsum[e];
+            for (int w = 1; w < TILE_WAVES; ++w) a += wsum[w * experts + e];        // fixed order
+            me_part[(int64_t)blockIdx.x * experts + e] = a;
+        }
         __syncthreads();
     }
 
@@ -182,7 +201,7 @@ __global__ __launch_bounds__(TILE) void route_tile_kernel(
         }
 
         // rank of this token among the tile's tokens with the same j-th choice
-        for (int e = tid; e < 4 * experts; e += TILE) wave_cnt[e] = 0;
+        for (int e = tid; e < TILE_WAVES * experts; e += TILE) wave_cnt[e] = 0;
         __syncthreads();
         int rank = 0;
         uint64_t todo = __ballot(valid);
@@ -200,9 +219,11 @@ __global__ __launch_bounds__(TILE) void route_tile_kernel(
             for (int w = 0; w < wave; ++w) before += wave_cnt[w * experts + best];
             locations[(int64_t)j * stride + t] = rank + before;
         }
-        for (int e = tid; e < experts; e += TILE)
-            hist[((int64_t)blockIdx.x * k + j) * experts + e] =
-                wave_cnt[e] + wave_cnt[experts + e] + wave_cnt[2 * experts + e] + wave_cnt[3 * experts + e];
+        for (int e = tid; e < experts; e += TILE) {
+            int32_t n = 0;
+            for (int w = 0; w < TILE_WAVES; ++w) n += wave_cnt[w * experts + e];
+            hist[((int64_t)blockIdx.x * k + j) * experts + e] = n;
+        }
         __syncthreads();
     }
 
@@ -225,7 +246,7 @@ __global__ __launch_bounds__(TILE) void locate_tile_kernel(
     const int32_t *__restrict__ indices, const int32_t *__restrict__ order, int32_t *__restrict__ locations,
     int64_t stride, int samples, int experts, int k, int32_t *__restrict__ hist)
 {
-    extern __shared__ int32_t wave_cnt[];           // [4][experts]
+    extern __shared__ int32_t wave_cnt[];           // [TILE_WAVES][experts]
     const int tid = threadIdx.x, lane = lane_id(), wave = tid >> 6;
     const int p = blockIdx.x * TILE + tid;
     const bool valid = p < samples;
@@ -233,7 +254,7 @@ __global__ __launch_bounds__(TILE) void locate_tile_kernel(
     for (int j = 0; j < k; ++j) {
         int best = valid ? indices[(int64_t)j * stride + t] : -1;
         const bool live = valid && best >= 0 && best < experts;     // anything else takes no slot
-        for (int e = tid; e < 4 * experts; e += TILE) wave_cnt[e] = 0;
+        for (int e = tid; e < TILE_WAVES * experts; e += TILE) wave_cnt[e] = 0;
         __syncthreads();
         int rank = 0;
         uint64_t todo = __ballot(live);
@@ -253,9 +274,11 @@ __global__ __launch_bounds__(TILE) void locate_tile_kernel(
         } else if (valid) {
             locations[(int64_t)j * stride + t] = -1;
         }
-        for (int e = tid; e < experts; e += TILE)
-            hist[((int64_t)blockIdx.x * k + j) * experts + e] =
-                wave_cnt[e] + wave_cnt[experts + e] + wave_cnt[2 * experts + e] + wave_cnt[3 * experts + e];
+        for (int e = tid; e < experts; e += TILE) {
+            int32_t n = 0;
+            for (int w = 0; w < TILE_WAVES; ++w) n += wave_cnt[w * experts + e];
+            hist[((int64_t)blockIdx.x * k + j) * experts + e] = n;
+        }
         __syncthreads();
     }
 }
@@ -496,8 +519,8 @@ extern "C" int planmoe_route_topk(const void *input, int dtype, int input_is_log
     int32_t *offs = hist + (size_t)tiles * k * experts;
     float *me = (float *)(offs + (size_t)tiles * k * experts);
     float *loss_part = me + (size_t)tiles * experts;
-    // 4 waves x experts counters, and for rows held in registers the staging area of half a tile
-    const size_t lds = 4 * (4 * (size_t)experts + (experts <= 64 ? (size_t)(TILE / 2) * (experts + 1) : 0));
+    // TILE_WAVES x experts counters, and for rows held in registers the staging area of half a tile
+    const size_t lds = 4 * (TILE_WAVES * (size_t)experts + (experts <= 64 ? (size_t)(TILE / 2) * (experts + 1) : 0));
 
     PM_DTYPE_SWITCH(dtype, DT,
         launch_route_tile<DT>(experts, dim3(tiles), lds, st, input, input_is_logits, logit_bias,
@@ -533,7 +556,7 @@ extern "C" int planmoe_route_locations(const int32_t *indices, int64_t plane_str
     const int tiles = (int)route_tiles(samples);
     int32_t *hist = (int32_t *)workspace;
     int32_t *offs = hist + (size_t)tiles * k * experts;
-    locate_tile_kernel<<<tiles, TILE, sizeof(int32_t) * 4 * (size_t)experts, st>>>(
+    locate_tile_kernel<<<tiles, TILE, sizeof(int32_t) * TILE_WAVES * (size_t)experts, st>>>(
         indices, order, locations, plane_stride, samples, experts, k, hist);
     const int epb = go_experts_per_block(experts, k);
     group_offsets_kernel<<<(experts + epb - 1) / epb, 256, 0, st>>>(hist, offs, nullptr, tiles, k, experts, epb,
