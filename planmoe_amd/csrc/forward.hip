@@ -100,7 +100,10 @@ __device__ __forceinline__ uint64_t lanes_below() { return ((uint64_t)1 << lane_
 // CAP: compile-time bound of the expert count held in registers by the routing epilogue
 // NT == 1: split-K over the 4 waves, weights straight from L2 (up to 16 experts);
 // NT > 1: weights shared through LDS, a wave per 16 tokens.
-template <int DT, int SDT, int NT, int CAP, bool SPLITK, int GROUP>
+// MODE 0: logits = x . wg^T computed here.  MODE 1 / 2: no GEMM; x holds the [samples, experts]
+// logits / scores in the routing dtype (the stand-alone routing entry point) and only the
+// epilogue runs, on 64-token groups.
+template <int DT, int SDT, int NT, int CAP, bool SPLITK, int GROUP, int MODE = 0>
 __global__ __launch_bounds__(256) void gate_route_kernel(
     const void *__restrict__ x, const void *__restrict__ wg, const float *__restrict__ logit_bias,
     int samples, int model_dim, int experts, int k, int normalize_gate,
@@ -120,10 +123,32 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
     const int groups = gridDim.x;
     const FwdWs ws = fwd_ws(workspace, groups, k, experts, samples);
     const int t0 = blockIdx.x * GROUP;
-    constexpr bool STATS = DT == PLANMOE_BF16;
+    constexpr bool STATS = DT == PLANMOE_BF16 && MODE == 0;
+    static_assert(MODE == 0 || (!SPLITK && GROUP == 64), "routing from memory runs on 64-token groups");
     __shared__ int32_t pstat[SPLITK ? 4 : 1][GROUP][3];
-    if constexpr (SPLITK) gate_tile_partials<DT, NT, GROUP / 16, 4, STATS>(x, wg, t0, samples, model_dim, experts, part, pstat);
-    else gate_tile_lds<DT, NT, STATS>(x, wg, t0, samples, model_dim, experts, smem, pstat[0]);
+    if constexpr (MODE != 0) {
+        // the group's rows land where the GEMM would have left its logits: 8 loads in flight per
+        // thread, at clamped indices so that they are straight-line loads
+        const int n = min(GROUP, samples - t0) * experts;
+        const int64_t base = (int64_t)t0 * experts;
+        for (int i0 = tid; i0 < n; i0 += 8 * 256) {
+            float v[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) v[q] = S::load(x, base + min(i0 + q * 256, n - 1));
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const int i = i0 + q * 256;
+                if (i < n) {
+                    const int tok = i / experts;
+                    part[0][tok][i - tok * experts] = v[q];
+                }
+            }
+        }
+    } else if constexpr (SPLITK) {
+        gate_tile_partials<DT, NT, GROUP / 16, 4, STATS>(x, wg, t0, samples, model_dim, experts, part, pstat);
+    } else {
+        gate_tile_lds<DT, NT, STATS>(x, wg, t0, samples, model_dim, experts, smem, pstat[0]);
+    }
     __syncthreads();
 
     // ---- routing epilogue, part 1: all four waves, wave w owns GROUP / 4 consecutive tokens.
@@ -157,29 +182,33 @@ __global__ __launch_bounds__(256) void gate_route_kernel(
                 if constexpr (SPLITK) v = ((part[0][tok][e] + part[1][tok][e]) + part[2][tok][e]) + part[3][tok][e];
                 else v = part[0][tok][e];
                 v = S::round(v);
-                if (logits_out && valid) S::store(logits_out, (int64_t)t * experts + e, v);
-                if (logit_bias) v = S::round(v + logit_bias[e]);
+                if constexpr (MODE != 2) {
+                    if (logits_out && valid) S::store(logits_out, (int64_t)t * experts + e, v);
+                    if (logit_bias) v = S::round(v + logit_bias[e]);
+                }
             }
-            sc[q] = v;
+            sc[q] = v;                                    // MODE 2: the score itself (-inf past the experts)
             mx = fmaxf(mx, v);
         }
-        mx = token_reduce(mx, [](float a, float b) { return fmaxf(a, b); });
-        float sum = 0.f;
+        if constexpr (MODE != 2) {
+            mx = token_reduce(mx, [](float a, float b) { return fmaxf(a, b); });
+            float sum = 0.f;
 #pragma unroll
-        for (int q = 0; q < EPL; ++q) {
-            sc[q] = (q * LPT + el < experts) ? expf(sc[q] - mx) : 0.f;
-            sum += sc[q];
-        }
-        sum = token_reduce(sum, [](float a, float b) { return a + b; });
-        const float inv = 1.0f / sum;                     // scores are tolerance-level quantities
+            for (int q = 0; q < EPL; ++q) {
+                sc[q] = (q * LPT + el < experts) ? expf(sc[q] - mx) : 0.f;
+                sum += sc[q];
+            }
+            sum = token_reduce(sum, [](float a, float b) { return a + b; });
+            const float inv = 1.0f / sum;                 // scores are tolerance-level quantities
 #pragma unroll
-        for (int q = 0; q < EPL; ++q) {
-            const int e = q * LPT + el;
-            if (e < experts) {
-                sc[q] = S::round(sc[q] * inv);
-                if (scores_out && valid) S::store(scores_out, (int64_t)t * experts + e, sc[q]);
-            } else {
-                sc[q] = -INFINITY;
+            for (int q = 0; q < EPL; ++q) {
+                const int e = q * LPT + el;
+                if (e < experts) {
+                    sc[q] = S::round(sc[q] * inv);
+                    if (scores_out && valid) S::store(scores_out, (int64_t)t * experts + e, sc[q]);
+                } else {
+                    sc[q] = -INFINITY;
+                }
             }
         }
         // column sums of the wave's scores (GShard loss): over the tokens of the pass, then passes
@@ -325,6 +354,113 @@ __global__ __launch_bounds__(256) void route_offsets_kernel(const int32_t *__res
     locations[o] = rank[i] + hist[((int64_t)(t / group_tokens) * k + j) * experts + indices[o]];
 }
 
+// ---- the prefix over the routing groups without a launch of its own (top_k <= 4): every wave
+// sums the columns of the transposed histogram it needs.
+
+// Lane j (< top_k) returns the slot of choice j of token t inside its expert: rank in the group +
+// entries of the earlier planes + entries of the earlier groups of plane j.  e_l: its expert.
+__device__ __forceinline__ int merged_location(const int32_t *__restrict__ indices, const int32_t *__restrict__ rank,
+                                               const int32_t *__restrict__ hist_t, int64_t stride, int top_k,
+                                               int samples, int experts, int t, int group_tokens, int groups,
+                                               int gstride, int &e_l)
+{
+    const int lane = lane_id();
+    int l = 0;
+    e_l = 0;
+    if (lane < top_k) {
+        e_l = indices[(int64_t)lane * stride + t];
+        l = rank[(int64_t)lane * samples + t];
+    }
+    const int g = t / group_tokens;
+    // slots of expert e taken before this group's plane-j tokens: every entry of the planes
+    // before j, and the groups before g in plane j
+    int before[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (j < top_k) {
+            const int e = rl_i(e_l, j);
+            before[j] = column_partial(hist_t + ((int64_t)j * experts + e) * gstride, g);
+            for (int jp = 0; jp < j; ++jp) before[j] += column_partial(hist_t + ((int64_t)jp * experts + e) * gstride, groups);
+        }
+    }
+    wave_sum_n(before);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) if (lane == j) l += before[j];
+    return l;
+}
+
+// One work-group (4 waves) finishes the GShard loss and the per-plane expert counts.
+// s_loss: 64 floats of LDS.
+__device__ __forceinline__ void merged_stats(const int32_t *__restrict__ hist_t, const float *__restrict__ me_t,
+                                             int groups, int gstride, int experts, int top_k, int samples,
+                                             int32_t *__restrict__ counts_out, float *__restrict__ l_aux,
+                                             float *s_loss)
+{
+    const int wave = threadIdx.x >> 6, lane = lane_id();
+    // the one block that finishes the loss: l_aux = sum_e me[e] * ce[e] / T with
+    // me[e] = column sum of the scores, ce[e] = first-choice count * E / T
+    // four experts per pass and wave: the loads of a pass are in flight together
+    for (int e0 = wave * 4; e0 < experts; e0 += 16) {
+        int c0[4] = {0, 0, 0, 0};
+        float m[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (e0 + q < experts) {
+                c0[q] = column_partial(hist_t + (int64_t)(e0 + q) * gstride, groups);
+                if (l_aux) m[q] = column_partial(me_t + (int64_t)(e0 + q) * gstride, groups);
+            }
+        }
+        wave_sum_n(c0);
+        wave_sum_n(m);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (lane == 0 && e0 + q < experts) {
+                if (counts_out) counts_out[e0 + q] = c0[q];
+                s_loss[e0 + q] = m[q] * ((float)c0[q] * ((float)experts / (float)samples));
+            }
+        }
+        if (counts_out) {
+            for (int j = 1; j < top_k; ++j) {
+                int c[4] = {0, 0, 0, 0};
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (e0 + q < experts) c[q] = column_partial(hist_t + ((int64_t)j * experts + e0 + q) * gstride, groups);
+                wave_sum_n(c);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) if (lane == 0 && e0 + q < experts) counts_out[j * experts + e0 + q] = c[q];
+            }
+        }
+    }
+    __syncthreads();
+    if (l_aux && threadIdx.x == 0) {
+        float a = 0.f;
+        for (int e = 0; e < experts; ++e) a += s_loss[e];
+        *l_aux = a / (float)samples;
+    }
+}
+
+// locations of a stand-alone routing call (top_k <= 4): block 0 finishes the loss and the counts,
+// the others take a token per wave
+__global__ __launch_bounds__(256) void route_locations_merged_kernel(
+    const int32_t *__restrict__ indices, int32_t *__restrict__ locations, int64_t stride, int top_k, int samples,
+    int experts, const int32_t *__restrict__ rank, int group_tokens, const int32_t *__restrict__ hist_t,
+    const float *__restrict__ me_t, int groups, int gstride, int32_t *__restrict__ counts_out,
+    float *__restrict__ l_aux)
+{
+    __shared__ float s_loss[64];
+    if (blockIdx.x == 0) {
+        if (l_aux || counts_out)
+            merged_stats(hist_t, me_t, groups, gstride, experts, top_k, samples, counts_out, l_aux, s_loss);
+        return;
+    }
+    const int t = ((int)blockIdx.x - 1) * 4 + (int)(threadIdx.x >> 6);
+    if (t >= samples) return;
+    int e_l;
+    const int l = merged_location(indices, rank, hist_t, stride, top_k, samples, experts, t, group_tokens, groups,
+                                  gstride, e_l);
+    if (lane_id() < top_k) locations[(int64_t)lane_id() * stride + t] = l;
+}
+
 // Dispatch + int8 with the slot offsets still to be added (see dispatch_int8_kernel for the
 // stand-alone variant).  Only the all-ones gate helper (is_postscore) is fused here.
 //
@@ -360,46 +496,7 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     if (fill_first && bid >= 0) bid = bid < fill_blocks ? token_blocks + bid : bid - fill_blocks;
     if constexpr (MERGED) {
         if ((int)blockIdx.x < stat_blocks) {
-            // the one block that finishes the loss: l_aux = sum_e me[e] * ce[e] / T with
-            // me[e] = column sum of the scores, ce[e] = first-choice count * E / T
-            // four experts per pass and wave: the loads of a pass are in flight together
-            for (int e0 = wave * 4; e0 < experts; e0 += 16) {
-                int c0[4] = {0, 0, 0, 0};
-                float m[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    if (e0 + q < experts) {
-                        c0[q] = column_partial(hist_t + (int64_t)(e0 + q) * gstride, groups);
-                        if (l_aux) m[q] = column_partial(me_t + (int64_t)(e0 + q) * gstride, groups);
-                    }
-                }
-                wave_sum_n(c0);
-                wave_sum_n(m);
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    if (lane == 0 && e0 + q < experts) {
-                        if (counts_out) counts_out[e0 + q] = c0[q];
-                        s_loss[e0 + q] = m[q] * ((float)c0[q] * ((float)experts / (float)samples));
-                    }
-                }
-                if (counts_out) {
-                    for (int j = 1; j < top_k; ++j) {
-                        int c[4] = {0, 0, 0, 0};
-#pragma unroll
-                        for (int q = 0; q < 4; ++q)
-                            if (e0 + q < experts) c[q] = column_partial(hist_t + ((int64_t)j * experts + e0 + q) * gstride, groups);
-                        wave_sum_n(c);
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) if (lane == 0 && e0 + q < experts) counts_out[j * experts + e0 + q] = c[q];
-                    }
-                }
-            }
-            __syncthreads();
-            if (l_aux && threadIdx.x == 0) {
-                float a = 0.f;
-                for (int e = 0; e < experts; ++e) a += s_loss[e];
-                *l_aux = a / (float)samples;
-            }
+            merged_stats(hist_t, me_t, groups, gstride, experts, top_k, samples, counts_out, l_aux, s_loss);
             return;
         }
     }
@@ -455,26 +552,9 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     // lane j finalises choice j: slot = expert * capacity + rank in group + group offset
     int slot = -1;
     if constexpr (MERGED) {
-        int e_l = 0, l = 0;
-        if (lane < top_k) {
-            e_l = indices[(int64_t)lane * stride + t];
-            l = rank[(int64_t)lane * samples + t];
-        }
-        const int g = t / group_tokens;
-        // slots of expert e taken before this group's plane-j tokens: every entry of the planes
-        // before j, and the groups before g in plane j
-        int before[4] = {0, 0, 0, 0};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (j < top_k) {
-                const int e = rl_i(e_l, j);
-                before[j] = column_partial(hist_t + ((int64_t)j * experts + e) * gstride, g);
-                for (int jp = 0; jp < j; ++jp) before[j] += column_partial(hist_t + ((int64_t)jp * experts + e) * gstride, groups);
-            }
-        }
-        wave_sum_n(before);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) if (lane == j) l += before[j];
+        int e_l;
+        const int l = merged_location(indices, rank, hist_t, stride, top_k, samples, experts, t, group_tokens, groups,
+                                      gstride, e_l);
         if (lane < top_k) {
             locations[(int64_t)lane * stride + t] = l;
             if (l < capacity) slot = e_l * capacity + l;
@@ -606,6 +686,68 @@ static void fwd_plan(FwdPlan &plan, void *workspace, int samples, int experts, i
     plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts, samples);
 }
 
+// ranks in groups -> final slots (and the loss and the expert counts): one launch in which every
+// wave sums the histogram columns it needs (top_k <= 4 and a small histogram), else the prefix
+// over the groups and a launch that adds it
+static void finish_routing(const FwdPlan &plan, const int32_t *indices, int32_t *locations, int64_t stride,
+                           int samples, int experts, float *l_aux, int32_t *counts, hipStream_t st)
+{
+    // measured: 38.4 vs 39.7 us (256 groups x 8 experts), 58.6 vs 45.2 us (512 groups x 64 experts, where
+    // nothing hides the one block that sums every column for the loss)
+    if (plan.k <= 4 && (int64_t)plan.groups * experts <= 8192) {
+        route_locations_merged_kernel<<<1 + (samples + 3) / 4, 256, 0, st>>>(
+            indices, locations, stride, plan.k, samples, experts, plan.ws.rank, plan.group_tokens, plan.ws.hist_t,
+            plan.ws.me_t, plan.groups, plan.ws.gstride, counts, l_aux);
+        return;
+    }
+    group_offsets_kernel<<<plan.blocks, 256, 0, st>>>(plan.ws.hist, plan.ws.offs, plan.ws.me, plan.groups, plan.k, experts,
+                                                      plan.experts_per_block, samples, plan.ws.totals, counts,
+                                                      plan.ws.loss_part, l_aux != nullptr);
+    route_offsets_kernel<<<(samples * plan.k + 255) / 256, 256, 0, st>>>(indices, locations, stride, samples, experts,
+                                                                        plan.k, plan.ws.offs, plan.ws.rank,
+                                                                        plan.group_tokens, plan.ws.loss_part, plan.blocks,
+                                                                        l_aux);
+}
+
+// stand-alone routing from logits / scores in memory: the epilogue of gate_route_kernel on 64-token
+// groups, then the prefix over the groups and the final slots
+template <int SDT>
+static void launch_route_groups(int experts, int groups, int mode, hipStream_t st, const void *input, const float *bias,
+                                int samples, int k, int normalize, int32_t *indices, int32_t *locations, void *gates,
+                                int64_t stride, void *scores_out, float *l_aux, int32_t *counts, void *ws)
+{
+#define PM_RG_(NT, CAP, MODE)                                                                              \
+    gate_route_kernel<SDT, SDT, NT, CAP, false, 64, MODE><<<groups, 256, 0, st>>>(input, nullptr, bias, samples, 0, \
+        experts, k, normalize, indices, locations, gates, stride, nullptr, scores_out, l_aux, counts, ws)
+#define PM_RG(NT, CAP) do { if (mode == 1) PM_RG_(NT, CAP, 1); else PM_RG_(NT, CAP, 2); } while (0)
+    if (experts <= 8) PM_RG(1, 8);
+    else if (experts <= 16) PM_RG(1, 16);
+    else if (experts <= 32) PM_RG(2, 32);
+    else PM_RG(4, 64);
+#undef PM_RG
+#undef PM_RG_
+}
+
+int route_groups(const void *input, int dtype, int is_logits, const float *logit_bias, int samples, int experts,
+                 int top_k, int normalize_gate, int32_t *indices, int32_t *locations, void *gates, int64_t stride,
+                 void *scores_out, float *l_aux, int32_t *counts, void *workspace, hipStream_t st)
+{
+    FwdPlan plan;
+    plan.k = top_k < experts ? top_k : experts;
+    plan.group_tokens = 64;
+    plan.groups = (samples + 63) / 64;
+    plan.experts_per_block = go_experts_per_block(experts, plan.k);
+    plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
+    plan.merged = false;
+    plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts, samples);
+    const int mode = is_logits ? 1 : 2;
+    PM_DTYPE_SWITCH(dtype, SDT, (launch_route_groups<SDT>(experts, plan.groups, mode, st, input, is_logits ? logit_bias : nullptr,
+                                                         samples, plan.k, normalize_gate, indices, locations, gates, stride,
+                                                         is_logits ? scores_out : nullptr, l_aux, counts, workspace)));
+    finish_routing(plan, indices, locations, stride, samples, experts, l_aux, counts, st);
+    return 0;
+}
+
 // launches gate_route_kernel and, unless the dispatch launch will do that part, group_offsets_kernel
 static int run_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
                           const float *logit_bias, int samples, int model_dim, int experts, int top_k,
@@ -694,10 +836,8 @@ extern "C" int planmoe_gate_route(const void *x, const void *wg, int dtype, int 
     FwdPlan plan;
     if (run_gate_route(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
                        normalize_gate, indices, locations, gates, plane_stride, logits_out, scores_out,
-                       l_aux, expert_counts, workspace, st, plan, true)) return 1;
-    route_offsets_kernel<<<(samples * plan.k + 255) / 256, 256, 0, st>>>(
-        indices, locations, plane_stride, samples, experts, plan.k, plan.ws.offs, plan.ws.rank,
-        plan.group_tokens, plan.ws.loss_part, plan.blocks, l_aux);
+                       l_aux, expert_counts, workspace, st, plan, false)) return 1;
+    finish_routing(plan, indices, locations, plane_stride, samples, experts, l_aux, expert_counts, st);
     PM_LAUNCH_CHECK("planmoe_gate_route");
     return 0;
 }

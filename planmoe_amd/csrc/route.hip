@@ -2,8 +2,9 @@
 //
 // planmoe_route_topk takes the place of extract_critical (impls/fast_dispatch.py:140-195):
 // about 25 ATen launches over [samples, experts] one-hot matrices plus the E-block
-// Blelloch scan of custom_kernel.cpp:339-376 become three launches that never build a
-// one-hot matrix:
+// Blelloch scan of custom_kernel.cpp:339-376 become two or three launches that never build a
+// one-hot matrix.  Up to 64 experts the work is done by the routing epilogue of the forward
+// chain's first kernel (forward.hip, route_groups); above that by the kernels of this file:
 //   route_tile_kernel   one thread per token, 256 tokens per tile: softmax (optional),
 //                       k-fold arg-max, rank of the token among the tile's tokens that
 //                       chose the same expert (wave ballots + an LDS table), per-tile
@@ -14,8 +15,11 @@
 //
 // Workspace layout (32-bit words): hist[tiles][k][E], offs[tiles][k][E], me[tiles][E] (fp32),
 // loss_part[E] (fp32).
+#include <algorithm>
+
 #include "common.hpp"
 #include "offsets.hpp"
+#include "rows.hpp"
 
 namespace pm {
 
@@ -469,8 +473,10 @@ extern "C" size_t planmoe_route_workspace_bytes(int samples, int experts, int to
     if (samples <= 0 || experts <= 0 || top_k <= 0) return 16;
     const size_t k = (size_t)(top_k < experts ? top_k : experts);
     const size_t tiles = route_tiles(samples);
-    // hist[tiles][k][E] + offs[tiles][k][E] + me[tiles][E] + loss_part[E]
-    return round_up((2 * tiles * k * experts + tiles * experts + (size_t)experts) * 4, 256);
+    // hist[tiles][k][E] + offs[tiles][k][E] + me[tiles][E] + loss_part[E]; up to 64 experts the
+    // routing runs on the forward chain's groups and takes that chain's workspace
+    const size_t own = round_up((2 * tiles * k * experts + tiles * experts + (size_t)experts) * 4, 256);
+    return experts <= 64 ? std::max(own, planmoe_forward_workspace_bytes(samples, experts, top_k)) : own;
 }
 
 template <int DT>
@@ -514,6 +520,14 @@ extern "C" int planmoe_route_topk(const void *input, int dtype, int input_is_log
     PM_REQUIRE(workspace && workspace_bytes >= planmoe_route_workspace_bytes(samples, experts, top_k),
                "planmoe_route_topk: workspace too small (%zu < %zu)", workspace_bytes,
                planmoe_route_workspace_bytes(samples, experts, top_k));
+    if (experts <= 64) {
+        // lanes share a token and the experts of a row (softmax and arg-max as butterflies), 64-token
+        // groups: several times the parallelism of the thread-per-token tiles below
+        if (route_groups(input, dtype, input_is_logits, logit_bias, samples, experts, top_k, normalize_gate, indices,
+                         locations, gates, plane_stride, scores_out, l_aux, expert_counts, workspace, st)) return 1;
+        PM_LAUNCH_CHECK("planmoe_route_topk");
+        return 0;
+    }
     const int tiles = (int)route_tiles(samples);
     int32_t *hist = (int32_t *)workspace;
     int32_t *offs = hist + (size_t)tiles * k * experts;

@@ -58,5 +58,10 @@ void launch_slot_flags(uint32_t *flags, const int32_t *indices, const int32_t *l
                        hipStream_t st);
 int check_planes(const char *who, const int32_t *indices, const int32_t *locations,
                  int64_t stride, int top_k, int samples);
+// routing of up to 64 experts from [samples, experts] logits / scores with the forward chain's
+// epilogue; workspace of planmoe_forward_workspace_bytes(samples, experts, top_k)
+int route_groups(const void *input, int dtype, int is_logits, const float *logit_bias, int samples, int experts,
+                 int top_k, int normalize_gate, int32_t *indices, int32_t *locations, void *gates, int64_t stride,
+                 void *scores_out, float *l_aux, int32_t *counts, void *workspace, hipStream_t st);
 
 } // namespace pm
