@@ -255,7 +255,7 @@ def main():
     # dominant kernel alone (dispatch + int8 on the routing the chain produced)
     chain()
     stages = {}
-    stages["gate_route entry point (gate GEMM + routing; stand-alone it adds two small launches)"] = event_time_us(
+    stages["gate_route entry point (gate GEMM + routing; stand-alone it adds a small launch that finishes the slots)"] = event_time_us(
         lambda: ops.gate_route(xd, wd, k, fp32_gate=True), 30, 5)
     stages["dispatch_int8_routed"] = event_time_us(plan.redispatch, 30, 5)
     chain_ev = event_time_us(chain, 30, 5)
