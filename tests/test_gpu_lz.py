@@ -112,6 +112,27 @@ def test_config5_full_size():
     assert int(got[1][-1]) < 0.8 * x.nbytes
 
 
+def test_largest_input():
+    """2^31 - 4096 bytes, the most the int32 offset tables can describe: nothing shrinks, so the last
+    offsets sit right under 2^31.  Checked through what holds at any size: the tables are the
+    prefix sums of a stored stream, the token bytes are the input, the decode gives it back."""
+    nbytes = (1 << 31) - 4096
+    x = torch.empty((nbytes // 4,), dtype=torch.float32, device=DEV)
+    x.view(torch.int32).copy_(torch.arange(nbytes // 4, dtype=torch.int32, device=DEV))      # all symbols differ
+    x.view(torch.int32).bitwise_and_(0x3fffffff)                                             # ... and none is a NaN
+    fo, do, flags, data = ops.lz_compress(x)
+    blocks = nbytes // 2048
+    assert fo.numel() == blocks + 1 and int(fo[-1]) == blocks * 64 and int(do[-1]) == nbytes
+    assert torch.equal(do, torch.arange(blocks + 1, dtype=torch.int64, device=DEV).mul_(2048).to(torch.int32))
+    assert not flags.any()
+    assert torch.equal(data.view(torch.int32), x.view(torch.int32))
+    out = torch.empty_like(x)
+    ops.lz_decompress(out, fo, do, flags, data)
+    assert torch.equal(out.view(torch.int32), x.view(torch.int32))
+    with pytest.raises(_lib.PlanMoEError, match="too large"):
+        ops.lz_compress(torch.empty(((1 << 31) // 4,), dtype=torch.float32, device=DEV))
+
+
 @pytest.mark.parametrize("nsym", [1, 8, 511, 513, 512 * 3 + 100, 512 * 17 - 1])
 def test_ragged_tail(nsym):
     rng = np.random.default_rng(nsym)
