@@ -56,8 +56,23 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert rc != 0 and b"dtype" in lib.planmoe_last_error()
     rc = lib.planmoe_route_topk(None, 0, 0, None, 4, 4096, 1, 1, None, None, None, 4, None, None, None, None, 0, None)
     assert rc != 0 and b"experts" in lib.planmoe_last_error()
+    # sizes that would overflow the 32-bit slot / offset arithmetic are refused, not wrapped
+    p16 = ctypes.c_void_p(16)
+    rc = lib.planmoe_dispatch_fwd(p16, 0, None, p16, p16, 8, 1, 8, 64, 70000, 70000, p16, p16, 1 << 40, None)
+    assert rc != 0 and b"overflows int32" in lib.planmoe_last_error()
+    rc = lib.planmoe_lz_compress(p16, 1 << 31, p16, p16, p16, p16, p16, 1 << 40, None)
+    assert rc != 0 and b"too large" in lib.planmoe_last_error()
+    rc = lib.planmoe_lz_compress(p16, 6, p16, p16, p16, p16, p16, 1 << 40, None)
+    assert rc != 0 and b"multiple of 4" in lib.planmoe_last_error()
+    rc = lib.planmoe_dispatch_zfp(p16, None, p16, p16, 8, 1, 8, 64, 3, 2, 8.0, p16, 1 << 40, p16, 1 << 40, None)
+    assert rc != 0 and b"zfp fails." in lib.planmoe_last_error()          # 6 slot rows
+    rc = lib.planmoe_forward_int8(p16, p16, 1, 1, None, 64, 512, 65, 2, 1, 16, p16, p16, p16, 64, None, None, None,
+                                  None, p16, p16, p16, p16, 1 << 40, None)
+    assert rc != 0 and b"64 experts" in lib.planmoe_last_error()
     # empty inputs are a successful no-op
     assert lib.planmoe_int8_compress(None, 0, 0, 8, None, None, None, None) == 0
+    assert lib.planmoe_lz_blocks(0) == 0 and lib.planmoe_lz_blocks(2049) == 2
+    assert lib.planmoe_lz_decompress(None, 0, None, None, None, None, None) == 0
     assert lib.planmoe_combine_fwd(None, 0, None, ctypes.c_void_p(16), ctypes.c_void_p(16), 0, 1, 0, 8, 4, None, None) == 0
 
 
