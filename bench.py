@@ -186,6 +186,44 @@ def kernel_table(only=None):
         print("%-30s %-4s %10.1f %9.1f %9.1f %8.0f %6.2f" % (name, cfg, nbytes / 1e6, avg, best, gbs, gbs / HBM_PEAK_GBS))
 
 
+def layer_table():
+    """moe_layer forward + backward with identity experts (the data path alone: gate, routing,
+    encode, codec, comm copy, codec, decode and their backward passes) for every compressor,
+    with the fused entry points and with the step-by-step pipeline of the reference's structure."""
+    import torch
+    import planmoe_amd
+    from planmoe_amd import overlap
+    dev = "cuda:0"
+
+    class Identity(torch.nn.Module):
+        def update(self, ctx):
+            self.dummy = torch.nn.Parameter(torch.zeros(1))
+
+        def forward(self, x, ctx):
+            return x
+
+    cases = [("2", 16384, 4096, 8, 2, 1.25, torch.bfloat16, "no"), ("2", 16384, 4096, 8, 2, 1.25, torch.bfloat16, "int8"),
+             ("5", 65536, 1024, 16, 2, 1.0, torch.float32, "no"), ("5", 65536, 1024, 16, 2, 1.0, torch.float32, "zfp"),
+             ("5", 65536, 1024, 16, 2, 1.0, torch.float32, "lz")]
+    print("%-4s %-6s %-9s %14s %14s" % ("cfg", "codec", "dtype", "fused ms", "stepwise ms"))
+    for cfg, T, M, E, k, cf, dtype, codec in cases:
+        times = []
+        for fused in (True, False):
+            overlap.FUSE_INT8 = overlap.FUSE_GATE = overlap.FUSE_ZFP = fused
+            layer = planmoe_amd.moe_layer({'type': 'top', 'k': k, 'capacity_factor': cf, 'fp32_gate': True}, M,
+                                          experts={'type': 'custom', 'module': Identity(), 'count_per_node': E},
+                                          seeds=(1, 2, 3), compress_name=codec).to(dev).to(dtype)
+            x = torch.randn(T, M, generator=torch.Generator().manual_seed(0)).to(dtype).to(dev).requires_grad_(True)
+
+            def step():
+                y = layer(x)
+                (y.float().mean() + y.l_aux.float()).backward()
+                x.grad = None
+            times.append(event_time_us(step, 5, 3, rounds=3)[0] / 1e3)
+        overlap.FUSE_INT8 = overlap.FUSE_GATE = overlap.FUSE_ZFP = True
+        print("%-4s %-6s %-9s %14.3f %14.3f" % (cfg, codec, str(dtype).replace("torch.", ""), times[0], times[1]))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -199,15 +237,21 @@ def main():
     ap.add_argument("--kernels", action="store_true",
                     help="instead of the JSON line, print a table of every entry point at full size "
                          "(device time, algorithmic bytes, fraction of the HBM peak)")
+    ap.add_argument("--layer", action="store_true",
+                    help="instead of the JSON line, time moe_layer forward + backward with identity experts for "
+                         "every compressor, with and without the fused entry points")
     ap.add_argument("--only", default=None, help="with --kernels: only the lines whose 'name [config]' contains this, e.g. lz_ or [5]")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
                  "(nothing here uses a second GPU)" % args.gpus)
-    if args.kernels:
+    if args.kernels or args.layer:
         import __graft_entry__
         __graft_entry__.ensure_built()
-        kernel_table(args.only)
+        if args.kernels:
+            kernel_table(args.only)
+        else:
+            layer_table()
         return
 
     import __graft_entry__
