@@ -112,9 +112,12 @@ def kernel_table(only=None):
     add("dispatch_int8 (fused)", "2", xb + R * M + R * 4 + plane, lambda: ops.dispatch_int8(x, idx, loc, None, E, C))
     add("combine_bwd_int8 (fused)", "4", xb + live * M * 2 + R * M + R * 4 + plane + T * k * 4,
         lambda: ops.combine_bwd_int8(x, d, idx, loc, gates, E, C))
+    dc = ops.int8_compress(d)
+    add("combine_bwd_int8 (coded in)", "4", xb + live * M + R * M + 2 * R * 4 + plane + T * k * 4,
+        lambda: ops.combine_bwd_int8(x, dc, idx, loc, gates, E, C))
     plan = ops.ForwardInt8Plan(x, wg, k, C, fp32_gate=True)
     add("forward_int8 (chain)", "2", xb + E * M * 2 + R * M + R * 4 + plane, plan.run)
-    del d, codes, plan
+    del d, dc, codes, plan
 
     # config 1: 8192 x 2048 fp32, 2 experts, top-2
     T1, M1, E1 = 8192, 2048, 2

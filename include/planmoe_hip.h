@@ -196,6 +196,18 @@ int planmoe_combine_bwd_int8(const void *grad_out, const void *expert_out, int d
                              int64_t plane_stride, int top_k, int samples, int model_dim,
                              int experts, int capacity, uint8_t *codes, void *bias, void *scale,
                              float *grad_gates, void *workspace, size_t workspace_bytes, void *stream);
+/* The same with the expert output given as the int8 codes the receive side holds anyway
+ * (expert_codes [experts * capacity, model_dim], expert_bias / expert_scale per row, as
+ * planmoe_int8_compress wrote them): the rows are decoded on the fly to the values
+ * planmoe_int8_decompress would give, so grad_gates and the outputs are bit-identical, and the
+ * decompressed copy of the expert output need not exist in the backward pass. */
+int planmoe_combine_bwd_int8_coded(const void *grad_out, const uint8_t *expert_codes,
+                                   const void *expert_bias, const void *expert_scale, int dtype,
+                                   const float *gates, const int32_t *indices,
+                                   const int32_t *locations, int64_t plane_stride, int top_k,
+                                   int samples, int model_dim, int experts, int capacity,
+                                   uint8_t *codes, void *bias, void *scale, float *grad_gates,
+                                   void *workspace, size_t workspace_bytes, void *stream);
 
 /* Decompress and combine in one pass (Decompress.apply with "int8" followed by fast_decode:
  * impls/overlap.py:22-29, int8.cpp:46-60, fast_dispatch.py:203-207): what planmoe_combine_fwd

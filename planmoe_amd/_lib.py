@@ -50,6 +50,9 @@ SIGNATURES = {
     "planmoe_combine_bwd_int8": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_int,
                                          c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                          c_void_p, c_size_t, c_void_p]),
+    "planmoe_combine_bwd_int8_coded": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                               c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p,
+                                               c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "planmoe_combine_int8": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int64,
                                      c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "planmoe_forward_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),

@@ -5,6 +5,8 @@
 // reduced to min/max across lanes, quantised, and the codes are written to every live slot
 // of the token.  With the all-ones gate helper every choice shares one set of codes.
 #include "rows.hpp"
+#include <type_traits>
+
 #include "int8_core.hpp"
 
 namespace pm {
@@ -12,14 +14,17 @@ namespace pm {
 // CACHE = 16-byte vectors per lane held in registers (0: re-read the row from cache)
 // GATED: rows are scaled by their gate first (one code row per choice); GRAD: the gate gradient
 // <x[t], other[slot]> rides along (GATED only)
-template <int DT, int CACHE, bool GATED, bool GRAD>
+// CODED: `other` is given as int8 codes + per-row bias / scale (what the decompressor would have
+// turned into the rows of `other`); the rows are decoded on the fly, same values, half the bytes
+template <int DT, int CACHE, bool GATED, bool GRAD, bool CODED = false>
 __global__ __launch_bounds__(256) void dispatch_int8_kernel(
     const void *__restrict__ x, const float *__restrict__ gates,
     const int32_t *__restrict__ indices, const int32_t *__restrict__ locations, int64_t stride,
     int top_k, int samples, int model_dim, int experts, int capacity,
     uint8_t *__restrict__ codes, void *__restrict__ bias_out, void *__restrict__ scale_out,
     const uint32_t *__restrict__ flags, int token_blocks,
-    const void *__restrict__ other, float *__restrict__ grad_gates)
+    const void *__restrict__ other, float *__restrict__ grad_gates,
+    const void *__restrict__ other_bias, const void *__restrict__ other_scale)
 {
     using E = Elem<DT>;
     constexpr int V = E::VEC;
@@ -60,22 +65,46 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
 
     // gate gradient of one choice: <x[t], other[slot]> (GatingDecoder.backward, fast_dispatch.py:73-78)
     auto dot_with = [&](int s) {
-        const uint4 *orow = reinterpret_cast<const uint4 *>((const char *)other + (int64_t)s * model_dim * (int64_t)sizeof(typename E::store_t));
         float acc = 0.f;
-        auto visit = [&](const uint4 &a, const uint4 &b) {
-            float fa[V], fb[V];
-            E::unpack(a, fa); E::unpack(b, fb);
+        if constexpr (CODED) {
+            // V codes per unit: one or two 32-bit words
+            using cword_t = typename std::conditional<V == 8, uint2, uint32_t>::type;
+            const cword_t *crow = reinterpret_cast<const cword_t *>((const uint8_t *)other + (int64_t)s * model_dim);
+            const RowDecoder<DT> dec(E::load(other_bias, s), E::load(other_scale, s));
+            auto visit = [&](const uint4 &a, const cword_t &cw) {
+                float fa[V], fb[V];
+                E::unpack(a, fa);
+                if constexpr (V == 8) { dec.word(cw.x, fb); dec.word(cw.y, fb + 4); }
+                else dec.word(cw, fb);
 #pragma unroll
-            for (int i = 0; i < V; ++i) acc = fmaf(fb[i], fa[i], acc);
-        };
-        if constexpr (CACHE > 0) {
-            uint4 o[CACHE];
+                for (int i = 0; i < V; ++i) acc = fmaf(fb[i], fa[i], acc);
+            };
+            if constexpr (CACHE > 0) {
+                cword_t o[CACHE];
 #pragma unroll
-            for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) o[c] = orow[c * WAVE + lane];
+                for (int c = 0; c < CACHE; ++c) o[c] = crow[min(c * WAVE + lane, units - 1)];
 #pragma unroll
-            for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) visit(cache_ref(c), o[c]);
+                for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) visit(cache_ref(c), o[c]);
+            } else {
+                for (int u = lane; u < units; u += WAVE) visit(src[u], crow[u]);
+            }
         } else {
-            for (int u = lane; u < units; u += WAVE) visit(src[u], orow[u]);
+            const uint4 *orow = reinterpret_cast<const uint4 *>((const char *)other + (int64_t)s * model_dim * (int64_t)sizeof(typename E::store_t));
+            auto visit = [&](const uint4 &a, const uint4 &b) {
+                float fa[V], fb[V];
+                E::unpack(a, fa); E::unpack(b, fb);
+#pragma unroll
+                for (int i = 0; i < V; ++i) acc = fmaf(fb[i], fa[i], acc);
+            };
+            if constexpr (CACHE > 0) {
+                uint4 o[CACHE];
+#pragma unroll
+                for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) o[c] = orow[c * WAVE + lane];
+#pragma unroll
+                for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) visit(cache_ref(c), o[c]);
+            } else {
+                for (int u = lane; u < units; u += WAVE) visit(src[u], orow[u]);
+            }
         }
         return wave_sum(acc);
     };
@@ -314,17 +343,18 @@ static void launch_dispatch_int8(int per_lane, unsigned grid, hipStream_t st, co
                                  int64_t stride, int top_k, int samples, int model_dim, int experts,
                                  int capacity, uint8_t *codes, void *bias, void *scale,
                                  const uint32_t *flags, int token_blocks, const void *other,
-                                 float *grad_gates)
+                                 float *grad_gates, const void *other_bias, const void *other_scale)
 {
-#define PM_DI8_(CACHE, GATED, GRAD)                                                              \
-    dispatch_int8_kernel<DT, CACHE, GATED, GRAD><<<grid, 256, 0, st>>>(x, gates, indices, locations, stride, \
+#define PM_DI8_(CACHE, GATED, GRAD, CODED)                                                       \
+    dispatch_int8_kernel<DT, CACHE, GATED, GRAD, CODED><<<grid, 256, 0, st>>>(x, gates, indices, locations, stride, \
         top_k, samples, model_dim, experts, capacity, codes, bias, scale, flags, token_blocks,   \
-        other, grad_gates)
+        other, grad_gates, other_bias, other_scale)
 #define PM_DI8(CACHE)                                                                            \
     do {                                                                                         \
-        if (!gates) PM_DI8_(CACHE, false, false);                                                \
-        else if (!grad_gates) PM_DI8_(CACHE, true, false);                                       \
-        else PM_DI8_(CACHE, true, true);                                                         \
+        if (!gates) PM_DI8_(CACHE, false, false, false);                                         \
+        else if (!grad_gates) PM_DI8_(CACHE, true, false, false);                                \
+        else if (!other_bias) PM_DI8_(CACHE, true, true, false);                                 \
+        else PM_DI8_(CACHE, true, true, true);                                                   \
     } while (0)
     if (per_lane <= 2) PM_DI8(2);
     else if (per_lane <= 4) PM_DI8(4);
@@ -343,7 +373,8 @@ static int run_dispatch_int8(const char *who, const void *x, int dtype, const fl
                              const int32_t *indices, const int32_t *locations, int64_t plane_stride,
                              int top_k, int samples, int model_dim, int experts, int capacity,
                              uint8_t *codes, void *bias, void *scale, void *workspace,
-                             size_t workspace_bytes, const void *other, float *grad_gates, void *stream)
+                             size_t workspace_bytes, const void *other, float *grad_gates, void *stream,
+                             const void *other_bias = nullptr, const void *other_scale = nullptr)
 {
     if (check_planes(who, indices, locations, plane_stride, top_k, samples)) return 1;
     PM_REQUIRE(dtype_ok(dtype), "%s: bad dtype %d", who, dtype);
@@ -364,7 +395,8 @@ static int run_dispatch_int8(const char *who, const void *x, int dtype, const fl
     PM_REQUIRE(workspace && workspace_bytes >= planmoe_dispatch_workspace_bytes(experts, capacity),
                "%s: workspace too small", who);
     const int vec = dtype == PLANMOE_F32 ? 4 : 8;
-    PM_REQUIRE(model_dim % vec == 0 && aligned16(x) && ((uintptr_t)codes % 8 == 0) && (!other || aligned16(other)),
+    PM_REQUIRE(model_dim % vec == 0 && aligned16(x) && ((uintptr_t)codes % 8 == 0) &&
+               (!other || (other_bias ? (uintptr_t)other % 8 == 0 : aligned16(other))),
                "%s: model_dim must be a multiple of %d and buffers 16-byte aligned; "
                "use the unfused entry points otherwise", who, vec);
     hipStream_t st = (hipStream_t)stream;
@@ -376,7 +408,7 @@ static int run_dispatch_int8(const char *who, const void *x, int dtype, const fl
     PM_DTYPE_SWITCH(dtype, DT,
         launch_dispatch_int8<DT>(per_lane, (unsigned)(token_blocks + fill_blocks), st, x, gates, indices,
                                  locations, plane_stride, top_k, samples, model_dim, experts, capacity,
-                                 codes, bias, scale, flags, token_blocks, other, grad_gates));
+                                 codes, bias, scale, flags, token_blocks, other, grad_gates, other_bias, other_scale));
     PM_LAUNCH_CHECK(who);
     return 0;
 }
@@ -405,6 +437,21 @@ extern "C" int planmoe_combine_bwd_int8(const void *grad_out, const void *expert
     return run_dispatch_int8("planmoe_combine_bwd_int8", grad_out, dtype, gates, indices, locations,
                              plane_stride, top_k, samples, model_dim, experts, capacity, codes, bias, scale,
                              workspace, workspace_bytes, expert_out, grad_gates, stream);
+}
+
+extern "C" int planmoe_combine_bwd_int8_coded(const void *grad_out, const uint8_t *expert_codes,
+                                              const void *expert_bias, const void *expert_scale, int dtype,
+                                              const float *gates, const int32_t *indices,
+                                              const int32_t *locations, int64_t plane_stride, int top_k,
+                                              int samples, int model_dim, int experts, int capacity,
+                                              uint8_t *codes, void *bias, void *scale, float *grad_gates,
+                                              void *workspace, size_t workspace_bytes, void *stream)
+{
+    PM_REQUIRE(gates && grad_gates && ((expert_codes && expert_bias && expert_scale) || (int64_t)experts * capacity == 0),
+               "planmoe_combine_bwd_int8_coded: gates, the coded expert output and grad_gates must not be NULL");
+    return run_dispatch_int8("planmoe_combine_bwd_int8_coded", grad_out, dtype, gates, indices, locations,
+                             plane_stride, top_k, samples, model_dim, experts, capacity, codes, bias, scale,
+                             workspace, workspace_bytes, expert_codes, grad_gates, stream, expert_bias, expert_scale);
 }
 
 extern "C" int planmoe_combine_int8(const uint8_t *codes, const void *bias, const void *scale, int dtype,

@@ -299,9 +299,29 @@ def dispatch_int8(x, indices, locations, gates, experts, capacity_):
 
 def combine_bwd_int8(grad_out, expert_out, indices, locations, gates, experts, capacity_):
     """GatingDecoder.backward + int8 compress of the gradient buffer in one pass.
+    expert_out: the [E*C, M] tensor fast_decode consumed, or the (codes, bias, scale) triple it was
+    decompressed from (same results, and the decompressed copy need not exist).
     Returns codes [E*C, M] uint8, bias, scale [E*C, 1], grad_gates [k, T] fp32."""
     _need_gpu(grad_out, "combine_bwd_int8")
     g_out = _contig(grad_out, "combine_bwd_int8")
+    if isinstance(expert_out, (tuple, list)):
+        e_codes, e_bias, e_scale = (_contig(t, "combine_bwd_int8") for t in expert_out)
+        if e_bias.dtype != g_out.dtype or e_scale.dtype != g_out.dtype or e_codes.dtype != torch.uint8:
+            raise PlanMoEError("combine_bwd_int8: coded expert output must be uint8 codes with bias / scale in grad_out's dtype")
+        T, M = g_out.shape
+        idx, loc, g, stride = _plane_args(indices, locations, gates, "combine_bwd_int8")
+        k = len(indices)
+        R = experts * capacity_
+        codes = torch.empty((R, M), dtype=torch.uint8, device=g_out.device)
+        bias = torch.empty((R, 1), dtype=g_out.dtype, device=g_out.device)
+        scale = torch.empty_like(bias)
+        gg = torch.empty((k, stride), dtype=torch.float32, device=g_out.device)
+        ws = _ws(lib.planmoe_dispatch_workspace_bytes(experts, capacity_), g_out.device)
+        check(lib.planmoe_combine_bwd_int8_coded(_ptr(g_out), _ptr(e_codes), _ptr(e_bias), _ptr(e_scale),
+                                                 _dt(g_out, "combine_bwd_int8"), _ptr(g), _ptr(idx), _ptr(loc), stride,
+                                                 k, T, M, experts, capacity_, _ptr(codes), _ptr(bias), _ptr(scale),
+                                                 _ptr(gg), _ptr(ws), ws.numel(), _stream(g_out)))
+        return codes, bias, scale, gg[:, :T]
     e_out = _contig(expert_out, "combine_bwd_int8")
     if g_out.dtype != e_out.dtype:
         raise PlanMoEError("combine_bwd_int8: grad_out and expert_out must share a dtype")

@@ -133,9 +133,10 @@ class _DecodeInt8(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         codes, bias, scale, indices, locations, *gates = ctx.saved_tensors
-        seen = ops.int8_decompress(codes, bias, scale)          # the tensor fast_decode consumed
+        # the tensor fast_decode consumed is decoded from its codes on the fly
         gcodes, gbias, gscale, grad_gates = ops.combine_bwd_int8(
-            grad_out.contiguous(), seen, list(indices), list(locations), list(gates), ctx.experts, ctx.capacity)
+            grad_out.contiguous(), (codes, bias, scale), list(indices), list(locations), list(gates), ctx.experts,
+            ctx.capacity)
         grad_y = ops.int8_decompress(gcodes, gbias, gscale)
         return (grad_y, None, None, None, None, None,
                 *[grad_gates[j].to(g.dtype) for j, g in enumerate(gates)])

@@ -271,6 +271,13 @@ def test_combine_bwd_int8_equals_the_unfused_backward(T, M, E, k, cf, dtype):
         assert (np.abs(got - want) <= rtol * np.abs(want) + 1e-6 * mag).all()
         assert (got[loc[j] >= C] == 0).all()
         assert np.allclose(got, g2[j].cpu().numpy(), rtol=1e-5, atol=1e-6 * mag.max())
+    # the expert output handed over as int8 codes: decoded on the fly to what int8_decompress gives
+    ec, eb, es = ops.int8_compress(eo.to(DEV))
+    seen = ops.int8_decompress(ec, eb, es)
+    c3, b3, s3, g3 = ops.combine_bwd_int8(dout.to(DEV), seen, i, l, gt, E, C)
+    c4, b4, s4, g4 = ops.combine_bwd_int8(dout.to(DEV), (ec, eb, es), i, l, gt, E, C)
+    assert torch.equal(c3, c4) and torch.equal(b3, b4) and torch.equal(s3, s4)
+    assert np.array_equal(raw(g3), raw(g4))
 
 
 @pytest.mark.parametrize("T,M,E,k,dtype,gated", [(1000, 512, 8, 2, torch.bfloat16, True), (300, 264, 5, 3, torch.bfloat16, False),
