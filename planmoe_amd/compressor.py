@@ -3,12 +3,19 @@ custom/compressor/* classes and of the compress / comm / decompress operations o
 custom/custom_kernel.cpp:194-288 (the pybind surface of ``schemoe_custom_kernel``).
 
 Objects are stateful and single use, exactly as in the reference: ``compress`` records what
-``decompress`` needs.  With one GPU the all-to-all is the identity: ``all_to_all`` copies the
-send buffer into ``g_output`` and the per-row state into its receive-side twins."""
+``decompress`` needs.  With one GPU the all-to-all is the identity: ``comm_operation`` hands the
+send buffers over as the receive buffers, or (``SINGLE_RANK_COMM_COPIES``) ``all_to_all`` copies
+the send buffer into ``g_output`` and the per-row state into its receive-side twins."""
 import torch
 
 from . import ops
 from ._lib import PlanMoEError
+
+
+# One rank: what the all-to-all delivers is what was sent.  With False the send buffers are handed
+# over as the receive buffers (no device copy); with True they are copied into g_output, as a
+# one-rank all_to_all of the reference would (naive.cpp:11-27).
+SINGLE_RANK_COMM_COPIES = False
 
 
 class AbstractComm:
@@ -43,6 +50,10 @@ class AbstractCompressor:
 
     def all_to_all(self, input, output):
         raise NotImplementedError
+
+    def adopt(self, input):
+        """One rank, no copy: the receive-side state is the send-side state."""
+        self.g_output = input
 
     def pre_comm(self, stream):
         pass
@@ -85,6 +96,9 @@ class Int8Compressor(AbstractCompressor):
         self.comm_ptr.all_to_all(input, output, self.length)
         self.comm_ptr.all_to_all(self.bias, self.g_bias, self.bias.numel() * self.bias.element_size())
         self.comm_ptr.all_to_all(self.scale, self.g_scale, self.scale.numel() * self.scale.element_size())
+
+    def adopt(self, input):
+        self.g_output, self.g_bias, self.g_scale = input, self.bias, self.scale
 
 
 class ZfpCompressor(AbstractCompressor):
@@ -155,6 +169,11 @@ class LzCompressor(AbstractCompressor):
                          (self.compressedDataGlobal, self.g_compressedDataGlobal)):
             self.comm_ptr.all_to_all(src, dst, src.numel() * src.element_size())
 
+    def adopt(self, input):
+        # g_output stays the zeroed twin the decoder writes into
+        self.g_flagArrOffsetGlobal, self.g_compressedDataOffsetGlobal = self.flagArrOffsetGlobal, self.compressedDataOffsetGlobal
+        self.g_flagArrGlobal, self.g_compressedDataGlobal = self.flagArrGlobal, self.compressedDataGlobal
+
 
 def get_compressor(name, comm_ptr):
     # custom_kernel.cpp:194-207
@@ -198,7 +217,10 @@ def comm_operation(input):
     _comm_cnt += 1
     c = _compress_ptr_lst[idx]
     c.pre_comm(None)
-    c.all_to_all(input, c.g_output)
+    if c.comm_ptr.g_world_size == 1 and not SINGLE_RANK_COMM_COPIES:
+        c.adopt(input)
+    else:
+        c.all_to_all(input, c.g_output)
     return c.g_output
 
 

@@ -71,6 +71,8 @@ def a2a_ffn_overlap_forward(input, expert_fn, a2a_ffn_overlap_degree, use_2dh, g
         input_split[i] = Comm.apply(input_split[i])
     for i in range(a2a_ffn_overlap_degree):
         input_split[i] = Decompress.apply(input_split[i], compress_name, comm_name)
+    if a2a_ffn_overlap_degree == 1:
+        return input_split[0].contiguous()              # nothing to put together
     return torch.cat(input_split, dim=split_dim).contiguous()
 
 
@@ -173,7 +175,7 @@ class _GateRouteEncodeInt8(torch.autograd.Function):
                                         counts if grad_l_aux is not None else None, through_softmax=True)
             g = grad_logits.to(x.dtype)
             dw = g.t() @ x
-            dx = g @ w if dx is None else dx + g @ w
+            dx = g @ w if dx is None else torch.addmm(dx, g, w)       # the sum rides in the GEMM's epilogue
         return dx, dw, None, None, None, None
 
 

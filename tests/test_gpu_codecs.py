@@ -198,9 +198,19 @@ def test_zfp_config5_full_size(dims):
     assert (dec2 - dec).abs().max().item() <= err
 
 
-def test_compressor_registry_round_trips():
-    """compress_operation / comm_operation / decompress_operation with 'no', 'int8', 'zfp'."""
+@pytest.mark.parametrize("copies", [False, True])
+def test_compressor_registry_round_trips(copies):
+    """compress_operation / comm_operation / decompress_operation with 'no', 'int8', 'zfp', 'lz';
+    the one-rank comm step hands the buffers over (default) or copies them."""
     from planmoe_amd import compressor
+    compressor.SINGLE_RANK_COMM_COPIES = copies
+    try:
+        _registry_round_trips(compressor, copies)
+    finally:
+        compressor.SINGLE_RANK_COMM_COPIES = False
+
+
+def _registry_round_trips(compressor, copies):
     g = torch.Generator().manual_seed(1)
     x = torch.randn(4, 64, 256, generator=g).to(DEV)
     compressor.clear_ptr_lst()
@@ -212,6 +222,7 @@ def test_compressor_registry_round_trips():
     assert outs[1][1].dtype == torch.float32 and outs[1][1].numel() == x.numel() // 4
     assert outs[2][1].dtype == torch.float16 and outs[2][1].numel() == (oracle.zfp_max_bytes(2, 256, 256) + 1) // 2
     recv = [compressor.comm_operation(c) for _, c in outs]
+    assert all((r.data_ptr() != c.data_ptr()) == copies for r, (_, c) in zip(recv, outs))
     dec = [compressor.decompress_operation(r) for r in recv]
     assert torch.equal(dec[0], x)
     rc, rb, rs = oracle.int8_compress(x.cpu().numpy())
