@@ -222,7 +222,7 @@ def layer_table():
                 y = layer(x)
                 (y.float().mean() + y.l_aux.float()).backward()
                 x.grad = None
-            times.append(event_time_us(step, 5, 3, rounds=3)[0] / 1e3)
+            times.append(event_time_us(step, 5, 5, rounds=5)[1] / 1e3)      # median of the rounds
         overlap.FUSE_INT8 = overlap.FUSE_GATE = overlap.FUSE_ZFP = True
         print("%-4s %-6s %-9s %14.3f %14.3f" % (cfg, codec, str(dtype).replace("torch.", ""), times[0], times[1]))
 
