@@ -98,24 +98,31 @@ __global__ __launch_bounds__(256) void combine_kernel(
     if (top_k <= WAVE) {
         int slot; float gate;
         fetch_planes(gates, indices, locations, stride, t, 0, top_k, 0x7fffffff, capacity, slot, gate);
-        for (int u = lane; u < units; u += WAVE) {
-            float acc[IO::U];
+        // four units of a row per lane and pass, fetched with straight-line loads at clamped
+        // addresses (a dropped choice reads slot 0 and contributes zeros): four loads in flight
+        // per choice instead of one load, one wait
+        constexpr int B = 4;
+        for (int u0 = lane; u0 < units; u0 += B * WAVE) {
+            float acc[B][IO::U];
             for (int j = 0; j < top_k; ++j) {
                 const int s = rl_i(slot, j);
                 const float g = rl_f(gate, j);
-                float term[IO::U];
-                if (s >= 0) {
-                    IO::load((const char *)dispatched + (int64_t)s * row_bytes, u, term);
+                const char *row = (const char *)dispatched + (int64_t)max(s, 0) * row_bytes;
+                float term[B][IO::U];
 #pragma unroll
-                    for (int i = 0; i < IO::U; ++i) term[i] = g * term[i];
-                } else {
+                for (int b = 0; b < B; ++b) IO::load(row, min(u0 + b * WAVE, units - 1), term[b]);
 #pragma unroll
-                    for (int i = 0; i < IO::U; ++i) term[i] = 0.f;
+                for (int b = 0; b < B; ++b) {
+#pragma unroll
+                    for (int i = 0; i < IO::U; ++i) {
+                        const float v = s >= 0 ? g * term[b][i] : 0.f;
+                        acc[b][i] = (j == 0) ? v : acc[b][i] + v;
+                    }
                 }
-#pragma unroll
-                for (int i = 0; i < IO::U; ++i) acc[i] = (j == 0) ? term[i] : acc[i] + term[i];
             }
-            IO::store(dst, u, acc);
+#pragma unroll
+            for (int b = 0; b < B; ++b)
+                if (u0 + b * WAVE < units) IO::store(dst, u0 + b * WAVE, acc[b]);
         }
     } else {
         // more planes than lanes: walk the planes straight from memory
@@ -140,6 +147,16 @@ __global__ __launch_bounds__(256) void combine_kernel(
             IO::store(dst, u, acc);
         }
     }
+}
+
+template <int DT, bool VECTOR>
+__global__ __launch_bounds__(256) void zero_rows_kernel(void *__restrict__ out, int samples, int model_dim)
+{
+    using IO = RowIO<DT, VECTOR>;
+    const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= samples) return;
+    char *dst = (char *)out + (int64_t)t * model_dim * (int64_t)sizeof(typename Elem<DT>::store_t);
+    for (int u = lane_id(); u < model_dim / IO::U; u += WAVE) IO::store_zero(dst, u);
 }
 
 // ------------------------------------------------------------------ gate gradient
@@ -275,6 +292,16 @@ extern "C" int planmoe_combine_fwd(const void *dispatched, int dtype, const floa
     const int vec = dtype == PLANMOE_F32 ? 4 : 8;
     const bool vector = (model_dim % vec == 0) && aligned16(out) && aligned16(dispatched);
     const int blocks = (samples + 3) / 4;
+    if (capacity == 0) {
+        // no slot exists, every choice is dropped: zero rows.  (combine_kernel fetches rows with
+        // unconditional loads at clamped slots and must not run without a row to read.)
+        PM_DTYPE_SWITCH(dtype, DT, {
+            if (vector) zero_rows_kernel<DT, true><<<blocks, 256, 0, st>>>(out, samples, model_dim);
+            else zero_rows_kernel<DT, false><<<blocks, 256, 0, st>>>(out, samples, model_dim);
+        });
+        PM_LAUNCH_CHECK("planmoe_combine_fwd");
+        return 0;
+    }
     PM_DTYPE_SWITCH(dtype, DT, {
         if (vector)
             combine_kernel<DT, true><<<blocks, 256, 0, st>>>(dispatched, gates, indices, locations,
