@@ -70,6 +70,7 @@ def kernel_table(only=None):
     dev = "cuda:0"
     g = torch.Generator().manual_seed(0)
     rows = []
+    scrub = torch.zeros((1 << 28,), dtype=torch.int32, device=dev)
 
     def add(name, cfg, nbytes, fn, iters=20):
         if only and only not in "%s [%s]" % (name, cfg):
@@ -84,8 +85,25 @@ def kernel_table(only=None):
             for _ in range(iters):
                 fn()
         avg, med, best = event_time_us(graph.replay, 1, 1, rounds=5)
-        rows.append((name, cfg, nbytes, avg / iters, best / iters))
         del graph
+        # cold: every call behind a pass over 1 GiB that leaves none of the call's operands in the
+        # L2s or the 256 MB memory-side cache; one event pair per call (the scrub runs long enough
+        # for the host to have the call enqueued before the device reaches it).  Two scrubs: one
+        # that only reads (the caches hold clean lines of other data) and one that also writes
+        # (they hold dirty lines, whose write-back then falls into the timed call).
+        cold = []
+        for scrub_fn in (lambda: torch.max(scrub), lambda: scrub.add_(1)):
+            pairs = []
+            for _ in range(7):
+                scrub_fn()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                fn()
+                b.record()
+                pairs.append((a, b))
+            torch.cuda.synchronize()
+            cold.append(sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)[len(pairs) // 2])
+        rows.append((name, cfg, nbytes, avg / iters, best / iters, cold[0], cold[1]))
 
     # configs 2 / 4: 16384 tokens x 4096, 8 experts, top-2, capacity_factor 1.25, bf16
     T, M, E, k = 16384, 4096, 8, 2
@@ -183,10 +201,81 @@ def kernel_table(only=None):
         out = torch.empty_like(buf)
         add("lz_decompress %s" % label, "5", buf.numel() * 4 + used, lambda: ops.lz_decompress(out, fo, do, fl, da), iters=5)
 
-    print("%-30s %-4s %10s %9s %9s %8s %6s" % ("entry point", "cfg", "alg MB", "avg us", "best us", "GB/s", "frac"))
-    for name, cfg, nbytes, avg, best in rows:
+    print("%-30s %-4s %10s %9s %9s %8s %6s %10s %10s" % ("entry point", "cfg", "alg MB", "avg us", "best us", "GB/s", "frac",
+                                                         "cold-r us", "cold-w us"))
+    for name, cfg, nbytes, avg, best, cold_r, cold_w in rows:
         gbs = nbytes / avg / 1e3
-        print("%-30s %-4s %10.1f %9.1f %9.1f %8.0f %6.2f" % (name, cfg, nbytes / 1e6, avg, best, gbs, gbs / HBM_PEAK_GBS))
+        print("%-30s %-4s %10.1f %9.1f %9.1f %8.0f %6.2f %10.1f %10.1f" % (name, cfg, nbytes / 1e6, avg, best, gbs,
+                                                                         gbs / HBM_PEAK_GBS, cold_r, cold_w))
+
+
+def cpu_stage_table(min_seconds=2.0):
+    """The CPU oracle, one thread, stage by stage on bounded samples of the same workloads (the
+    first `sample` tokens or rows; slot capacity recomputed for the sample): seconds per call and
+    algorithmic bytes per second, to set beside the device table of --kernels."""
+    import numpy as np
+    import oracle
+    rng = np.random.default_rng(0)
+    rows = []
+
+    def add(name, cfg, sample, nbytes, fn):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt >= min_seconds:
+                break
+        rows.append((name, cfg, sample, nbytes, dt / reps))
+
+    # configs 2 / 4 on 4096 of the 16384 tokens (bf16 data as the fp32 the reference computes in)
+    T, M, E, k = 4096, 4096, 8, 2
+    C = oracle.capacity(T, E, k, 1.25, 4); R = E * C
+    xb = (rng.standard_normal((T, M), dtype=np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    wb = ((rng.standard_normal((E, M), dtype=np.float32) * M ** -0.5).view(np.uint32) >> 16).astype(np.uint16)
+    x = (xb.astype(np.uint32) << 16).view(np.float32)
+    logits = oracle.gate_logits(xb, wb).astype(np.float32)
+    scores = oracle.softmax(logits)
+    idx, loc, gates, _ = oracle.route_topk(scores, k)
+    idx, loc, gates = list(idx), list(loc), list(gates)
+    tok = "%d tokens" % T
+    add("gate_logits", "2", tok, T * M * 2 + E * M * 2 + T * E * 4, lambda: oracle.gate_logits(xb, wb))
+    add("softmax + route_topk", "2", tok, T * E * 4 + T * k * 12, lambda: oracle.route_topk(oracle.softmax(logits), k))
+    add("dispatch_fwd (encode)", "2", tok, T * M * 2 + R * M * 2, lambda: oracle.encode(x, idx, loc, None, E, C))
+    d = oracle.encode(x, idx, loc, None, E, C)
+    add("combine_fwd (decode)", "2", tok, T * k * M * 2 + T * M * 2, lambda: oracle.decode(d, idx, loc, gates, T, C))
+    add("bwd_gate", "2", tok, T * k * M * 2 + T * M * 2,
+        lambda: [oracle.bwd_gate(idx[j], loc[j], x, d, C) for j in range(k)])
+    db = (d.view(np.uint32) >> 16).astype(np.uint16)
+    add("int8_compress", "2", tok, R * M * 2 + R * M, lambda: oracle.int8_compress(db))
+    codes, bias, scale = oracle.int8_compress(db)
+    add("int8_decompress", "2", tok, R * M * 2 + R * M, lambda: oracle.int8_decompress(codes, bias, scale))
+
+    # config 3's routing: 64 experts, top-1
+    T3, E3 = 8192, 64
+    mask = (rng.random((T3, E3)) < 0.1).astype(np.int32)
+    add("cumsum_sub_one", "3", "%d tokens" % T3, 2 * T3 * E3 * 4, lambda: oracle.cumsum_sub_one(mask))
+    s3 = oracle.softmax(rng.standard_normal((T3, E3), dtype=np.float32))
+    add("route_topk", "3", "%d tokens" % T3, T3 * E3 * 4 + T3 * 12, lambda: oracle.route_topk(s3, 1))
+
+    # config 5's codecs on 2048 of the 131072 slot rows
+    R5, M5 = 2048, 1024
+    f = rng.standard_normal((R5, M5), dtype=np.float32)
+    rw = "%d rows" % R5
+    for dims in (2, 1):
+        add("zfp_compress %d-D" % dims, "5", rw, R5 * M5 * 5, lambda: oracle.zfp_compress(f, dims))
+        st = oracle.zfp_compress(f, dims)
+        add("zfp_decompress %d-D" % dims, "5", rw, R5 * M5 * 5, lambda: oracle.zfp_decompress(st, R5, M5, dims))
+    f[rng.random(R5) < 0.3] = 0.0
+    add("lz_compress 30% empty", "5", rw, R5 * M5 * 4, lambda: oracle.lz_compress(f))
+    lz = oracle.lz_compress(f)
+    add("lz_decompress 30% empty", "5", rw, R5 * M5 * 4, lambda: oracle.lz_decompress(*lz))
+
+    print("CPU oracle, 1 thread of %d (%s)" % (os.cpu_count(), "bounded samples; GB/s of algorithmic bytes"))
+    print("%-26s %-4s %-12s %10s %10s %8s" % ("stage", "cfg", "sample", "alg MB", "ms / call", "GB/s"))
+    for name, cfg, sample, nbytes, sec in rows:
+        print("%-26s %-4s %-12s %10.1f %10.2f %8.3f" % (name, cfg, sample, nbytes / 1e6, sec * 1e3, nbytes / sec / 1e9))
 
 
 def layer_table():
@@ -243,11 +332,19 @@ def main():
     ap.add_argument("--layer", action="store_true",
                     help="instead of the JSON line, time moe_layer forward + backward with identity experts for "
                          "every compressor, with and without the fused entry points")
+    ap.add_argument("--cpu-stages", action="store_true",
+                    help="instead of the JSON line, time the CPU oracle (one thread) stage by stage on bounded "
+                         "samples of the same workloads; needs no GPU")
     ap.add_argument("--only", default=None, help="with --kernels: only the lines whose 'name [config]' contains this, e.g. lz_ or [5]")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU's share of the path; --gpus %d is not supported "
                  "(nothing here uses a second GPU)" % args.gpus)
+    if args.cpu_stages:
+        import __graft_entry__
+        __graft_entry__.ensure_built()
+        cpu_stage_table()
+        return
     if args.kernels or args.layer:
         import __graft_entry__
         __graft_entry__.ensure_built()
@@ -307,6 +404,21 @@ def main():
     stages["dispatch_int8_routed"] = event_time_us(plan.redispatch, 30, 5)
     chain_ev = event_time_us(chain, 30, 5)
 
+    # the chain with none of its operands in the L2s or the 256 MB memory-side cache: a reduction
+    # over 1 GiB of other data before every call, one event pair per call, median of 9
+    scrub = torch.zeros((1 << 28,), dtype=torch.int32, device=dev)
+    pairs = []
+    for _ in range(9):
+        torch.max(scrub)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        chain()
+        b.record()
+        pairs.append((a, b))
+    torch.cuda.synchronize()
+    cold_us = sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)[len(pairs) // 2]
+    del scrub
+
     # algorithmic bytes: every input read once, every output written once
     chain_bytes = T * M * 2 + R * M + R * 2 * 2 + T * k * 12 + E * M * 2
     dom_bytes = T * M * 2 + R * M + R * 2 * 2 + T * k * 12         # last launch alone: x, codes, bias/scale, idx/rank/loc
@@ -330,6 +442,7 @@ def main():
                      "algorithmic_bytes": dom_bytes, "avg_us": dom_avg_us},
         "chain": {"algorithmic_bytes": chain_bytes, "device_us_avg": chain_ev[0], "device_us_min": chain_ev[2],
                   "GBps": chain_bytes / chain_ev[0] / 1e3, "frac_of_hbm_peak": chain_bytes / chain_ev[0] / 1e3 / HBM_PEAK_GBS,
+                  "device_us_cold_caches": cold_us,
                   "stage_us_avg": {n: v[0] for n, v in stages.items()}},
     }
     if args.cpu_sample > 0:
