@@ -51,6 +51,16 @@ __global__ __launch_bounds__(256) void int8_compress_vec_kernel(
     if (lane == 0) { E::store(bias_out, r, mn); E::store(scale_out, r, scale); }
 
     uint8_t *dst = codes + r * row_len;
+    // A scale of 0 (constant row: an empty capacity slot), infinity or NaN turns every quotient into
+    // 0 or NaN, and both encode to 0: such rows are written as zeros without going through the
+    // quantiser (which would take the IEEE division for them).
+    if (!(scale > 0.f && scale < INFINITY)) {
+        for (int u = lane; u < units; u += WAVE) {
+            if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(dst) + u, make_uint2(0u, 0u));
+            else stream_store(reinterpret_cast<uint32_t *>(dst) + u, 0u);
+        }
+        return;
+    }
     const RowEncoder<DT> enc(mn, scale);
     auto body = [&](auto mode) {
         constexpr bool FAST = decltype(mode)::value;

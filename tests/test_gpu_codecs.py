@@ -77,6 +77,45 @@ def test_int8_nan_row():
     assert torch.isnan(bias[1]).all() and torch.isnan(scale[1]).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+@pytest.mark.parametrize("M", [64, 4096, 37])
+def test_int8_rows_without_a_usable_scale(dtype, M):
+    """Rows whose scale is 0, infinite or NaN (all codes 0) next to rows whose scale is merely
+    extreme (IEEE division), against the literal torch-CPU op chain and the oracle."""
+    from planmoe_amd import ops
+    big = {torch.bfloat16: 3e38, torch.float32: 3e38, torch.float16: 6e4}[dtype]
+    tiny = {torch.bfloat16: 2.0 ** -120, torch.float32: 2.0 ** -120, torch.float16: 2.0 ** -20}[dtype]
+    x = torch.randn(12, M, generator=torch.Generator().manual_seed(M)).to(dtype)
+    x[0] = 2.5                                             # constant
+    x[1] = 0.0; x[1, ::2] = -0.0                           # +0 / -0
+    x[2, 3] = float("inf")
+    x[3, 5] = float("-inf")
+    x[4] = float("inf")
+    x[5] = float("-inf")
+    x[6, 0] = big; x[6, 1] = -big                          # max - min overflows
+    x[7, 7] = float("nan")
+    x[8, 1] = float("inf"); x[8, 2] = float("-inf")
+    x[9] = (torch.randn(M) * tiny).to(dtype)               # tiny but usable scale
+    x[10] = (torch.randn(M) * (big / 8)).to(dtype)         # huge but finite scale
+    codes, bias, scale = ops.int8_compress(x.to(DEV))
+    b = torch.min(x, -1, True)[0]; sc = torch.max(x, -1, True)[0] - b
+    want = torch.mul(torch.div(torch.sub(x, b), sc), 255.0).to(torch.uint8)
+    usable = (sc.view(-1) > 0) & torch.isfinite(sc.view(-1))
+    assert usable.tolist() == [False] * 9 + [True] * 3
+    # float -> uint8 of NaN is not defined by torch; every backend here gives 0, the oracle pins 0
+    want[~usable] = 0
+    assert np.array_equal(codes.cpu().numpy(), want.numpy())
+
+    def same(got, ref):                                    # bit for bit, any NaN for a NaN (inf - inf has no fixed sign)
+        got, ref = got.cpu().view(-1), ref.view(-1)
+        nan = torch.isnan(ref)
+        return torch.equal(torch.isnan(got), nan) and np.array_equal(raw(got[~nan]), raw(ref[~nan]))
+    assert same(bias, b) and same(scale, sc)
+    if dtype != torch.float16:
+        rc, rb, rs = oracle.int8_compress(to_np(x))
+        assert np.array_equal(codes.cpu().numpy(), rc)
+
+
 def test_int8_config2_full_size():
     """[8, 5120, 4096] bf16: codes checked on a row sample against the oracle, everything through
     invariants (row min -> 0, row max -> 255, |decode - x| <= scale/255 + bf16 rounding)."""
