@@ -161,6 +161,9 @@ def kernel_table(only=None):
     add("gate_route (gate + routing)", "3", T3 * M3 * 2 + T3 * 12, lambda: ops.gate_route(x3, w3, 1, logit_bias=bias))
     add("forward_int8 (chain)", "3", T3 * M3 * 2 + E3 * C3 * M3 + T3 * 12,
         lambda: ops.forward_int8(x3, w3, 1, C3, logit_bias=bias))
+    r3 = ops.gate_route(x3, w3, 1, logit_bias=bias)
+    i3, l3 = list(r3["indices"]), list(r3["locations"])
+    add("dispatch_fwd", "3", T3 * M3 * 2 + E3 * C3 * M3 * 2 + T3 * 12, lambda: ops.dispatch_fwd(x3, i3, l3, None, E3, C3))
     lg = ops.gate_logits(x3, w3, torch.float32)
     add("route_topk (logits in)", "3", T3 * E3 * 4 + T3 * 12, lambda: ops.route_topk(lg, 1, is_logits=True, logit_bias=bias))
     mask = (torch.rand(T3, E3, device=dev) < 0.1).to(torch.int32)
