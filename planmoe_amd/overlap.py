@@ -6,6 +6,7 @@ import torch
 
 from . import compressor as _ck
 from . import ops
+from .gates import weight_grad
 
 MAX_NUM_SPLIT = 32     # AllToAllStatus.max_num_split of the reference (communicate.py)
 
@@ -174,8 +175,8 @@ class _GateRouteEncodeInt8(torch.autograd.Function):
             grad_logits = ops.route_bwd(scores, indices, grad_gates.contiguous(), ctx.normalize_gate, grad_l_aux,
                                         counts if grad_l_aux is not None else None, through_softmax=True)
             g = grad_logits.to(x.dtype)
-            dw = g.t() @ x
-            dx = g @ w if dx is None else torch.addmm(dx, g, w)       # the sum rides in the GEMM's epilogue
+            dw = weight_grad(g, x)
+            dx = g @ w if dx is None else dx.addmm_(g, w)             # the sum rides in the GEMM's epilogue, in place
         return dx, dw, None, None, None, None
 
 
