@@ -16,7 +16,8 @@ from . import losses, ops
 from .fast_dispatch import extract_critical, fast_decode, fast_encode, route
 from . import overlap as _overlap
 from .overlap import (a2a_ffn_overlap_forward, fused_gate_eligible, fused_gate_forward, fused_int8_eligible,
-                      fused_int8_forward, fused_zfp_eligible, fused_zfp_forward)
+                      fused_int8_forward, fused_zfp_eligible, fused_zfp_forward, gate_route_eligible,
+                      gate_route_encode, zfp_experts_decode)
 
 
 class MOELayer(torch.nn.Module):
@@ -171,6 +172,34 @@ class MOELayer(torch.nn.Module):
                 return self.expert_local(expert_input, original_shape[-reserve_dims:])
             y, l_aux = fused_gate_forward(x, gctx, kk, cap, self.normalize_gate, expert_fn, degree)
             l_aux = l_aux.to(torch.float32 if gctx.fp32_gate else x.dtype)
+            y = y.view(list(original_shape)).to(original_dtype)
+            self.l_aux = y.l_aux = l_aux
+            return self.result_func(y) if self.result_func is not None else y
+
+        if plain and not noisy and gate_route_eligible(x, gctx, self.num_global_experts, self.is_postscore):
+            # gate GEMM + routing as one call and one node of the graph together with the encode (the
+            # same routing and the same bits as the steps below); codec, comm and decode as below
+            kk = min(k, self.num_global_experts)
+            cap = ops.capacity(x.size(0), self.num_global_experts, kk, cf, alignment)
+            zfp = fused_zfp_eligible(x, self.compress_name, degree, self.is_postscore, self.num_global_experts, cap)
+            y, gates, l_aux, indices, locations = gate_route_encode(x, gctx, kk, cap, self.normalize_gate,
+                                                                    'zfp' if zfp else 'plain')
+            l_aux = l_aux.to(torch.float32 if gctx.fp32_gate else x.dtype)
+            if self.training:
+                self.save_count = self.save_count + 1
+
+            def expert_fn(expert_input):
+                return self.expert_local(expert_input, original_shape[-reserve_dims:])
+            y = y.view(self.num_global_experts, cap, x.shape[-1])
+            if zfp:
+                y = zfp_experts_decode(y, expert_fn, degree, indices, locations, gates, x.shape[0])
+            else:
+                y = a2a_ffn_overlap_forward(y, expert_fn=expert_fn, a2a_ffn_overlap_degree=degree,
+                                            use_2dh=self.use_2dh, group=self.group,
+                                            compress_name=self.compress_name, comm_name=self.comm_name)
+                crit = (self.num_global_experts, [indices[j] for j in range(kk)],
+                        [locations[j] for j in range(kk)], [gates[j] for j in range(kk)], cap)
+                y = fast_decode(y.to(x.dtype), crit, self.is_postscore)
             y = y.view(list(original_shape)).to(original_dtype)
             self.l_aux = y.l_aux = l_aux
             return self.result_func(y) if self.result_func is not None else y

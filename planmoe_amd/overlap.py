@@ -57,7 +57,8 @@ def a2a_ffn_overlap_forward(input, expert_fn, a2a_ffn_overlap_degree, use_2dh, g
         "Excepting input.shape[%d] (%d) be multiple of a2a_ffn_overlap_degree (%d)." % (
             split_dim, input.shape[split_dim], a2a_ffn_overlap_degree)
     split_size = input.shape[split_dim] // a2a_ffn_overlap_degree
-    input_split = list(input.split(split_size, dim=split_dim))
+    # (one slice: the tensor itself -- the backward of a split is a cat, i.e. a copy of the whole gradient)
+    input_split = [input] if a2a_ffn_overlap_degree == 1 else list(input.split(split_size, dim=split_dim))
     _ck.clear_ptr_lst()
 
     for i in range(a2a_ffn_overlap_degree):
@@ -165,19 +166,86 @@ class _GateRouteEncodeInt8(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_y, grad_gates, grad_l_aux, *unused):
         x, w, scores, indices, locations, counts = ctx.saved_tensors
-        dx = dw = None
+        dx = None
         if grad_y is not None:
             codes, bias, scale = ops.int8_compress(grad_y.contiguous())
             dx = ops.combine_int8(codes, bias, scale, list(indices), list(locations), None, x.shape[0], ctx.capacity)
-        if grad_gates is not None or grad_l_aux is not None:
-            if grad_gates is None:
-                grad_gates = torch.zeros((indices.shape[0], x.shape[0]), dtype=scores.dtype, device=x.device)
-            grad_logits = ops.route_bwd(scores, indices, grad_gates.contiguous(), ctx.normalize_gate, grad_l_aux,
-                                        counts if grad_l_aux is not None else None, through_softmax=True)
-            g = grad_logits.to(x.dtype)
-            dw = weight_grad(g, x)
-            dx = g @ w if dx is None else dx.addmm_(g, w)             # the sum rides in the GEMM's epilogue, in place
+        dx, dw = _gate_backward(x, w, scores, indices, counts, ctx.normalize_gate, dx, grad_gates, grad_l_aux)
         return dx, dw, None, None, None, None
+
+
+def _gate_backward(x, w, scores, indices, counts, normalize_gate, dx, grad_gates, grad_l_aux):
+    """Gradients of the gates and of l_aux back through planmoe_route_bwd to the logits, and from
+    there into x (added to dx, the gradient through the dispatched rows, in the GEMM's epilogue)
+    and into the gate weight."""
+    if grad_gates is None and grad_l_aux is None:
+        return dx, None
+    if grad_gates is None:
+        grad_gates = torch.zeros((indices.shape[0], x.shape[0]), dtype=scores.dtype, device=x.device)
+    grad_logits = ops.route_bwd(scores, indices, grad_gates.contiguous(), normalize_gate, grad_l_aux,
+                                counts if grad_l_aux is not None else None, through_softmax=True)
+    g = grad_logits.to(x.dtype)
+    dw = weight_grad(g, x)
+    dx = g @ w if dx is None else dx.addmm_(g, w)
+    return dx, dw
+
+
+class _GateRouteEncode(torch.autograd.Function):
+    """Gate GEMM, routing and fast_encode as one node of the graph for the compressors without an
+    int8 send side: x has one consumer, so its two gradients (through the dispatched rows and
+    through the gate) meet in the epilogue of one GEMM instead of a pass of their own.
+    codec 'plain': x -> the [E * C, M] buffer (planmoe_gate_route + planmoe_dispatch_fwd);
+    codec 'zfp':   x -> Decompress(Comm(Compress(buffer))) (planmoe_dispatch_zfp, as _EncodeZfp).
+    Outputs as _GateRouteEncodeInt8."""
+
+    @staticmethod
+    def forward(ctx, x, w, top_k, experts, capacity, fp32_gate, normalize_gate, codec):
+        out = ops.gate_route(x, w, top_k, fp32_gate=fp32_gate, normalize_gate=normalize_gate,
+                             want_scores=True, want_counts=True)
+        indices, locations = out["indices"], out["locations"]
+        ctx.save_for_backward(x, w, out["scores"], indices, locations, out["counts"])
+        ctx.experts, ctx.capacity, ctx.normalize_gate, ctx.codec = experts, capacity, normalize_gate, codec
+        ctx.mark_non_differentiable(indices, locations)
+        if codec == 'zfp':
+            stream = ops.dispatch_zfp(x, list(indices), list(locations), None, experts, capacity)
+            y = ops.zfp_decompress(stream, x.shape[1], experts * capacity, 2)
+        else:
+            y = ops.dispatch_fwd(x, list(indices), list(locations), None, experts, capacity)
+        return y, out["gates"], out["l_aux"], indices, locations
+
+    @staticmethod
+    def backward(ctx, grad_y, grad_gates, grad_l_aux, *unused):
+        x, w, scores, indices, locations, counts = ctx.saved_tensors
+        dx = None
+        if grad_y is not None:
+            grad_y = grad_y.contiguous()
+            if ctx.codec == 'zfp':
+                R, M = grad_y.shape
+                stream = ops.zfp_compress(grad_y, M, R, 2)
+                dx = ops.combine_zfp(stream, list(indices), list(locations), None, x.shape[0], ctx.experts,
+                                     ctx.capacity, M)
+            else:
+                dx = ops.combine_fwd(grad_y, list(indices), list(locations), None, x.shape[0], ctx.capacity)
+        dx, dw = _gate_backward(x, w, scores, indices, counts, ctx.normalize_gate, dx, grad_gates, grad_l_aux)
+        return dx, dw, None, None, None, None, None, None
+
+
+def gate_route_eligible(x, gate, experts, is_postscore):
+    """Gate, routing and encode as one call chain (planmoe_gate_route) for any compressor."""
+    from .gates import LinearTopKGate
+    vec = 4 if x.dtype == torch.float32 else 8
+    return (FUSE_GATE and is_postscore and type(gate) is LinearTopKGate and experts <= 64 and x.is_cuda and
+            x.dtype in (torch.float32, torch.bfloat16, torch.float16) and x.shape[-1] % vec == 0 and
+            x.shape[0] >= 1)
+
+
+def gate_route_encode(x, gate, top_k, capacity, normalize_gate, codec):
+    """-> (buffer [E * C, M], gates [k, T], l_aux, indices [k, T], locations [k, T])."""
+    w = gate.wg.weight
+    if w.dtype != x.dtype:
+        w = w.to(x.dtype)
+    return _GateRouteEncode.apply(x.contiguous(), w.contiguous(), top_k, w.shape[0], capacity,
+                                  bool(gate.fp32_gate), bool(normalize_gate), codec)
 
 
 def fused_gate_eligible(x, gate, experts, compress_name, degree, is_postscore):
@@ -274,6 +342,15 @@ def fused_zfp_forward(x, crit, expert_fn, degree=1):
     y = y.reshape(experts * capacity, -1).to(x.dtype)
     gates = [g.float() for g in gates_s]
     return _DecodeZfp.apply(y, indices, locations, experts, capacity, x.shape[0], *gates)
+
+
+def zfp_experts_decode(y, expert_fn, degree, indices, locations, gates, samples):
+    """The part of fused_zfp_forward after the encode: experts on the [E, C, M] buffer, then
+    compress + decompress + decode in one pass."""
+    experts, capacity, M = y.shape
+    y = _experts_in_chunks(expert_fn, y, degree)
+    y = y.reshape(experts * capacity, -1).to(torch.float32)
+    return _DecodeZfp.apply(y, indices, locations, experts, capacity, samples, *[g.float() for g in gates])
 
 
 def fused_int8_eligible(x, compress_name, degree, is_postscore):

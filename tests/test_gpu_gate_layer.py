@@ -393,6 +393,42 @@ def test_moe_layer_with_the_gate_in_the_fused_send_side(dtype):
     assert fused[2].abs().sum() > 0
 
 
+@pytest.mark.parametrize("compress,dtype", [("no", torch.bfloat16), ("no", torch.float32), ("lz", torch.float32),
+                                            ("zfp", torch.float32)])
+def test_moe_layer_with_gate_routing_and_encode_as_one_node(compress, dtype):
+    """The layer's default for the other compressors: gate GEMM + routing (planmoe_gate_route) and
+    the encode as one autograd node, so that the two gradients of x meet in one GEMM epilogue.
+    Against the staged pipeline (gate, routing and encode as separate nodes) to rounding: the
+    fused softmax sums in another order, and the staged x.grad is rounded once more."""
+    import planmoe_amd
+    from planmoe_amd import overlap
+
+    def run():
+        layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 1.25}, 128,
+                                      experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 64},
+                                      seeds=(1, 2, 3), compress_name=compress).to(DEV).to(dtype)
+        x = torch.randn(6, 50, 128, generator=torch.Generator().manual_seed(5)).to(dtype).to(DEV).requires_grad_(True)
+        y = layer(x)
+        (y.float().pow(2).mean() + y.l_aux.float()).backward()
+        return (y.detach(), x.grad.detach(), layer.gates[0].wg.weight.grad.detach(),
+                layer.experts.batched_fc1_w.grad.detach(), y.l_aux.detach())
+
+    assert overlap.FUSE_GATE
+    fused = run()
+    overlap.FUSE_GATE = False
+    try:
+        staged = run()
+    finally:
+        overlap.FUSE_GATE = True
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-4
+    for name, a, b in zip(("y", "dx", "dwg", "dfc1", "l_aux"), fused, staged):
+        a, b = a.float(), b.float()
+        assert a.shape == b.shape
+        err = (a - b).abs().max().item()
+        assert err <= tol * max(b.abs().max().item(), 1e-6), (name, err)
+    assert fused[1].abs().sum() > 0 and fused[2].abs().sum() > 0
+
+
 def test_moe_layer_prescore_noise_and_load_importance_loss():
     """The remaining layer options run end to end: gates applied at encode (is_postscore=False),
     gate noise with the load-importance loss, a data-dependent capacity (capacity_factor = 0)."""
