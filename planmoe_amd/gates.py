@@ -23,8 +23,8 @@ def weight_grad(g, x):
     main = (T // _SPLIT) * _SPLIT
     if main < 16 * _SPLIT:
         return g.t() @ x
-    gs = g[:main].view(_SPLIT, main // _SPLIT, -1).transpose(1, 2)
-    xs = x[:main].view(_SPLIT, main // _SPLIT, -1)
+    gs = g[:main].reshape(_SPLIT, main // _SPLIT, -1).transpose(1, 2)
+    xs = x[:main].reshape(_SPLIT, main // _SPLIT, -1)
     parts = None
     if x.dtype != torch.float32 and _bmm_fp32_out is not False:
         try:
