@@ -429,6 +429,22 @@ def test_moe_layer_with_gate_routing_and_encode_as_one_node(compress, dtype):
     assert fused[1].abs().sum() > 0 and fused[2].abs().sum() > 0
 
 
+@pytest.mark.parametrize("T,M,E,dtype", [(4099, 256, 16, torch.bfloat16), (16384, 512, 8, torch.float32),
+                                         (100, 64, 4, torch.float32), (1024, 128, 64, torch.float16)])
+def test_gate_weight_gradient_split_over_token_chunks(T, M, E, dtype):
+    """gates.weight_grad (a batched GEMM over token chunks + a sum) against the product in fp64:
+    ragged token counts, the short-input fall-back, a gradient that is a transposed view."""
+    from planmoe_amd import gates
+    g0 = torch.Generator().manual_seed(T)
+    x = torch.randn(T, M, generator=g0).to(dtype).to(DEV)
+    g = (torch.randn(E, T, generator=g0) * 0.01).to(dtype).to(DEV).t()          # [T, E], not contiguous
+    got = gates.weight_grad(g, x)
+    assert got.dtype == dtype and got.shape == (E, M)
+    ref = g.double().t() @ x.double()
+    tol = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float16: 2e-3}[dtype]
+    assert (got.double() - ref).abs().max().item() <= tol * ref.abs().max().item()
+
+
 def test_moe_layer_prescore_noise_and_load_importance_loss():
     """The remaining layer options run end to end: gates applied at encode (is_postscore=False),
     gate noise with the load-importance loss, a data-dependent capacity (capacity_factor = 0)."""
