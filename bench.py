@@ -62,7 +62,7 @@ def cpu_baseline(T_sample, M, E, k, cf, x_bits, wg_bits, min_seconds):
 
 
 def kernel_table(only=None):
-    """Every entry point at the full size of its workload (BASELINE configs 1-5): device time over
+    """Every entry point at the full size of its workload (the five benchmark configurations): device time over
     back-to-back launches (HIP events) against the algorithmic bytes = inputs read once + outputs
     written once.  One line per entry point; an entry point may be several launches."""
     import torch
