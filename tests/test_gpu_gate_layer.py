@@ -393,9 +393,10 @@ def test_moe_layer_with_the_gate_in_the_fused_send_side(dtype):
     assert fused[2].abs().sum() > 0
 
 
+@pytest.mark.parametrize("degree", [1, 2])
 @pytest.mark.parametrize("compress,dtype", [("no", torch.bfloat16), ("no", torch.float32), ("lz", torch.float32),
                                             ("zfp", torch.float32)])
-def test_moe_layer_with_gate_routing_and_encode_as_one_node(compress, dtype):
+def test_moe_layer_with_gate_routing_and_encode_as_one_node(compress, dtype, degree):
     """The layer's default for the other compressors: gate GEMM + routing (planmoe_gate_route) and
     the encode as one autograd node, so that the two gradients of x meet in one GEMM epilogue.
     Against the staged pipeline (gate, routing and encode as separate nodes) to rounding: the
@@ -406,7 +407,8 @@ def test_moe_layer_with_gate_routing_and_encode_as_one_node(compress, dtype):
     def run():
         layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 1.25}, 128,
                                       experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 64},
-                                      seeds=(1, 2, 3), compress_name=compress).to(DEV).to(dtype)
+                                      seeds=(1, 2, 3), compress_name=compress,
+                                      a2a_ffn_overlap_degree=degree).to(DEV).to(dtype)
         x = torch.randn(6, 50, 128, generator=torch.Generator().manual_seed(5)).to(dtype).to(DEV).requires_grad_(True)
         y = layer(x)
         (y.float().pow(2).mean() + y.l_aux.float()).backward()
