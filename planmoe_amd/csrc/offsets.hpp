@@ -117,21 +117,21 @@ static __global__ __launch_bounds__(256) void group_offsets_kernel(
             }
         }
         __syncthreads();
-        if (threadIdx.x < experts_per_block) {
+        if ((int)threadIdx.x < experts_per_block) {
             int32_t add = 0;
             for (int p = 0; p < planes_per_chunk; ++p) add += s_tot[p * experts_per_block + threadIdx.x];
             s_base[threadIdx.x] += add;
         }
     }
     __syncthreads();
-    if (totals && threadIdx.x < ne) totals[e0 + threadIdx.x] = s_base[threadIdx.x];
+    if (totals && (int)threadIdx.x < ne) totals[e0 + threadIdx.x] = s_base[threadIdx.x];
 
     if (want_loss) {
         s_me[rl][cl] = mes;
         __syncthreads();
         if (threadIdx.x < WAVE) {
             float acc = 0.f;
-            if (threadIdx.x < ne) {
+            if ((int)threadIdx.x < ne) {
                 float m = 0.f;
 #pragma unroll
                 for (int r = 0; r < GO_ROWS; ++r) m += s_me[r][threadIdx.x];
