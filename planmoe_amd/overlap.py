@@ -56,6 +56,12 @@ def a2a_ffn_overlap_forward(input, expert_fn, a2a_ffn_overlap_degree, use_2dh, g
     assert input.shape[split_dim] % a2a_ffn_overlap_degree == 0, \
         "Excepting input.shape[%d] (%d) be multiple of a2a_ffn_overlap_degree (%d)." % (
             split_dim, input.shape[split_dim], a2a_ffn_overlap_degree)
+    if compress_name not in ("int8", "zfp", "lz") and not _ck.SINGLE_RANK_COMM_COPIES:
+        # NoCompressor on one rank: compress, comm and decompress all return their argument
+        # (no.cpp:3-20, the comm hand-over), so the six autograd nodes around the experts are pure
+        # host work; only the experts' slicing remains
+        _ck.clear_ptr_lst()
+        return _experts_in_chunks(expert_fn, input, a2a_ffn_overlap_degree).contiguous()
     split_size = input.shape[split_dim] // a2a_ffn_overlap_degree
     # (one slice: the tensor itself -- the backward of a split is a cat, i.e. a copy of the whole gradient)
     input_split = [input] if a2a_ffn_overlap_degree == 1 else list(input.split(split_size, dim=split_dim))
