@@ -345,9 +345,11 @@ _forward_ws = {}
 
 
 def _forward_workspace(T, E, k, device):
-    """Per-device workspace of the fused chain, grown on demand."""
+    """Workspace of the fused chain, grown on demand: one per device and stream (calls on one
+    stream follow each other; calls on two streams must not share it)."""
     need = lib.planmoe_forward_workspace_bytes(T, E, k)
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
     ws = _forward_ws.get(key)
     if ws is None or ws.numel() < need:
         ws = torch.empty((max(need, 1 << 20),), dtype=torch.uint8, device=device)
