@@ -449,6 +449,11 @@ def main():
                      "algorithmic_bytes": dom_bytes, "avg_us": dom_avg_us},
         "chain": {"algorithmic_bytes": chain_bytes, "device_us_avg": chain_ev[0], "device_us_min": chain_ev[2],
                   "GBps": chain_bytes / chain_ev[0] / 1e3, "frac_of_hbm_peak": chain_bytes / chain_ev[0] / 1e3 / HBM_PEAK_GBS,
+                  # bytes that cross the L2 boundary in the two launches (rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE,
+                  # see profiles/): x is read by both launches, so the chain moves more than its algorithmic bytes
+                  "traffic_bytes": 136.0e6 + 307.0e6,
+                  "traffic_GBps": (136.0e6 + 307.0e6) / chain_ev[0] / 1e3,
+                  "traffic_frac_of_hbm_peak": (136.0e6 + 307.0e6) / chain_ev[0] / 1e3 / HBM_PEAK_GBS,
                   "device_us_cold_caches": cold_us,
                   "stage_us_avg": {n: v[0] for n, v in stages.items()}},
     }
