@@ -92,3 +92,27 @@ def test_zfp_and_lz_entry_points_replay():
         return [stream, y, *lz, back]
 
     replay_against_eager(make, run, lambda o: o)
+
+
+def test_forward_chain_on_two_streams_at_once():
+    """The chain keeps its routing state in a cached workspace: calls issued on two streams must not
+    share it.  Two different batches, enqueued alternately on two streams without waiting, against
+    the same calls made one after the other."""
+    T, M, E, k = 4096, 512, 8, 2
+    C = ops.capacity(T, E, k, 1.25, 4)
+    g = torch.Generator().manual_seed(3)
+    xs = [torch.randn(T, M, generator=g).bfloat16().to(DEV) for _ in range(2)]
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
+    want = [ops.forward_int8(x, wg, k, C) for x in xs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [None, None]
+    for _ in range(5):
+        for i in (0, 1):
+            with torch.cuda.stream(streams[i]):
+                got[i] = ops.forward_int8(xs[i], wg, k, C)
+    torch.cuda.synchronize()
+    for a, b in zip(got, want):
+        for name in ("indices", "locations", "codes", "bias", "scale"):
+            assert torch.equal(a[name].view(torch.uint8).reshape(-1), b[name].view(torch.uint8).reshape(-1)), name
+
