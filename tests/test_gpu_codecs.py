@@ -237,6 +237,37 @@ def test_zfp_config5_full_size(dims):
     assert (dec2 - dec).abs().max().item() <= err
 
 
+def test_zfp_field_beyond_two_to_the_31_values():
+    """A [8, 75000, 4096] fp32 buffer (2.46 G values, 9.8 GB; stream 2.46 GB): block and row addresses
+    need 64 bits.  Blocks are coded independently, so the stream of the last 8 rows must be the
+    stream of those rows coded alone, and the fused entry points must equal their two stages."""
+    from planmoe_amd import ops
+    T, M, E, k = 600000, 4096, 8, 1
+    C = ops.capacity(T, E, k, 1.0, 4)
+    R = E * C
+    g = torch.Generator(device=DEV).manual_seed(2)
+    x = torch.randn(T, M, generator=g, device=DEV, dtype=torch.float32)
+    r = ops.route_topk(torch.softmax(torch.randn(T, E, generator=g, device=DEV), 1), k)
+    idx, loc, gates = list(r["indices"]), list(r["locations"]), [t.float() for t in r["gates"]]
+    d = ops.dispatch_fwd(x, idx, loc, None, E, C)
+    assert d.numel() > 2 ** 31
+    st = ops.zfp_compress(d, M, R, 2)
+    n = ops.zfp_stream_bytes(2, M, R)
+    tail = ops.zfp_compress(d[R - 8:].contiguous(), M, 8, 2)
+    nt = ops.zfp_stream_bytes(2, M, 8)
+    assert torch.equal(st[n - nt:n], tail[:nt])
+    fused = ops.dispatch_zfp(x, idx, loc, None, E, C)
+    assert torch.equal(fused[:n], st[:n])
+    del fused
+    dec = ops.zfp_decompress(st, M, R, 2)
+    assert torch.equal(dec[R - 8:], ops.zfp_decompress(tail, M, 8, 2))
+    del d
+    y = ops.combine_fwd(dec, idx, loc, gates, T, C)
+    del dec
+    y2 = ops.combine_zfp(st, idx, loc, gates, T, E, C, M)
+    assert torch.equal(y.view(torch.int32), y2.view(torch.int32))
+
+
 @pytest.mark.parametrize("copies", [False, True])
 def test_compressor_registry_round_trips(copies):
     """compress_operation / comm_operation / decompress_operation with 'no', 'int8', 'zfp', 'lz';

@@ -157,6 +157,46 @@ def test_config2_full_size_bf16_against_oracle():
     assert np.array_equal(raw(y), raw(wy))
 
 
+def test_buffers_beyond_two_to_the_31_elements():
+    """600 000 tokens x 4096 bf16 (2.46 G elements, 4.9 GB per buffer): row addresses need 64 bits in
+    every kernel of the path.  Checked through what holds at any size: dispatch then combine gives
+    every kept token row back and zero rows for the dropped ones; the fused int8 kernels equal their
+    two stages; the forward chain equals routing + the fused dispatch."""
+    from planmoe_amd import ops
+    T, M, E, k = 600000, 4096, 8, 1
+    C = ops.capacity(T, E, k, 1.0, 4)
+    g = torch.Generator(device=DEV).manual_seed(1)
+    x = torch.randn(T, M, generator=g, device=DEV, dtype=torch.float32).bfloat16()
+    wg = (torch.randn(E, M, generator=g, device=DEV) * M ** -0.5).bfloat16()
+    r = ops.gate_route(x, wg, k)
+    idx, loc = list(r["indices"]), list(r["locations"])
+    kept = (loc[0] >= 0) & (loc[0] < C)
+    assert 0 < int(kept.sum()) < T                                   # some tokens are dropped
+    d = ops.dispatch_fwd(x, idx, loc, None, E, C)
+    assert d.numel() > 2 ** 31
+    slot = idx[0].long() * C + loc[0].long()
+    last = int(torch.nonzero(kept)[-1])
+    assert torch.equal(d[slot[last]], x[last])                       # the highest token row, the slot it went to
+    y = ops.combine_fwd(d, idx, loc, None, T, C)
+    assert torch.equal(y[kept].view(torch.int16), (x[kept] + 0.0).view(torch.int16))
+    assert not y[~kept].any()
+    del y
+    codes, bias, scale = ops.dispatch_int8(x, idx, loc, None, E, C)
+    c2, b2, s2 = ops.int8_compress(d)
+    assert torch.equal(codes.view(-1), c2.view(-1))
+    assert torch.equal(bias.view(torch.int16).view(-1), b2.view(torch.int16).view(-1))
+    assert torch.equal(scale.view(torch.int16).view(-1), s2.view(torch.int16).view(-1))
+    del c2, b2, s2
+    dec = ops.int8_decompress(codes, bias, scale)
+    y8 = ops.combine_int8(codes, bias, scale, idx, loc, list(r["gates"]), T, C)
+    y2 = ops.combine_fwd(dec, idx, loc, list(r["gates"]), T, C)
+    assert torch.equal(y8.view(torch.int16), y2.view(torch.int16))
+    del dec, y8, y2, d
+    f = ops.forward_int8(x, wg, k, C)
+    assert torch.equal(f["indices"], r["indices"]) and torch.equal(f["locations"], r["locations"])
+    assert torch.equal(f["codes"].view(-1), codes.view(-1))
+
+
 def test_autograd_wiring_matches_the_reference_functions():
     """fast_encode / fast_decode backward: which gradients exist and what they equal."""
     import planmoe_amd
