@@ -191,7 +191,19 @@ def test_buffers_beyond_two_to_the_31_elements():
     y8 = ops.combine_int8(codes, bias, scale, idx, loc, list(r["gates"]), T, C)
     y2 = ops.combine_fwd(dec, idx, loc, list(r["gates"]), T, C)
     assert torch.equal(y8.view(torch.int16), y2.view(torch.int16))
-    del dec, y8, y2, d
+    del dec, y8, y2
+    # backward pieces: bwd_gate on sampled tokens against a dot product, the fused backward of
+    # fast_decode against its stages (gated dispatch + int8, bwd_gate)
+    gates = [t.float() for t in r["gates"]]
+    gg = ops.bwd_gate(x, d, idx, loc, C)
+    sample = torch.tensor([0, 1, T // 2, last, T - 1], device=DEV)
+    want = (x[sample].float() * d[slot[sample].clamp(0, E * C - 1)].float()).sum(1) * kept[sample]
+    assert torch.allclose(gg[0][sample], want, rtol=1e-2, atol=1e-2)
+    c5, b5, s5, g5 = ops.combine_bwd_int8(x, d, idx, loc, gates, E, C)
+    c6, b6, s6 = ops.dispatch_int8(x, idx, loc, gates, E, C)
+    assert torch.equal(c5.view(-1), c6.view(-1)) and torch.equal(b5.view(torch.int16).view(-1), b6.view(torch.int16).view(-1))
+    assert torch.allclose(g5[0], gg[0], rtol=1e-5, atol=1e-4)
+    del c5, b5, s5, g5, c6, b6, s6, d
     f = ops.forward_int8(x, wg, k, C)
     assert torch.equal(f["indices"], r["indices"]) and torch.equal(f["locations"], r["locations"])
     assert torch.equal(f["codes"].view(-1), codes.view(-1))
