@@ -46,6 +46,19 @@ def test_against_oracle(T, E, k):
     _check(tie_free_scores(T, E, k, seed=T + E), k)
 
 
+@pytest.mark.parametrize("T,E,k", [(600000, 8, 2), (400000, 128, 2), (300001, 64, 1)])
+def test_many_tokens(T, E, k):
+    """Token counts an order of magnitude above the configs (thousands of routing tiles / groups)."""
+    _check(tie_free_scores(T, E, k, seed=T + E), k)
+
+
+def test_cumsum_many_rows():
+    from planmoe_amd import ops
+    mask = (torch.rand(600001, 64, generator=torch.Generator().manual_seed(9)) < 0.2).to(torch.int32).to(DEV)
+    got = ops.cumsum_sub_one(mask)
+    assert torch.equal(got, torch.cumsum(mask, 0, dtype=torch.int32) - 1)
+
+
 def test_without_gate_normalisation():
     _check(tie_free_scores(700, 8, 2, seed=3), 2, normalize=False)
 
