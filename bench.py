@@ -192,6 +192,8 @@ def kernel_table(only=None):
     add("combine_zfp (fused)", "5", E5 * C5 * M5 + T5 * M5 * 4,
         lambda: ops.combine_zfp(zs, i5, l5, g5, T5, E5, C5, M5), iters=5)
     add("dispatch_zfp (fused)", "5", T5 * M5 * 4 + E5 * C5 * M5, lambda: ops.dispatch_zfp(x5, i5, l5, None, E5, C5, out=zs), iters=5)
+    add("bwd_gate", "5", 3 * T5 * M5 * 4, lambda: ops.bwd_gate(x5, d5, i5, l5, C5), iters=5)
+    add("bwd_gate_zfp (fused)", "5", E5 * C5 * M5 + T5 * M5 * 4, lambda: ops.bwd_gate_zfp(zs, x5, i5, l5, E5, C5), iters=5)
 
     # the same buffer through the lossless codec: as it is (no symbol repeats, nothing shrinks) and
     # with 30 % of the capacity slots empty (zero rows shrink to 44 bytes per 2048)

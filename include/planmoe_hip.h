@@ -306,6 +306,18 @@ int planmoe_combine_zfp(const void *stream_in, double rate, const float *gates, 
                         int model_dim, int experts, int capacity, float *out, void *workspace,
                         size_t workspace_bytes, void *stream);
 
+/* The gate gradients of GatingDecoder.backward (create_backward_gate, fast_dispatch.py:73-78)
+ * straight from the stream of the expert output that the decode consumed (what
+ * ZfpCompressor::decompress would have produced, zfpc.cpp:66-86):
+ * grad_gates[j][t] = <grad_out[t], decoded slot row of choice j>, 0 for a choice without a slot;
+ * what planmoe_zfp_decompress + planmoe_bwd_gate give to rounding (the sum runs in another
+ * order), without the decoded buffer.  fp32, 2-D stream with nx = model_dim, ny = experts *
+ * capacity; workspace as for planmoe_combine_zfp.  4 launches. */
+int planmoe_bwd_gate_zfp(const void *stream_in, double rate, const float *grad_out, const int32_t *indices,
+                         const int32_t *locations, int64_t plane_stride, int top_k, int samples,
+                         int model_dim, int experts, int capacity, float *grad_gates, void *workspace,
+                         size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------- GPULZ ("lz") lossless codec
  * Replaces lz_compress / lz_decompress (custom/compressor/gpulz.cu:408-535), the codec behind
  * LzCompressor (custom/compressor/lz.cpp:3-60).  The input is taken as 32-bit symbols in blocks

@@ -576,6 +576,62 @@ __global__ __launch_bounds__(256) void combine_zfp2_kernel(const uint32_t *__res
     }
 }
 
+// GatingDecoder.backward's gate gradients (create_backward_gate, fast_dispatch.py:73-78) straight
+// from the stream of the expert output the decode consumed: grad_gate[plane][t] = <grad_out[t],
+// decoded slot row>, so the backward pass never writes the decoded buffer.  One work-group owns
+// the four slot rows of one row of blocks; a thread decodes its blocks along the row and keeps four
+// partial sums, which the work-group adds in a fixed order.  grad_gates must be zero beforehand
+// (choices that take no slot keep their zero).
+template <int NW>
+__global__ __launch_bounds__(256) void bwd_gate_zfp2_kernel(const uint32_t *__restrict__ in,
+                                                           const int32_t *__restrict__ src,
+                                                           const int32_t *__restrict__ splane,
+                                                           const float *__restrict__ grad_out, int64_t stride,
+                                                           int64_t model_dim, int64_t nbx,
+                                                           float *__restrict__ grad_gates)
+{
+    __shared__ uint32_t lds[NW <= 2 ? 1 : (NW + 1) * 256];
+    __shared__ float s_part[4][4];
+    const int64_t by = blockIdx.x;
+    const int4 tok = *reinterpret_cast<const int4 *>(src + 4 * by);
+    const int t[4] = {tok.x, tok.y, tok.z, tok.w};
+    if (t[0] < 0 && t[1] < 0 && t[2] < 0 && t[3] < 0) return;        // four empty slots (the whole work-group leaves)
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t bx0 = 0; bx0 < nbx; bx0 += 256) {
+        const int64_t bx = bx0 + threadIdx.x;
+        const bool in_row = bx < nbx;
+        const int64_t bxc = in_row ? bx : nbx - 1;                   // clamped: straight-line loads
+        float4 g[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            g[j] = *reinterpret_cast<const float4 *>(grad_out + (int64_t)max(t[j], 0) * model_dim + 4 * bxc);
+        uint32_t w[NW];
+        load_words<NW>(in + (by * nbx + bxc) * NW, w);
+        BitReader<NW> br;
+        br.init(lds, w);
+        float f[16];
+        decode_block<16, NW>(br, f);
+        if (in_row) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[j] += ((f[4 * j] * g[j].x + f[4 * j + 1] * g[j].y) + f[4 * j + 2] * g[j].z) + f[4 * j + 3] * g[j].w;
+        }
+    }
+    const int wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float r = wave_sum(acc[j]);
+        if (lane_id() == 0) s_part[wave][j] = r;
+    }
+    __syncthreads();
+    if (threadIdx.x < 4) {
+        const int j = threadIdx.x;
+        if (t[j] >= 0)
+            grad_gates[(int64_t)splane[4 * by + j] * stride + t[j]] =
+                ((s_part[0][j] + s_part[1][j]) + s_part[2][j]) + s_part[3][j];
+    }
+}
+
 // tokens whose choice `plane` takes no slot: a zero row (plane 0) or row + 0 (later planes)
 __global__ __launch_bounds__(256) void combine_dropped_kernel(const int32_t *__restrict__ indices,
                                                              const int32_t *__restrict__ locations,
@@ -790,6 +846,49 @@ extern "C" int planmoe_combine_zfp(const void *stream_in, double rate, const flo
         combine_dropped_kernel<<<(unsigned)((samples + 3) / 4), 256, 0, st>>>(indices, locations, plane_stride, j,
                                                                             samples, model_dim, experts, capacity, out);
     }
+    PM_LAUNCH_CHECK(who);
+    return 0;
+}
+
+extern "C" int planmoe_bwd_gate_zfp(const void *stream_in, double rate, const float *grad_out,
+                                    const int32_t *indices, const int32_t *locations, int64_t plane_stride,
+                                    int top_k, int samples, int model_dim, int experts, int capacity,
+                                    float *grad_gates, void *workspace, size_t workspace_bytes, void *stream)
+{
+    const char *who = "planmoe_bwd_gate_zfp";
+    PM_REQUIRE((indices && locations) || samples == 0, "%s: indices/locations must not be NULL", who);
+    PM_REQUIRE(top_k >= 1 && samples >= 0 && plane_stride >= samples, "%s: bad routing planes", who);
+    PM_REQUIRE(model_dim >= 1 && experts >= 1 && capacity >= 0, "%s: bad shape", who);
+    PM_REQUIRE((int64_t)experts * capacity < (1ll << 31) && (int64_t)samples * top_k < (1ll << 31),
+               "%s: experts*capacity or samples*top_k overflows int32", who);
+    const int64_t rows = (int64_t)experts * capacity;
+    int nw; int64_t blocks;
+    if (zfp_check(who, 2, model_dim, rows, rate, nw, blocks)) return 1;
+    if (samples == 0) return 0;
+    PM_REQUIRE(grad_gates, "%s: grad_gates is NULL", who);
+    hipStream_t st = (hipStream_t)stream;
+    // every plane row in full: plane_stride may exceed samples, the padding is the caller's
+    for (int j = 0; j < top_k; ++j)
+        fill_u32((uint32_t *)(grad_gates + (int64_t)j * plane_stride), (size_t)samples, 0u, st);
+    if (blocks == 0) {                                  // no slot at all: every gradient is zero
+        PM_LAUNCH_CHECK(who);
+        return 0;
+    }
+    PM_REQUIRE(stream_in && aligned16(stream_in), "%s: the stream must be a 16-byte aligned buffer", who);
+    PM_REQUIRE(grad_out && aligned16(grad_out), "%s: grad_out must be a 16-byte aligned buffer", who);
+    PM_REQUIRE(workspace && aligned16(workspace) &&
+               workspace_bytes >= planmoe_combine_zfp_workspace_bytes(experts, capacity),
+               "%s: workspace too small or not 16-byte aligned", who);
+    int32_t *src = (int32_t *)workspace;
+    float *sgate = (float *)(src + rows);
+    int32_t *splane = (int32_t *)(sgate + rows);
+    fill_u32((uint32_t *)src, (size_t)rows, 0xffffffffu, st);
+    slot_source_mark<<<(unsigned)(((int64_t)samples * top_k + 255) / 256), 256, 0, st>>>(
+        src, sgate, splane, nullptr, indices, locations, plane_stride, top_k, samples, experts, capacity);
+    PM_NW_SWITCH(nw, NW, {
+        bwd_gate_zfp2_kernel<NW><<<(unsigned)(rows / 4), 256, 0, st>>>((const uint32_t *)stream_in, src, splane, grad_out,
+                                                                     plane_stride, model_dim, model_dim / 4, grad_gates);
+    });
     PM_LAUNCH_CHECK(who);
     return 0;
 }

@@ -508,6 +508,24 @@ def combine_zfp(stream, indices, locations, gates, samples, experts, capacity_, 
     return out
 
 
+def bwd_gate_zfp(stream, grad_out, indices, locations, experts, capacity_, rate=8.0):
+    """grad_gates[k, T] (fp32) = <grad_out[t], decoded slot row> with the slot rows taken straight
+    from the 2-D stream (nx = model_dim, ny = experts * capacity) of the tensor fast_decode consumed."""
+    _need_gpu(stream, "bwd_gate_zfp")
+    stream = _contig(stream, "bwd_gate_zfp")
+    grad_out = _contig(grad_out, "bwd_gate_zfp")
+    if grad_out.dtype != torch.float32:
+        raise PlanMoEError("bwd_gate_zfp: grad_out must be float32 (the zfp codec reads its field as fp32)")
+    T, M = grad_out.shape
+    idx, loc, _, stride = _plane_args(indices, locations, None, "bwd_gate_zfp")
+    k = len(indices)
+    out = torch.empty((k, stride), dtype=torch.float32, device=grad_out.device)
+    ws = _ws(lib.planmoe_combine_zfp_workspace_bytes(experts, capacity_), grad_out.device)
+    check(lib.planmoe_bwd_gate_zfp(_ptr(stream), float(rate), _ptr(grad_out), _ptr(idx), _ptr(loc), stride, k, T, M,
+                                   experts, capacity_, _ptr(out), _ptr(ws), ws.numel(), _stream(grad_out)))
+    return out[:, :T]
+
+
 # ------------------------------------------------------------------------------ GPULZ ("lz") codec
 LZ_BLOCK_BYTES = 2048
 

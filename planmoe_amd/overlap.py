@@ -320,10 +320,14 @@ class _DecodeZfp(torch.autograd.Function):
         stream, indices, locations, *gates = ctx.saved_tensors
         R, M = ctx.shape
         grad_out = grad_out.contiguous()
-        seen = ops.zfp_decompress(stream, M, R, 2)              # the tensor fast_decode consumed
         gstream = ops.dispatch_zfp(grad_out, list(indices), list(locations), list(gates), ctx.experts, ctx.capacity)
         grad_y = ops.zfp_decompress(gstream, M, R, 2)
-        gg = ops.bwd_gate(grad_out, seen, list(indices), list(locations), ctx.capacity)
+        if FUSE_ZFP:
+            # the gate gradients straight from the stream of the tensor fast_decode consumed
+            gg = ops.bwd_gate_zfp(stream, grad_out, list(indices), list(locations), ctx.experts, ctx.capacity)
+        else:
+            seen = ops.zfp_decompress(stream, M, R, 2)
+            gg = ops.bwd_gate(grad_out, seen, list(indices), list(locations), ctx.capacity)
         return (grad_y, None, None, None, None, None, *[gg[j].to(g.dtype) for j, g in enumerate(gates)])
 
 

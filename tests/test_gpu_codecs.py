@@ -237,6 +237,35 @@ def test_zfp_config5_full_size(dims):
     assert (dec2 - dec).abs().max().item() <= err
 
 
+@pytest.mark.parametrize("T,M,E,k,cf", [(1000, 256, 8, 2, 1.25), (333, 1024, 16, 2, 0.5), (64, 4, 4, 4, 1.0),
+                                        (5000, 132, 12, 1, 1.0), (7, 64, 4, 2, 4.0), (300, 2048, 4, 3, 1.0)])
+def test_bwd_gate_zfp_equals_decompress_then_bwd_gate(T, M, E, k, cf):
+    """planmoe_bwd_gate_zfp: the gate gradients from the stream of the expert output, against
+    planmoe_zfp_decompress + planmoe_bwd_gate (another summation order: rtol 1e-5 on the sum of
+    the terms' magnitudes) and against a dot product in fp64; exact zeros for dropped choices."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(T * 3 + M)
+    r = ops.route_topk(torch.softmax(torch.randn(T, E, generator=g), 1).to(DEV), k)
+    C = ops.capacity(T, E, k, cf, 4)
+    idx, loc = list(r["indices"]), list(r["locations"])
+    y = torch.randn(E * C, M, generator=g).to(DEV)                   # expert outputs
+    dout = torch.randn(T, M, generator=g).to(DEV)
+    st = ops.zfp_compress(y, M, E * C, 2)
+    seen = ops.zfp_decompress(st, M, E * C, 2)
+    want = ops.bwd_gate(dout, seen, idx, loc, C)
+    got = ops.bwd_gate_zfp(st, dout, idx, loc, E, C)
+    assert got.shape == want.shape
+    for j in range(k):
+        kept = (loc[j] >= 0) & (loc[j] < C)
+        slot = (idx[j].long() * C + loc[j].long()).clamp(0, max(E * C - 1, 0))
+        rows = seen[slot] if E * C > 0 else torch.zeros_like(dout)
+        ref = (dout.double() * rows.double()).sum(1) * kept
+        mag = (dout.double() * rows.double()).abs().sum(1) * kept
+        assert ((got[j].double() - ref).abs() <= 1e-5 * mag + 1e-30).all()
+        assert ((got[j].double() - want[j].double()).abs() <= 2e-5 * mag + 1e-30).all()
+        assert (got[j][~kept] == 0).all()
+
+
 def test_zfp_field_beyond_two_to_the_31_values():
     """A [8, 75000, 4096] fp32 buffer (2.46 G values, 9.8 GB; stream 2.46 GB): block and row addresses
     need 64 bits.  Blocks are coded independently, so the stream of the last 8 rows must be the

@@ -312,7 +312,9 @@ def test_moe_layer_fused_int8_path_equals_the_stepwise_pipeline(dtype):
 
 def test_moe_layer_fused_zfp_send_side_equals_the_stepwise_pipeline():
     """compress_name='zfp' (fp32): fast_encode + compress as planmoe_dispatch_zfp in forward and in
-    the backward of fast_decode -- outputs and every gradient bit for bit against the steps."""
+    the backward of fast_decode -- the output and the gradients that do not pass through the gate
+    bit for bit against the steps; the gate gradients come from planmoe_bwd_gate_zfp, which sums in
+    another order, so x.grad and the gate weight's gradient agree to rounding."""
     import planmoe_amd
     from planmoe_amd import overlap
     results = []
@@ -329,9 +331,19 @@ def test_moe_layer_fused_zfp_send_side_equals_the_stepwise_pipeline():
                             layer.experts.batched_fc1_w.grad.detach()))
         finally:
             overlap.FUSE_ZFP = True
-    for a, b in zip(*results):
-        assert torch.equal(a, b)
+    _same_but_for_the_gate_gradients(*results)
     assert results[0][1].abs().sum() > 0 and results[0][2].abs().sum() > 0
+
+
+def _same_but_for_the_gate_gradients(fused, staged, exact_gate=False):
+    """(y, x.grad, gate weight grad, fc1 grad): y and the expert gradient bit for bit; the two that
+    pass through the gate gradients bit for bit (exact_gate) or to fp32 rounding."""
+    assert torch.equal(fused[0], staged[0]) and torch.equal(fused[3], staged[3])
+    for a, b in ((fused[1], staged[1]), (fused[2], staged[2])):
+        if exact_gate:
+            assert torch.equal(a, b)
+        else:
+            assert (a.float() - b.float()).abs().max().item() <= 1e-4 * max(b.float().abs().max().item(), 1e-6)
 
 
 @pytest.mark.parametrize("compress,dtype", [("int8", torch.bfloat16), ("int8", torch.float32), ("zfp", torch.float32)])
@@ -355,8 +367,7 @@ def test_fused_paths_with_two_chunks_equal_the_stepwise_pipeline(compress, dtype
                             layer.experts.batched_fc1_w.grad.detach()))
         finally:
             overlap.FUSE_INT8 = overlap.FUSE_ZFP = overlap.FUSE_GATE = True
-    for a, b in zip(*results):
-        assert torch.equal(a, b)
+    _same_but_for_the_gate_gradients(*results, exact_gate=(compress != "zfp"))
 
 
 def _layer_pass(planmoe_amd, dtype):

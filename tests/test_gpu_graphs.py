@@ -86,10 +86,11 @@ def test_zfp_and_lz_entry_points_replay():
     def run(inp):
         stream = ops.dispatch_zfp(inp[0], idx, loc, None, E, C)
         y = ops.combine_zfp(stream, idx, loc, gates, T, E, C, M)
+        gg = ops.bwd_gate_zfp(stream, inp[0], idx, loc, E, C)
         lz = ops.lz_compress(inp[0])
         back = torch.empty_like(inp[0])
         ops.lz_decompress(back, *lz)
-        return [stream, y, *lz, back]
+        return [stream, y, gg.contiguous(), *lz, back]
 
     replay_against_eager(make, run, lambda o: o)
 
