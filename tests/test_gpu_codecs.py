@@ -266,6 +266,21 @@ def test_bwd_gate_zfp_equals_decompress_then_bwd_gate(T, M, E, k, cf):
         assert (got[j][~kept] == 0).all()
 
 
+def test_bwd_gate_zfp_without_slots_or_tokens():
+    from planmoe_amd import ops
+    T, M, E, k = 63, 64, 33, 2                                       # capacity_factor 0.25 leaves no slot
+    C = ops.capacity(T, E, k, 0.25, 4)
+    assert C == 0
+    r = ops.route_topk(torch.softmax(torch.randn(T, E, generator=torch.Generator().manual_seed(0)), 1).to(DEV), k)
+    empty = torch.empty((0,), dtype=torch.uint8, device=DEV)
+    gg = ops.bwd_gate_zfp(empty, torch.randn(T, M, device=DEV), list(r["indices"]), list(r["locations"]), E, C)
+    assert gg.shape == (k, T) and not gg.any()
+    none = ops.bwd_gate_zfp(torch.zeros((4 * 64,), dtype=torch.uint8, device=DEV), torch.empty((0, M), device=DEV),
+                            [torch.empty((0,), dtype=torch.int32, device=DEV)],
+                            [torch.empty((0,), dtype=torch.int32, device=DEV)], 1, 4)
+    assert none.shape == (1, 0)
+
+
 def test_zfp_field_beyond_two_to_the_31_values():
     """A [8, 75000, 4096] fp32 buffer (2.46 G values, 9.8 GB; stream 2.46 GB): block and row addresses
     need 64 bits.  Blocks are coded independently, so the stream of the last 8 rows must be the
