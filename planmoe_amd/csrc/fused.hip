@@ -30,6 +30,7 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
     constexpr int V = E::VEC;
     const int wave = threadIdx.x >> 6, lane = lane_id();
     const int units = model_dim / V;
+    __shared__ float s_dtab[CODED ? 4 : 1][CODED ? 256 : 1];         // [wave][code]: decoded values of one row
 
     if ((int)blockIdx.x >= token_blocks) {
         // slots no live pair addresses: all-zero row -> codes 0, bias 0, scale 0
@@ -70,12 +71,27 @@ __global__ __launch_bounds__(256) void dispatch_int8_kernel(
             // V codes per unit: one or two 32-bit words
             using cword_t = typename std::conditional<V == 8, uint2, uint32_t>::type;
             const cword_t *crow = reinterpret_cast<const cword_t *>((const uint8_t *)other + (int64_t)s * model_dim);
-            const RowDecoder<DT> dec(E::load(other_bias, s), E::load(other_scale, s));
+            // the 256 values a code of this row can stand for, worked out once (4 per lane, the
+            // decompressor's arithmetic) and looked up per element; the table is the wave's own
+            const RowDequant<DT> dq(E::load(other_bias, s), E::load(other_scale, s));
+            float *tab = s_dtab[wave];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int q = 0; q < 4; ++q) tab[q * WAVE + lane] = dq((uint32_t)(q * WAVE + lane));
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             auto visit = [&](const uint4 &a, const cword_t &cw) {
                 float fa[V], fb[V];
                 E::unpack(a, fa);
-                if constexpr (V == 8) { dec.word(cw.x, fb); dec.word(cw.y, fb + 4); }
-                else dec.word(cw, fb);
+                if constexpr (V == 8) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { fb[i] = tab[(cw.x >> (8 * i)) & 0xffu]; fb[4 + i] = tab[(cw.y >> (8 * i)) & 0xffu]; }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) fb[i] = tab[(cw >> (8 * i)) & 0xffu];
+                }
 #pragma unroll
                 for (int i = 0; i < V; ++i) acc = fmaf(fb[i], fa[i], acc);
             };
@@ -251,6 +267,7 @@ __global__ __launch_bounds__(256) void combine_int8_kernel(
         if constexpr (V == 8) { const uint2 c = reinterpret_cast<const uint2 *>(row)[u]; w[0] = c.x; w[1] = c.y; }
         else { w[0] = reinterpret_cast<const uint32_t *>(row)[u]; w[1] = 0; }
     };
+    __shared__ float s_tab[4][4][256];                               // [wave][plane][code]
     if (top_k <= 4) {
         // the usual case: all planes of four units are requested before any is decoded
         constexpr int UB = 4;
@@ -258,6 +275,20 @@ __global__ __launch_bounds__(256) void combine_int8_kernel(
         fetch_planes(gates, indices, locations, stride, t, 0, top_k, 0x7fffffff, capacity, slot, gate);
         float b_l = 0.f, s_l = 0.f;
         if (lane < top_k && slot >= 0) { b_l = E::load(bias_in, slot); s_l = E::load(scale_in, slot); }
+        // A row has 256 possible values: gate * decoded(code), worked out once per row (4 entries per
+        // lane and plane, the same arithmetic as the decoder) and looked up per element.
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (j < top_k && rl_i(slot, j) >= 0) {
+                const RowDequant<DT> dq(rl_f(b_l, j), rl_f(s_l, j));
+                const float g = rl_f(gate, j);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) s_tab[wave][j][q * WAVE + lane] = g * dq((uint32_t)(q * WAVE + lane));
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");       // the wave's own table: no work-group barrier
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         for (int u0 = 0; u0 < units; u0 += UB * WAVE) {
             uint32_t cw[4][UB][2];
 #pragma unroll
@@ -280,14 +311,11 @@ __global__ __launch_bounds__(256) void combine_int8_kernel(
                 for (int j = 0; j < 4; ++j) {
                     if (j < top_k) {
                         const int s = rl_i(slot, j);
-                        const float g = rl_f(gate, j);
                         float term[V];
                         if (s >= 0) {
-                            const RowDecoder<DT> dec(rl_f(b_l, j), rl_f(s_l, j));
+                            const float *tab = s_tab[wave][j];
 #pragma unroll
-                            for (int q = 0; q < V / 4; ++q) dec.word(cw[j][b][q], term + 4 * q);
-#pragma unroll
-                            for (int i = 0; i < V; ++i) term[i] = g * term[i];
+                            for (int i = 0; i < V; ++i) term[i] = tab[(cw[j][b][i / 4] >> (8 * (i % 4))) & 0xffu];
                         } else {
 #pragma unroll
                             for (int i = 0; i < V; ++i) term[i] = 0.f;
