@@ -132,13 +132,21 @@ __global__ __launch_bounds__(256) void int8_decompress_vec_kernel(
     const int units = row_len / V;
     const uint8_t *src = codes + r * row_len;
     uint4 *dst = reinterpret_cast<uint4 *>((char *)out + r * row_len * (int64_t)sizeof(typename E::store_t));
+    // the 256 values of this row, worked out once (4 per lane) into the wave's own table
+    __shared__ float s_tab[4][256];
+    float *tab = s_tab[threadIdx.x >> 6];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) tab[q * WAVE + lane] = dq((uint32_t)(q * WAVE + lane));
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     for (int u = lane; u < units; u += WAVE) {
         uint32_t w[2];
         if constexpr (V == 8) { const uint2 c = reinterpret_cast<const uint2 *>(src)[u]; w[0] = c.x; w[1] = c.y; }
         else { w[0] = reinterpret_cast<const uint32_t *>(src)[u]; w[1] = 0; }
         float f[V];
 #pragma unroll
-        for (int i = 0; i < V; ++i) f[i] = dq((w[i / 4] >> (8 * (i % 4))) & 0xffu);
+        for (int i = 0; i < V; ++i) f[i] = tab[(w[i / 4] >> (8 * (i % 4))) & 0xffu];
         stream_store(dst + u, E::pack(f));
     }
 }
