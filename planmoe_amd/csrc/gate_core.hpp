@@ -283,15 +283,15 @@ __device__ __forceinline__ void gate_tile_lds(const void *__restrict__ x, const 
         __syncthreads();
         int c = 0;
         while (true) {
-            if (c + 1 >= full) { compute(a0, 0); scan(a0); __syncthreads(); break; }
+            if (c + 1 >= full) { scan(a0); compute(a0, 0); __syncthreads(); break; }
             load_a(a1, c + 1); load_b(bs, c + 1);
-            compute(a0, 0); scan(a0);
+            scan(a0); compute(a0, 0);
             store_b(bs, 1);
             __syncthreads();
             ++c;
-            if (c + 1 >= full) { compute(a1, 1); scan(a1); __syncthreads(); break; }
+            if (c + 1 >= full) { scan(a1); compute(a1, 1); __syncthreads(); break; }
             load_a(a0, c + 1); load_b(bs, c + 1);
-            compute(a1, 1); scan(a1);
+            scan(a1); compute(a1, 1);
             store_b(bs, 0);
             __syncthreads();
             ++c;

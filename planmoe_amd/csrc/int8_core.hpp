@@ -167,20 +167,19 @@ struct RowEncoder {
 };
 
 // bf16: two elements per 32-bit word all the way.  Min / max run on 16-bit order-preserving
-// keys (sign-magnitude -> two's complement) with packed integer min / max; NaNs are found by a
-// packed unsigned max of the magnitudes.
+// keys (sign-magnitude -> two's complement) with packed integer min / max.  NaNs need no scan of
+// their own: the keys of positive NaNs lie above the key of +inf (0x7f80) and those of negative
+// NaNs below the key of -inf (0x807f), so a NaN shows in the maximum or in the minimum.
 typedef short          s16x2_t __attribute__((ext_vector_type(2)));
 typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
 
 template <bool CANON>
 struct RowStats<PLANMOE_BF16, CANON> {
     s16x2_t mn, mx;
-    u16x2_t mag;
     __device__ __forceinline__ void init()
     {
         mn = s16x2_t{(short)0x7fff, (short)0x7fff};
         mx = s16x2_t{(short)0x8000, (short)0x8000};
-        mag = u16x2_t{0, 0};
     }
     __device__ __forceinline__ void add_word(uint32_t w)
     {
@@ -188,7 +187,6 @@ struct RowStats<PLANMOE_BF16, CANON> {
         const s16x2_t key = v ^ ((v >> 15) & (short)0x7fff);
         mn = __builtin_elementwise_min(mn, key);
         mx = __builtin_elementwise_max(mx, key);
-        mag = __builtin_elementwise_max(mag, __builtin_bit_cast(u16x2_t, w & 0x7fff7fffu));
     }
     __device__ __forceinline__ void add(const uint4 &raw)
     {
@@ -200,12 +198,13 @@ struct RowStats<PLANMOE_BF16, CANON> {
         if (CANON && bits == 0x8000u) bits = 0u;         // 0 + (-0) = +0
         return bf16_to_f32(bits);
     }
-    // this lane's share as three plain integers: min key, max key, largest magnitude
+    // this lane's share as three plain integers: min key, max key, and a word that exceeds 0x7f80
+    // when the share holds a NaN (kept so that shares merge with min / max / max)
     __device__ __forceinline__ void reduced(int &a, int &b, int &n) const
     {
         a = min((int)mn.x, (int)mn.y);
         b = max((int)mx.x, (int)mx.y);
-        n = max((int)mag.x, (int)mag.y);
+        n = (b > 0x7f80 || a < -0x7f81) ? 0x7fff : 0;
     }
     // min / max of the row from combined integers (any number of shares merged with min / max / max)
     __device__ static __forceinline__ void decode(int a, int b, int n, float &lo, float &hi)
@@ -220,7 +219,7 @@ struct RowStats<PLANMOE_BF16, CANON> {
         reduced(a, b, n);
         a = wave_allreduce(a, [](int p, int q) { return min(p, q); });
         b = wave_allreduce(b, [](int p, int q) { return max(p, q); });
-        n = wave_allreduce(n, [](int p, int q) { return max(p, q); });
+        n = (b > 0x7f80 || a < -0x7f81) ? 0x7fff : 0;        // a NaN anywhere in the row shows in the extremes
         decode(a, b, n, lo, hi);
     }
 };
