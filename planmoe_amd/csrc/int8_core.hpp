@@ -166,52 +166,56 @@ struct RowEncoder {
     }
 };
 
-// bf16: two elements per 32-bit word all the way.  Min / max run on 16-bit order-preserving
-// keys (sign-magnitude -> two's complement) with packed integer min / max.  NaNs need no scan of
-// their own: the keys of positive NaNs lie above the key of +inf (0x7f80) and those of negative
-// NaNs below the key of -inf (0x807f), so a NaN shows in the maximum or in the minimum.
+// bf16: two elements per 32-bit word all the way, three packed integer operations per word and no
+// key to compute.  Read as signed 16-bit integers the non-negative values are in order, read as
+// unsigned ones every negative value lies above every non-negative one and a larger pattern is a
+// more negative value.  So with  b = max as signed,  a = min as unsigned,  n = max as unsigned:
+//   row max = b if the row has a value >= +0 (b >= 0), else a (the least negative);
+//   row min = n if the row has a negative value (n >= 0x8000), else a (the least positive);
+//   a NaN shows as b > 0x7f80 (positive) or n > 0xff80 (negative).
+// Shares of a row merge with min / max / max.
 typedef short          s16x2_t __attribute__((ext_vector_type(2)));
 typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
 
 template <bool CANON>
 struct RowStats<PLANMOE_BF16, CANON> {
-    s16x2_t mn, mx;
+    s16x2_t mxs;
+    u16x2_t mnu, mxu;
     __device__ __forceinline__ void init()
     {
-        mn = s16x2_t{(short)0x7fff, (short)0x7fff};
-        mx = s16x2_t{(short)0x8000, (short)0x8000};
+        mxs = s16x2_t{(short)0x8000, (short)0x8000};
+        mnu = u16x2_t{0xffff, 0xffff};
+        mxu = u16x2_t{0, 0};
     }
     __device__ __forceinline__ void add_word(uint32_t w)
     {
-        const s16x2_t v = __builtin_bit_cast(s16x2_t, w);
-        const s16x2_t key = v ^ ((v >> 15) & (short)0x7fff);
-        mn = __builtin_elementwise_min(mn, key);
-        mx = __builtin_elementwise_max(mx, key);
+        mxs = __builtin_elementwise_max(mxs, __builtin_bit_cast(s16x2_t, w));
+        mnu = __builtin_elementwise_min(mnu, __builtin_bit_cast(u16x2_t, w));
+        mxu = __builtin_elementwise_max(mxu, __builtin_bit_cast(u16x2_t, w));
     }
     __device__ __forceinline__ void add(const uint4 &raw)
     {
         add_word(raw.x); add_word(raw.y); add_word(raw.z); add_word(raw.w);
     }
-    __device__ static __forceinline__ float key_to_f32(int key)
+    __device__ static __forceinline__ float bits_to_f32(int pattern)
     {
-        uint32_t bits = (uint32_t)(key ^ ((key >> 15) & 0x7fff)) & 0xffffu;
+        uint32_t bits = (uint32_t)pattern & 0xffffu;
         if (CANON && bits == 0x8000u) bits = 0u;         // 0 + (-0) = +0
         return bf16_to_f32(bits);
     }
-    // this lane's share as three plain integers: min key, max key, and a word that exceeds 0x7f80
-    // when the share holds a NaN (kept so that shares merge with min / max / max)
+    // this lane's share as three plain integers (merge with min / max / max)
     __device__ __forceinline__ void reduced(int &a, int &b, int &n) const
     {
-        a = min((int)mn.x, (int)mn.y);
-        b = max((int)mx.x, (int)mx.y);
-        n = (b > 0x7f80 || a < -0x7f81) ? 0x7fff : 0;
+        a = min((int)mnu.x, (int)mnu.y);
+        b = max((int)mxs.x, (int)mxs.y);
+        n = max((int)mxu.x, (int)mxu.y);
     }
-    // min / max of the row from combined integers (any number of shares merged with min / max / max)
+    // min / max of the row from combined integers
     __device__ static __forceinline__ void decode(int a, int b, int n, float &lo, float &hi)
     {
-        lo = key_to_f32(a);
-        hi = key_to_f32(b);
-        if (n > 0x7f80) { lo = __uint_as_float(0x7fc00000u); hi = lo; }
+        hi = bits_to_f32(b >= 0 ? b : a);
+        lo = bits_to_f32(n >= 0x8000 ? n : a);
+        if (b > 0x7f80 || n > 0xff80) { lo = __uint_as_float(0x7fc00000u); hi = lo; }
     }
     __device__ __forceinline__ void finish(float &lo, float &hi) const
     {
@@ -219,7 +223,7 @@ struct RowStats<PLANMOE_BF16, CANON> {
         reduced(a, b, n);
         a = wave_allreduce(a, [](int p, int q) { return min(p, q); });
         b = wave_allreduce(b, [](int p, int q) { return max(p, q); });
-        n = (b > 0x7f80 || a < -0x7f81) ? 0x7fff : 0;        // a NaN anywhere in the row shows in the extremes
+        n = wave_allreduce(n, [](int p, int q) { return max(p, q); });
         decode(a, b, n, lo, hi);
     }
 };

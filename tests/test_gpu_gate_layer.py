@@ -292,6 +292,60 @@ def test_forward_entry_point_full_size(T, M, E, k, cf, use_bias):
     assert np.array_equal(raw(out["scale"]).reshape(-1), raw(s2).reshape(-1))
 
 
+def test_row_statistics_on_special_rows():
+    """Row min / max as the three kernels that scan bf16 rows compute them (the gate kernel of the
+    chain, the stand-alone dispatch + int8, the stand-alone compressor): rows that are all negative,
+    all positive, mixed signs of zero, constant, tiny, huge, and -- where no gate has to digest them --
+    rows with infinities and NaNs, against the literal torch-CPU chain on the dispatched buffer."""
+    from planmoe_amd import ops
+    T, M, E, k = 256, 512, 4, 2
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(T, M, generator=g)
+    x[0] = -x[0].abs() - 1.0                      # all negative
+    x[1] = x[1].abs() + 1.0                       # all positive
+    x[2] = 0.0; x[2, ::2] = -0.0                  # zeros of both signs
+    x[3] = -0.0
+    x[4] = 3.25
+    x[5] = -3.25
+    x[6] *= 2.0 ** -120
+    x[7] *= 2.0 ** 120
+    x[8, 1:] = x[8, 1:].abs(); x[8, 0] = -0.0     # -0 as the only "negative"
+    x[9] = -x[9].abs(); x[9, 5] = 0.0             # +0 as the only non-negative
+    x = x.bfloat16()
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16()
+    C = ops.capacity(T, E, k, 2.0, 4)
+
+    def expect(buf):                              # Int8Compressor's chain, op by op in bf16 on the CPU
+        b = torch.min(buf, -1, True)[0]; sc = torch.max(buf, -1, True)[0] - b
+        codes = torch.mul(torch.div(torch.sub(buf, b), sc), 255.0)
+        codes = torch.nan_to_num(codes, nan=0.0, posinf=0.0, neginf=0.0).to(torch.uint8)
+        return codes, b, sc
+
+    def same(got, ref):                           # bit for bit, any NaN for a NaN, either zero for a zero
+        got, ref = got.cpu().view(-1).float(), ref.view(-1).float()
+        nan = torch.isnan(ref)
+        return torch.equal(torch.isnan(got), nan) and torch.equal(got[~nan], ref[~nan])
+
+    xd, wd = x.to(DEV), wg.to(DEV)
+    out = ops.forward_int8(xd, wd, k, C)
+    idx, loc = list(out["indices"]), list(out["locations"])
+    d = ops.dispatch_fwd(xd, idx, loc, None, E, C).cpu()
+    codes, b, sc = expect(d)
+    assert torch.equal(out["codes"].cpu(), codes) and same(out["bias"], b) and same(out["scale"], sc)
+    # with infinities and NaNs in the rows: routing given, stand-alone kernels
+    y = x.clone()
+    y[10, 3] = float("inf"); y[11, 4] = float("-inf"); y[12, 5] = float("nan"); y[13] = float("inf")
+    y[14, 0] = float("nan"); y[14, 1] = float("-inf"); y[15] = -y[15].abs(); y[15, 7] = float("nan")
+    y[16] = -y[16].abs(); y[16, 9] = -float("nan")
+    yd = y.to(DEV)
+    d = ops.dispatch_fwd(yd, idx, loc, None, E, C).cpu()
+    codes, b, sc = expect(d)
+    c2, b2, s2 = ops.dispatch_int8(yd, idx, loc, None, E, C)
+    assert torch.equal(c2.cpu(), codes) and same(b2, b) and same(s2, sc)
+    c3, b3, s3 = ops.int8_compress(d.to(DEV))
+    assert torch.equal(c3.cpu(), codes) and same(b3, b) and same(s3, sc)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_moe_layer_fused_int8_path_equals_the_stepwise_pipeline(dtype):
     """moe_layer with compress_name='int8': the fused send / receive sides (dispatch+compress,
