@@ -56,6 +56,33 @@ class _GateLogits(torch.autograd.Function):
         return g @ w, weight_grad(g, x), None
 
 
+class _GateLogitsSplit(torch.autograd.Function):
+    """fp32 logits of 16-bit activations against an fp32 gate weight (the reference's fp32_gate
+    case when the gate is kept in fp32, top.py:21-26) without reading x as fp32: the weight is
+    split into two 16-bit parts, w = hi + lo up to 2^-17 of its magnitude, both go through the MFMA
+    kernel as 2 E rows, and the two halves of the result are added.  Rounding the weight to one
+    16-bit value instead would move logits by about 1e-3 and tokens near a tie to another expert."""
+
+    @staticmethod
+    def forward(ctx, x, w32):
+        hi = w32.to(x.dtype)
+        lo = (w32 - hi.float()).to(x.dtype)
+        E = w32.shape[0]
+        if 2 * E <= 128:
+            both = ops.gate_logits(x, torch.cat([hi, lo]).contiguous(), torch.float32)
+            logits = both[:, :E] + both[:, E:]
+        else:
+            logits = ops.gate_logits(x, hi.contiguous(), torch.float32) + ops.gate_logits(x, lo.contiguous(), torch.float32)
+        ctx.save_for_backward(x, hi)
+        return logits
+
+    @staticmethod
+    def backward(ctx, grad):
+        x, hi = ctx.saved_tensors
+        g = grad.to(x.dtype)
+        return g @ hi, weight_grad(g, x).float()
+
+
 class LinearTopKGate(torch.nn.Module):
     # gates/top.py:6-26
     def __init__(self, model_dim, num_global_experts, k=1, fp32_gate=False, **options):
@@ -75,9 +102,11 @@ class LinearTopKGate(torch.nn.Module):
         """Logits [T, E], fp32 when fp32_gate (top.py:21-26).
 
         The reference up-casts x and the weight to fp32 and runs an fp32 GEMM; here x is read
-        once in its own dtype by the MFMA kernel, which accumulates in fp32.  An fp32 weight is
-        rounded to x's dtype first when x is bf16/fp16 (exact if it holds such values)."""
+        once in its own dtype by the MFMA kernel, which accumulates in fp32.  A weight kept in
+        fp32 next to 16-bit activations enters as two 16-bit parts (_GateLogitsSplit)."""
         w = self.wg.weight
+        if self.fp32_gate and w.dtype == torch.float32 and x.dtype in (torch.bfloat16, torch.float16):
+            return _GateLogitsSplit.apply(x.contiguous(), w)
         if x.dtype != w.dtype:
             w = w.to(x.dtype)
         return _GateLogits.apply(x.contiguous(), w.contiguous(),

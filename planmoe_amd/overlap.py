@@ -236,13 +236,20 @@ class _GateRouteEncode(torch.autograd.Function):
         return dx, dw, None, None, None, None, None, None
 
 
+def gate_weight_fits(gate, x):
+    """The chain's gate GEMM takes the weight in x's dtype.  A weight kept in fp32 next to 16-bit
+    activations would have to be rounded for it, which moves tokens near a tie to another expert:
+    those layers take the staged gate, which feeds the weight in as two 16-bit parts."""
+    return gate.wg.weight.dtype == x.dtype
+
+
 def gate_route_eligible(x, gate, experts, is_postscore):
     """Gate, routing and encode as one call chain (planmoe_gate_route) for any compressor."""
     from .gates import LinearTopKGate
     vec = 4 if x.dtype == torch.float32 else 8
     return (FUSE_GATE and is_postscore and type(gate) is LinearTopKGate and experts <= 64 and x.is_cuda and
             x.dtype in (torch.float32, torch.bfloat16, torch.float16) and x.shape[-1] % vec == 0 and
-            x.shape[0] >= 1)
+            x.shape[0] >= 1 and gate_weight_fits(gate, x))
 
 
 def gate_route_encode(x, gate, top_k, capacity, normalize_gate, codec):
@@ -258,7 +265,7 @@ def fused_gate_eligible(x, gate, experts, compress_name, degree, is_postscore):
     """The whole send side (gate, routing, encode, compress) as planmoe_forward_int8."""
     from .gates import LinearTopKGate
     return (fused_int8_eligible(x, compress_name, degree, is_postscore) and type(gate) is LinearTopKGate and
-            experts <= 64 and x.shape[0] >= 1)
+            experts <= 64 and x.shape[0] >= 1 and gate_weight_fits(gate, x))
 
 
 def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn, degree=1):

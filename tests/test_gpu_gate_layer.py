@@ -125,8 +125,10 @@ def test_moe_layer_forward_matches_the_oracle_composition():
             y = layer(x.to(DEV))
         assert y.shape == x.shape and y.dtype == torch.bfloat16
         from planmoe_amd import ops
-        wg = layer.gates[0].wg.weight.detach().to(torch.bfloat16)
-        logits = ops.gate_logits(x.view(T, M).to(DEV), wg.contiguous(), torch.float32)
+        # the gate is kept in fp32 here: its logits (the weight as two bf16 parts) are what the layer routes on
+        with torch.no_grad():
+            logits = layer.gates[0](x.view(T, M).to(DEV))
+        assert logits.dtype == torch.float32
         r = ops.route_topk(logits, k, is_logits=True, want_scores=True)
         idx, loc, gates, _ = oracle.route_topk(r["scores"].cpu().numpy(), k)
         C = oracle.capacity(T, E, k, 1.0, 4)
@@ -510,6 +512,45 @@ def test_gate_weight_gradient_split_over_token_chunks(T, M, E, dtype):
     ref = g.double().t() @ x.double()
     tol = {torch.float32: 1e-5, torch.bfloat16: 1e-2, torch.float16: 2e-3}[dtype]
     assert (got.double() - ref).abs().max().item() <= tol * ref.abs().max().item()
+
+
+def test_fp32_gate_weight_next_to_bf16_activations():
+    """fp32_gate with the gate kept in fp32 (top.py:21-26: x.float() @ wg.float()): the weight goes
+    through the MFMA kernel as two bf16 parts, so the logits stay within fp32 summation noise of the
+    fp32 product, where a weight rounded to bf16 is off by 1e-3 and re-routes tokens near a tie."""
+    import planmoe_amd
+    from planmoe_amd import gates
+    T, M, E, k = 4096, 1024, 8, 2
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(T, M, generator=g).bfloat16().to(DEV)
+    gate = gates.LinearTopKGate(M, E, k=k, fp32_gate=True).to(DEV)
+    assert gate.wg.weight.dtype == torch.float32
+    with torch.no_grad():
+        gate.wg.weight.copy_(torch.randn(E, M, generator=g) * M ** -0.5)
+    logits = gate(x)
+    assert logits.dtype == torch.float32
+    ref = x.double() @ gate.wg.weight.double().t()
+    err = (logits.double() - ref).abs().max().item()
+    rounded = (x.double() @ gate.wg.weight.bfloat16().double().t() - ref).abs().max().item()
+    assert err <= 2e-5 and rounded > 20 * err
+    # same choices as the fp32 product wherever the runner-up is not within the noise
+    top = torch.topk(ref, k + 1, dim=1)
+    clear = (top.values[:, k - 1] - top.values[:, k]) > 1e-4
+    mine = torch.topk(logits, k, dim=1).indices
+    assert torch.equal(mine[clear], top.indices[clear][:, :k]) and clear.float().mean() > 0.99
+
+    # the layer end to end with such a gate: experts in bf16, gate in fp32; gradients reach the fp32 weight
+    layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'fp32_gate': True, 'capacity_factor': 1.25}, 128,
+                                  experts={'type': 'ffn', 'count_per_node': 4, 'hidden_size_per_expert': 64},
+                                  seeds=(1, 2, 3), compress_name='int8').to(DEV)
+    layer.experts.to(torch.bfloat16)
+    assert layer.gates[0].wg.weight.dtype == torch.float32
+    xin = torch.randn(300, 128, generator=g).bfloat16().to(DEV).requires_grad_(True)
+    y = layer(xin)
+    (y.float().pow(2).mean() + y.l_aux.float()).backward()
+    wgrad = layer.gates[0].wg.weight.grad
+    assert y.dtype == torch.bfloat16 and wgrad.dtype == torch.float32 and wgrad.abs().sum() > 0
+    assert torch.isfinite(xin.grad).all() and xin.grad.abs().sum() > 0
 
 
 def test_moe_layer_prescore_noise_and_load_importance_loss():
