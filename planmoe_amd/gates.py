@@ -66,13 +66,16 @@ class _GateLogitsSplit(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, w32):
         hi = w32.to(x.dtype)
-        lo = (w32 - hi.float()).to(x.dtype)
+        # fp16: the low part would sit among the subnormals; scaled by a power of two it does not
+        up = 1024.0 if x.dtype == torch.float16 else 1.0
+        lo = ((w32 - hi.float()) * up).to(x.dtype)
         E = w32.shape[0]
         if 2 * E <= 128:
             both = ops.gate_logits(x, torch.cat([hi, lo]).contiguous(), torch.float32)
-            logits = both[:, :E] + both[:, E:]
+            logits = both[:, :E] + both[:, E:] * (1.0 / up)
         else:
-            logits = ops.gate_logits(x, hi.contiguous(), torch.float32) + ops.gate_logits(x, lo.contiguous(), torch.float32)
+            logits = (ops.gate_logits(x, hi.contiguous(), torch.float32) +
+                      ops.gate_logits(x, lo.contiguous(), torch.float32) * (1.0 / up))
         ctx.save_for_backward(x, hi)
         return logits
 

@@ -514,6 +514,19 @@ def test_gate_weight_gradient_split_over_token_chunks(T, M, E, dtype):
     assert (got.double() - ref).abs().max().item() <= tol * ref.abs().max().item()
 
 
+@pytest.mark.parametrize("E", [8, 96])
+def test_fp32_gate_weight_next_to_fp16_activations(E):
+    from planmoe_amd import gates
+    T, M = 1000, 512
+    g = torch.Generator().manual_seed(22)
+    x = torch.randn(T, M, generator=g).half().to(DEV)
+    gate = gates.LinearTopKGate(M, E, k=2, fp32_gate=True).to(DEV)
+    with torch.no_grad():
+        gate.wg.weight.copy_(torch.randn(E, M, generator=g) * M ** -0.5)
+    ref = x.double() @ gate.wg.weight.double().t()
+    assert (gate(x).double() - ref).abs().max().item() <= 2e-5
+
+
 def test_fp32_gate_weight_next_to_bf16_activations():
     """fp32_gate with the gate kept in fp32 (top.py:21-26: x.float() @ wg.float()): the weight goes
     through the MFMA kernel as two bf16 parts, so the logits stay within fp32 summation noise of the
