@@ -185,16 +185,28 @@ __global__ __launch_bounds__(256) void bwd_gate_kernel(
 #pragma unroll
         for (int j = 0; j < G; ++j) s[j] = (j < np) ? rl_i(slot, j) : -1;
         float acc[G] = {0.f, 0.f, 0.f, 0.f};
-        for (int u = lane; u < units; u += WAVE) {
-            float a[IO::U];
-            IO::load_stream(xr, u, a);
+        // two units of the row per lane and pass; the slot rows of all choices are requested with
+        // straight-line loads at clamped addresses (a dropped choice reads slot 0 and is left out
+        // of the sum; the caller guarantees a slot 0 to read: capacity >= 1)
+        constexpr int B = 2;
+        for (int u0 = lane; u0 < units; u0 += B * WAVE) {
+            float a[B][IO::U];
+#pragma unroll
+            for (int b = 0; b < B; ++b) IO::load_stream(xr, min(u0 + b * WAVE, units - 1), a[b]);
 #pragma unroll
             for (int j = 0; j < G; ++j) {
-                if (s[j] < 0) continue;
-                float d[IO::U];
-                IO::load_stream((const char *)dispatched + (int64_t)s[j] * row_bytes, u, d);
+                if (j < np) {
+                    const char *row = (const char *)dispatched + (int64_t)max(s[j], 0) * row_bytes;
+                    float d[B][IO::U];
 #pragma unroll
-                for (int i = 0; i < IO::U; ++i) acc[j] = fmaf(d[i], a[i], acc[j]);
+                    for (int b = 0; b < B; ++b) IO::load_stream(row, min(u0 + b * WAVE, units - 1), d[b]);
+#pragma unroll
+                    for (int b = 0; b < B; ++b) {
+                        const bool live = s[j] >= 0 && u0 + b * WAVE < units;
+#pragma unroll
+                        for (int i = 0; i < IO::U; ++i) acc[j] = live ? fmaf(d[b][i], a[b][i], acc[j]) : acc[j];
+                    }
+                }
             }
         }
 #pragma unroll
@@ -328,6 +340,11 @@ extern "C" int planmoe_bwd_gate(const void *x, const void *dispatched, int dtype
     PM_REQUIRE(x && grad_gates, "planmoe_bwd_gate: NULL argument");
     PM_REQUIRE(dispatched || capacity == 0, "planmoe_bwd_gate: dispatched is NULL");
     hipStream_t st = (hipStream_t)stream;
+    if (capacity == 0) {                               // no slot, no row to read: every gradient is zero
+        for (int j = 0; j < top_k; ++j) fill_u32((uint32_t *)(grad_gates + (int64_t)j * plane_stride), (size_t)samples, 0u, st);
+        PM_LAUNCH_CHECK("planmoe_bwd_gate");
+        return 0;
+    }
     const int vec = dtype == PLANMOE_F32 ? 4 : 8;
     const bool vector = (model_dim % vec == 0) && aligned16(x) && aligned16(dispatched);
     const int blocks = (samples + 3) / 4;
