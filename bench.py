@@ -264,6 +264,27 @@ def cpu_stage_table(min_seconds=2.0):
     s3 = oracle.softmax(rng.standard_normal((T3, E3), dtype=np.float32))
     add("route_topk", "3", "%d tokens" % T3, T3 * E3 * 4 + T3 * 12, lambda: oracle.route_topk(s3, 1))
 
+    # the routing as the reference's CPU path runs it: ATen ops on the CPU, multi-threaded by torch
+    # (softmax, top-k, one-hot masks, cumsum, fast_dispatch.py:140-172 restated)
+    import torch
+
+    def torch_routing(lg, kk):
+        sc = torch.softmax(lg, 1)
+        top = torch.topk(sc, kk, dim=1).indices
+        masks = [torch.zeros_like(sc, dtype=torch.int64).scatter_(1, top[:, j:j + 1], 1) for j in range(kk)]
+        gs = [(sc * m).sum(1) for m in masks]
+        locs, base = [], torch.zeros((1, sc.shape[1]), dtype=torch.int64)
+        for j in range(kk):
+            locs.append((((torch.cumsum(masks[j], 0) - 1) + base) * masks[j]).sum(1).to(torch.int32))
+            base = base + masks[j].sum(0, keepdim=True)
+        den = torch.clamp(sum(gs), min=torch.finfo(sc.dtype).eps)
+        return top, locs, [v / den for v in gs]
+
+    tl2 = torch.from_numpy(logits)
+    add("routing, torch-CPU x%d thr" % torch.get_num_threads(), "2", tok, T * E * 4 + T * k * 12, lambda: torch_routing(tl2, k))
+    tl3 = torch.from_numpy(rng.standard_normal((T3, E3), dtype=np.float32))
+    add("routing, torch-CPU x%d thr" % torch.get_num_threads(), "3", "%d tokens" % T3, T3 * E3 * 4 + T3 * 12, lambda: torch_routing(tl3, 1))
+
     # config 5's codecs on 2048 of the 131072 slot rows
     R5, M5 = 2048, 1024
     f = rng.standard_normal((R5, M5), dtype=np.float32)
