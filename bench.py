@@ -298,7 +298,7 @@ def cpu_stage_table(min_seconds=2.0):
     lz = oracle.lz_compress(f)
     add("lz_decompress 30% empty", "5", rw, R5 * M5 * 4, lambda: oracle.lz_decompress(*lz))
 
-    print("CPU oracle, 1 thread of %d (%s)" % (os.cpu_count(), "bounded samples; GB/s of algorithmic bytes"))
+    print("CPU oracle, 1 thread of %d (%s)" % (os.cpu_count(), "bounded samples; GB/s of algorithmic bytes; the torch-CPU rows use torch's threads"))
     print("%-26s %-4s %-12s %10s %10s %8s" % ("stage", "cfg", "sample", "alg MB", "ms / call", "GB/s"))
     for name, cfg, sample, nbytes, sec in rows:
         print("%-26s %-4s %-12s %10.1f %10.2f %8.3f" % (name, cfg, sample, nbytes / 1e6, sec * 1e3, nbytes / sec / 1e9))
