@@ -128,6 +128,15 @@ int planmoe_route_bwd(const void *scores, int dtype, const int32_t *indices, con
 int planmoe_gate_logits(const void *x, const void *wg, int dtype, void *logits, int out_dtype,
                         int samples, int model_dim, int experts, void *stream);
 
+/* The gate's share of the gradient of x, added in place: dx[t, :] += sum_e grad_logits[t, e] *
+ * wg[e, :] -- the backward of LinearTopKGate.forward (gates/top.py:20-26, which autograd runs as
+ * a GEMM and an accumulation into x.grad) as one streaming read-modify-write of dx.  dx and wg in
+ * `dtype`, grad_logits fp32 [samples, experts] (rounded to `dtype` first, as the cast in front of
+ * the GEMM would); up to 8 experts (above that a GEMM is the better tool); model_dim a multiple
+ * of 16 bytes' worth of elements. */
+int planmoe_gate_dx_accumulate(void *dx, int dtype, const float *grad_logits, const void *wg, int samples,
+                               int model_dim, int experts, void *stream);
+
 /* ---------------------------------------------------------------- dispatch / combine
  * Replace the JIT kernels of jit_kernels/sparse.py (create_forward :17-35,
  * create_backward_data :38-64, create_backward_gate :67-134), their CPU twins

@@ -78,6 +78,7 @@ SIGNATURES = {
     "planmoe_combine_zfp_workspace_bytes": (c_size_t, [c_int, c_int]),
     "planmoe_combine_zfp": (c_int, [c_void_p, c_double, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int,
                                     c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "planmoe_gate_dx_accumulate": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "planmoe_bwd_gate_zfp": (c_int, [c_void_p, c_double, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int,
                                      c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "planmoe_lz_blocks": (c_int64, [c_int64]),

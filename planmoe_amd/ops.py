@@ -173,6 +173,23 @@ def gate_logits(x, wg, out_dtype=None):
     return out
 
 
+def gate_dx_accumulate(dx, grad_logits, wg):
+    """dx[T, M] += grad_logits[T, E] @ wg[E, M] in place (up to 8 experts): the gate's share of x.grad."""
+    _need_gpu(dx, "gate_dx_accumulate")
+    dx = _contig(dx, "gate_dx_accumulate")
+    wg = _contig(wg, "gate_dx_accumulate")
+    if dx.dtype != wg.dtype:
+        raise PlanMoEError("gate_dx_accumulate: dx and wg must share a dtype")
+    g = grad_logits.to(torch.float32).contiguous()
+    T, M = dx.shape
+    E = wg.shape[0]
+    if tuple(g.shape) != (T, E) or wg.shape[1] != M:
+        raise PlanMoEError("gate_dx_accumulate: shapes do not fit")
+    check(lib.planmoe_gate_dx_accumulate(_ptr(dx), _dt(dx, "gate_dx_accumulate"), _ptr(g), _ptr(wg), T, M, E,
+                                         _stream(dx)))
+    return dx
+
+
 # ------------------------------------------------------------------------------ dispatch / combine
 def _plane_args(indices, locations, gates, who):
     idx, s1 = planes(indices, torch.int32)

@@ -192,7 +192,13 @@ def _gate_backward(x, w, scores, indices, counts, normalize_gate, dx, grad_gates
                                 counts if grad_l_aux is not None else None, through_softmax=True)
     g = grad_logits.to(x.dtype)
     dw = weight_grad(g, x)
-    dx = g @ w if dx is None else dx.addmm_(g, w)
+    vec = 4 if x.dtype == torch.float32 else 8
+    if dx is None:
+        dx = g @ w
+    elif w.shape[0] <= 8 and x.shape[1] % vec == 0 and dx.is_contiguous():
+        ops.gate_dx_accumulate(dx, grad_logits, w)           # one pass over dx instead of a GEMM with K = experts
+    else:
+        dx.addmm_(g, w)
     return dx, dw
 
 

@@ -514,6 +514,25 @@ def test_gate_weight_gradient_split_over_token_chunks(T, M, E, dtype):
     assert (got.double() - ref).abs().max().item() <= tol * ref.abs().max().item()
 
 
+@pytest.mark.parametrize("T,M,E,dtype", [(1000, 512, 8, torch.bfloat16), (257, 264, 3, torch.bfloat16), (4099, 1024, 7, torch.float16),
+                                         (300, 100, 2, torch.float32), (1, 8, 1, torch.bfloat16), (16384, 4096, 8, torch.bfloat16)])
+def test_gate_dx_accumulate(T, M, E, dtype):
+    """planmoe_gate_dx_accumulate (dx += g @ wg in one pass over dx) against the product in fp64."""
+    from planmoe_amd import ops
+    g0 = torch.Generator().manual_seed(T + E)
+    dx = torch.randn(T, M, generator=g0).to(dtype).to(DEV)
+    w = (torch.randn(E, M, generator=g0) * M ** -0.5).to(dtype).to(DEV)
+    g = (torch.randn(T, E, generator=g0) * 0.1).to(DEV)
+    ref = dx.double() + g.to(dtype).double() @ w.double()
+    guard = dx.clone()
+    got = ops.gate_dx_accumulate(dx, g, w)
+    assert got.data_ptr() == dx.data_ptr() and not torch.equal(dx, guard)
+    ulp = {torch.float32: 2.0 ** -23, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+    assert ((dx.double() - ref).abs() <= ulp * ref.abs() + 1e-6).all()
+    with pytest.raises(Exception):
+        ops.gate_dx_accumulate(dx, torch.zeros(T, 9, device=DEV), torch.zeros(9, M, device=DEV, dtype=dtype))
+
+
 @pytest.mark.parametrize("E", [8, 96])
 def test_fp32_gate_weight_next_to_fp16_activations(E):
     from planmoe_amd import gates
