@@ -133,6 +133,9 @@ def kernel_table(only=None):
     dc = ops.int8_compress(d)
     add("combine_bwd_int8 (coded in)", "4", xb + live * M + R * M + 2 * R * 4 + plane + T * k * 4,
         lambda: ops.combine_bwd_int8(x, dc, idx, loc, gates, E, C))
+    dxb = torch.randn(T, M, generator=g).bfloat16().to(dev)
+    glog = (torch.randn(T, E, generator=g) * 0.01).to(dev)
+    add("gate_dx_accumulate", "2", 2 * xb + T * E * 4 + E * M * 2, lambda: ops.gate_dx_accumulate(dxb, glog, wg))
     plan = ops.ForwardInt8Plan(x, wg, k, C, fp32_gate=True)
     add("forward_int8 (chain)", "2", xb + E * M * 2 + R * M + R * 4 + plane, plan.run)
     del d, dc, codes, plan
