@@ -558,6 +558,9 @@ extern "C" int planmoe_route_locations(const int32_t *indices, int64_t plane_str
     PM_REQUIRE(samples >= 0 && experts >= 1 && top_k >= 1, "planmoe_route_locations: bad shape");
     PM_REQUIRE(experts <= ROUTE_MAX_E, "planmoe_route_locations: experts %d > supported %d", experts, ROUTE_MAX_E);
     PM_REQUIRE(plane_stride >= samples, "planmoe_route_locations: plane_stride < samples");
+    // the workspace query sizes its tables with min(top_k, experts) planes; the planes given here
+    // are used as they are, so more planes than experts would run past it
+    PM_REQUIRE(top_k <= experts, "planmoe_route_locations: top_k %d > experts %d", top_k, experts);
     hipStream_t st = (hipStream_t)stream;
     if (samples == 0) {
         if (expert_counts) fill_u32((uint32_t *)expert_counts, (size_t)top_k * experts, 0u, st);

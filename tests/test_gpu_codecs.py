@@ -263,6 +263,14 @@ def test_bwd_gate_zfp_equals_decompress_then_bwd_gate(T, M, E, k, cf):
         ref = (dout.double() * rows.double()).sum(1) * kept
         mag = (dout.double() * rows.double()).abs().sum(1) * kept
         assert ((got[j].double() - ref).abs() <= 1e-5 * mag + 1e-30).all()
+        # the oracle's leg: its own decode of its own stream, then its dot product in fp64
+        if E * C > 0:
+            n = ops.zfp_stream_bytes(2, M, E * C)
+            ost = oracle.zfp_compress(y.cpu().numpy(), 2)
+            assert np.array_equal(st.cpu().numpy()[:n], ost)
+            orows = oracle.zfp_decompress(ost, E * C, M, 2).astype(np.float64)
+            oref = oracle.bwd_gate(idx[j].cpu().numpy(), loc[j].cpu().numpy(), dout.double().cpu().numpy(), orows, C)
+            assert (np.abs(got[j].double().cpu().numpy() - oref) <= 1e-5 * mag.cpu().numpy() + 1e-30).all()
         assert ((got[j].double() - want[j].double()).abs() <= 2e-5 * mag + 1e-30).all()
         assert (got[j][~kept] == 0).all()
 
@@ -404,6 +412,66 @@ def test_combine_bwd_int8_equals_the_unfused_backward(T, M, E, k, cf, dtype):
     c4, b4, s4, g4 = ops.combine_bwd_int8(dout.to(DEV), (ec, eb, es), i, l, gt, E, C)
     assert torch.equal(c3, c4) and torch.equal(b3, b4) and torch.equal(s3, s4)
     assert np.array_equal(raw(g3), raw(g4))
+
+
+def test_config4_backward_full_size():
+    """Config 4 at its own shape: 16384 x 4096 bf16, 8 experts, top-2, cf 1.25 (capacity 5120), the
+    routing of config 2 (x, wg seed 0), upstream gradient N(0,1) seed 1, expert output seed 2.
+    (i) backward of combine fused with the int8 compress of the gradient buffer, expert output
+    given as bf16 and as int8 codes: codes / bias / scale bit-exact against the oracle, gate
+    gradients within rtol 1e-2 of the fp64 dot product (+ 1e-6 of the sum of the terms'
+    magnitudes); (ii) int8 decompress bit-exact; (iii) backward of dispatch (gather-sum without
+    gates) bit-exact, stand-alone and fused with the decompress."""
+    from planmoe_amd import ops
+    T, M, E, k = 16384, 4096, 8, 2
+    g0 = torch.Generator().manual_seed(0)
+    x = torch.randn(T, M, generator=g0).bfloat16()
+    wg = (torch.randn(E, M, generator=g0) * M ** -0.5).bfloat16()
+    r = ops.gate_route(x.to(DEV), wg.to(DEV), k, want_scores=True)
+    idx, loc, gates, _ = oracle.route_topk(r["scores"].cpu().numpy(), k)
+    assert np.array_equal(r["indices"].cpu().numpy(), idx) and np.array_equal(r["locations"].cpu().numpy(), loc)
+    C = oracle.capacity(T, E, k, 1.25, 4)
+    assert C == 5120
+    dout = torch.randn(T, M, generator=torch.Generator().manual_seed(1)).bfloat16()
+    eo = torch.randn(E * C, M, generator=torch.Generator().manual_seed(2)).bfloat16()
+    i, l = list(r["indices"]), list(r["locations"])
+    gt = [torch.from_numpy(a).to(DEV) for a in gates]
+    dd, ed = dout.to(DEV), eo.to(DEV)
+    codes, bias, scale, gg = ops.combine_bwd_int8(dd, ed, i, l, gt, E, C)
+    # (i) the gradient buffer [E * C, M] = scatter of round(gate * dOut), then the codec
+    d = torch.from_numpy(oracle.encode(dout.float().numpy(), list(idx), list(loc), list(gates), E, C)).bfloat16()
+    rc, rb, rs = oracle.int8_compress(bf16_bits(d))
+    del d
+    assert np.array_equal(codes.cpu().numpy(), rc)
+    assert np.array_equal(raw(bias), np_raw(rb)) and np.array_equal(raw(scale), np_raw(rs))
+    xd, e64 = dout.double().numpy(), eo.double().numpy()
+    for j in range(k):
+        want = oracle.bwd_gate(idx[j], loc[j], xd, e64, C)
+        mag = oracle.bwd_gate(idx[j], loc[j], np.abs(xd), np.abs(e64), C)
+        got = gg[j].float().cpu().numpy()
+        assert (np.abs(got - want) <= 1e-2 * np.abs(want) + 1e-6 * mag).all()
+        assert (got[loc[j] >= C] == 0).all()
+    del e64
+    # the expert output as the int8 codes the receive side holds: what decompress would have given
+    ec, eb, es = ops.int8_compress(ed)
+    oc, ob, os_ = oracle.int8_compress(bf16_bits(eo))
+    assert np.array_equal(ec.cpu().numpy(), oc)
+    seen = from_bf16_bits(oracle.int8_decompress(oc, ob, os_)).double().numpy()
+    c4, b4, s4, g4 = ops.combine_bwd_int8(dd, (ec, eb, es), i, l, gt, E, C)
+    assert torch.equal(c4, codes) and torch.equal(b4, bias) and torch.equal(s4, scale)
+    for j in range(k):
+        want = oracle.bwd_gate(idx[j], loc[j], xd, seen, C)
+        mag = oracle.bwd_gate(idx[j], loc[j], np.abs(xd), np.abs(seen), C)
+        got = g4[j].float().cpu().numpy()
+        assert (np.abs(got - want) <= 1e-2 * np.abs(want) + 1e-6 * mag).all()
+    del seen, xd
+    # (ii) decompress of the gradient buffer, (iii) backward of dispatch: sum of the slot rows
+    dec_ref = oracle.int8_decompress(rc, rb, rs)
+    dec = ops.int8_decompress(codes, bias, scale)
+    assert np.array_equal(raw(dec), np_raw(dec_ref))
+    dx_ref = torch.from_numpy(oracle.decode(from_bf16_bits(dec_ref).float().numpy(), list(idx), list(loc), None, T, C)).bfloat16()
+    assert np.array_equal(raw(ops.combine_fwd(dec, i, l, None, T, C)), raw(dx_ref))
+    assert np.array_equal(raw(ops.combine_int8(codes, bias, scale, i, l, None, T, C)), raw(dx_ref))
 
 
 @pytest.mark.parametrize("T,M,E,k,dtype,gated", [(1000, 512, 8, 2, torch.bfloat16, True), (300, 264, 5, 3, torch.bfloat16, False),

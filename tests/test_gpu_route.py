@@ -148,6 +148,14 @@ def test_extract_critical_structure():
     # data-dependent capacity (capacity_factor = 0): max location + 1, aligned
     (_, _, _, _, C0), _ = planmoe_amd.extract_critical(scores.to(DEV), 2, capacity_factor=0, alignment=4)
     assert C0 == (int(loc.max()) + 1 + 3) // 4 * 4
+    # capacity_factor < 0 (fast_dispatch.py:185-186): the data-dependent capacity, capped at
+    # top_k * int(-cf * ceil(T / E)); both sides of the cap
+    need = int(loc.max()) + 1
+    per_expert = (1000 + 7) // 8
+    for cf in (-0.25, -1.0, -64.0):
+        (_, _, _, _, Cn), _ = planmoe_amd.extract_critical(scores.to(DEV), 2, capacity_factor=cf, alignment=4)
+        assert Cn == (min(need, 2 * int(-cf * per_expert)) + 3) // 4 * 4
+    assert 2 * int(0.25 * per_expert) < need < 2 * int(64.0 * per_expert)
     # custom loss callables see (scores, top-k ids [T, k])
     (_, _, _, _, _), l2 = planmoe_amd.extract_critical(scores.to(DEV), 2, loss_fn=lambda s, ids: ids.float().mean())
     assert abs(float(l2) - float(np.stack(list(idx), 1).mean())) < 1e-5
