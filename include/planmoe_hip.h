@@ -261,6 +261,24 @@ int planmoe_forward_int8(const void *x, const void *wg, int dtype, int fp32_gate
                          float *l_aux, int32_t *expert_counts, uint8_t *codes, void *bias, void *scale,
                          void *workspace, size_t workspace_bytes, void *stream);
 
+/* planmoe_forward_int8 for callers that cannot allocate device memory or carry a workspace
+ * around (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * the same launches with the workspace taken from a 4 MiB buffer built into the library's device
+ * image (a static __device__ array; every GPU the library runs on holds its own copy until the
+ * process ends).  It has no counterpart in the reference.  Calls no allocator.  Shapes whose
+ * planmoe_forward_workspace_bytes exceed 4 MiB are refused with an error (the five benchmark
+ * configurations need 0.4 - 1.7 MiB).  All calls on one GPU share that GPU's buffer, which keeps
+ * the previous call's contents: calls that overlap on one GPU (two streams, two threads) race;
+ * calls on one stream do not.  The first call on a device looks the buffer's address up
+ * (hipGetSymbolAddress): make that call outside a graph capture.  Outputs as planmoe_forward_int8. */
+int planmoe_forward_int8_static(const void *x, const void *wg, int dtype, int fp32_gate,
+                                const float *logit_bias, int samples, int model_dim, int experts,
+                                int top_k, int normalize_gate, int capacity, int32_t *indices,
+                                int32_t *locations, void *gates, int64_t plane_stride,
+                                void *logits_out, void *scores_out, float *l_aux,
+                                int32_t *expert_counts, uint8_t *codes, void *bias, void *scale,
+                                void *stream);
+
 /* Runs only the last launch of planmoe_forward_int8 (slot finalisation + dispatch + int8
  * compress) again, from the state a preceding planmoe_forward_int8 call with the same shapes
  * left in `workspace`.  Same outputs; meant for profiling that launch on its own.  It has no

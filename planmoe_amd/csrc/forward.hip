@@ -24,6 +24,7 @@
 #include "rows.hpp"
 #include "int8_core.hpp"
 #include "offsets.hpp"
+#include <mutex>
 
 namespace pm {
 
@@ -867,6 +868,60 @@ extern "C" int planmoe_forward_int8(const void *x, const void *wg, int dtype, in
                             plane_stride, l_aux, expert_counts, codes, bias, scale, plan, st)) return 1;
     PM_LAUNCH_CHECK("planmoe_forward_int8");
     return 0;
+}
+
+// ---- the same entry point for callers that can allocate nothing: its workspace is a file-scope
+// array in device memory.  Host code must not hand `static_scratch` itself to a kernel (on the
+// host the name is a stand-in, not a device address): the address is asked for once per device
+// and kept.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)4 << 20;
+constexpr int STATIC_SCRATCH_DEVICES = 64;
+static __device__ __align__(256) unsigned char static_scratch[STATIC_SCRATCH_BYTES];
+static void *g_static_scratch[STATIC_SCRATCH_DEVICES];
+static std::mutex g_static_scratch_lock;
+
+// device address of this device's copy of the array (every GPU holds its own), NULL + error text on failure
+static void *static_scratch_address()
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= STATIC_SCRATCH_DEVICES) {
+        set_error("planmoe_forward_int8_static: no current device (%s)", hipGetErrorString(e));
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> hold(g_static_scratch_lock);
+    if (!g_static_scratch[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch));
+        if (e != hipSuccess || !p) {
+            set_error("planmoe_forward_int8_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_static_scratch[dev] = p;
+    }
+    return g_static_scratch[dev];
+}
+
+extern "C" int planmoe_forward_int8_static(const void *x, const void *wg, int dtype, int fp32_gate,
+                                           const float *logit_bias, int samples, int model_dim, int experts,
+                                           int top_k, int normalize_gate, int capacity, int32_t *indices,
+                                           int32_t *locations, void *gates, int64_t plane_stride,
+                                           void *logits_out, void *scores_out, float *l_aux,
+                                           int32_t *expert_counts, uint8_t *codes, void *bias, void *scale,
+                                           void *stream)
+{
+    const size_t need = planmoe_forward_workspace_bytes(samples, experts, top_k);
+    PM_REQUIRE(need <= STATIC_SCRATCH_BYTES,
+               "planmoe_forward_int8_static: %d tokens x %d experts x top-%d need %zu bytes of scratch, the "
+               "built-in buffer holds %zu; use planmoe_forward_int8 with a workspace of the caller's",
+               samples, experts, top_k, need, STATIC_SCRATCH_BYTES);
+    void *ws = static_scratch_address();
+    if (!ws) return 1;
+    // nothing in the workspace has to start at zero: every word a launch reads was written by the
+    // launch before it in the same call (the padding of the transposed histogram included)
+    return planmoe_forward_int8(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
+                                normalize_gate, capacity, indices, locations, gates, plane_stride, logits_out,
+                                scores_out, l_aux, expert_counts, codes, bias, scale, ws, STATIC_SCRATCH_BYTES, stream);
 }
 
 extern "C" int planmoe_forward_int8_redispatch(const void *x, int dtype, int samples, int model_dim,

@@ -370,7 +370,10 @@ def _forward_workspace(T, E, k, device):
     ws = _forward_ws.get(key)
     if ws is None or ws.numel() < need:
         ws = torch.empty((max(need, 1 << 20),), dtype=torch.uint8, device=device)
-        _forward_ws[key] = ws
+        # memory allocated during a graph capture belongs to the graph's private pool: such a
+        # buffer serves this call only and is not kept for later eager calls
+        if not torch.cuda.is_current_stream_capturing():
+            _forward_ws[key] = ws
     return ws
 
 
@@ -431,14 +434,37 @@ def forward_int8(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, norma
     return out
 
 
+def forward_int8_static(x, wg, top_k, capacity_, out, fp32_gate=True, logit_bias=None, normalize_gate=True):
+    """forward_int8 through the entry point that allocates nothing: the workspace is the library's
+    built-in device buffer and every output is the caller's (`out`: the dict of tensors a
+    forward_int8 call returned, or tensors of those shapes).  x, wg and logit_bias must be
+    contiguous GPU tensors already (fp32 bias): nothing is copied or created here."""
+    T, M = x.shape
+    E = wg.shape[0]
+    k = min(int(top_k), E)
+    for t in (x, wg) + tuple(v for v in out.values() if v is not None):
+        if not (t.is_cuda and t.is_contiguous()):
+            raise PlanMoEError("forward_int8_static: contiguous GPU tensors only")
+    check(lib.planmoe_forward_int8_static(_ptr(x), _ptr(wg), _dt(x, "forward_int8_static"), int(bool(fp32_gate)),
+                                          _ptr(logit_bias), T, M, E, k, int(bool(normalize_gate)), capacity_,
+                                          _ptr(out["indices"]), _ptr(out["locations"]), _ptr(out["gates"]),
+                                          out["indices"].shape[1], _ptr(out.get("logits")), _ptr(out.get("scores")),
+                                          _ptr(out.get("l_aux")), _ptr(out.get("counts")), _ptr(out["codes"]),
+                                          _ptr(out["bias"]), _ptr(out["scale"]), _stream(x)))
+    return out
+
+
 class ForwardInt8Plan:
     """forward_int8 with every output and the workspace allocated once: `run()` is a single
     C-ABI call that enqueues the two launches (for serving loops that reuse their buffers)."""
 
     def __init__(self, x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
                  want_l_aux=True, want_counts=False):
-        x, wg, T, M, E, k, bias, out, ws = _forward_common(x, wg, top_k, fp32_gate, logit_bias, False,
-                                                           False, want_l_aux, want_counts)
+        x, wg, T, M, E, k, bias, out, _ = _forward_common(x, wg, top_k, fp32_gate, logit_bias, False,
+                                                          False, want_l_aux, want_counts)
+        # a workspace of the plan's own: redispatch() reads the routing state run() left in it, which
+        # another forward call on the same stream would overwrite in a shared one
+        ws = torch.empty((max(lib.planmoe_forward_workspace_bytes(T, E, k), 256),), dtype=torch.uint8, device=x.device)
         R = E * capacity_
         out["codes"] = torch.empty((R, M), dtype=torch.uint8, device=x.device)
         out["bias"] = torch.empty((R, 1), dtype=x.dtype, device=x.device)
