@@ -261,6 +261,27 @@ int planmoe_forward_int8(const void *x, const void *wg, int dtype, int fp32_gate
                          float *l_aux, int32_t *expert_counts, uint8_t *codes, void *bias, void *scale,
                          void *workspace, size_t workspace_bytes, void *stream);
 
+/* The same chain in ONE launch that reads x once (the two launches above read it twice: the slot
+ * of a second choice needs the first-choice counts of the whole batch).  One work-group per compute
+ * unit holds the codes of its tokens on chip (LDS and registers) until every work-group has
+ * published its expert histogram, then writes them to their slots.  Served shapes: bf16, model_dim
+ * 4096, experts <= 16, top_k <= 4, samples <= 64 x the number of compute units; any other shape is
+ * an error here (planmoe_forward_int8 picks between the two on its own).  Outputs as
+ * planmoe_forward_int8 (logits may differ from it in the last bit: another summation order).
+ * The wait between the work-groups is bounded: spin_limit polls (0 = the default, about a second);
+ * a work-group that gives up writes none of its rows and sets *gave_up to 1 (optional device
+ * word, cleared by the caller).  Two such launches that run at the same time on one GPU can keep
+ * each other's work-groups from becoming resident: run them one after the other.
+ * It has no counterpart in the reference. */
+int planmoe_forward_int8_single(const void *x, const void *wg, int dtype, int fp32_gate,
+                                const float *logit_bias, int samples, int model_dim, int experts,
+                                int top_k, int normalize_gate, int capacity, int32_t *indices,
+                                int32_t *locations, void *gates, int64_t plane_stride,
+                                void *logits_out, void *scores_out, float *l_aux,
+                                int32_t *expert_counts, uint8_t *codes, void *bias, void *scale,
+                                void *workspace, size_t workspace_bytes, int spin_limit,
+                                int32_t *gave_up, void *stream);
+
 /* planmoe_forward_int8 for callers that cannot allocate device memory or carry a workspace
  * around (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
  * the same launches with the workspace taken from a 4 MiB buffer built into the library's device

@@ -25,8 +25,12 @@
 #include "int8_core.hpp"
 #include "offsets.hpp"
 #include <mutex>
+#include <atomic>
+#include <random>
 
 namespace pm {
+
+constexpr int STATIC_SCRATCH_DEVICES_MAX = 64;
 
 // tokens per work-group of the gate kernel = tokens per routing group (one lane each in the
 // routing epilogue): 64, or 32 on the split-K path (up to 16 experts) when 64 would leave
@@ -810,15 +814,108 @@ static int run_dispatch_routed(const void *x, int dtype, int samples, int model_
 
 } // namespace pm
 
+#include "forward_single.hpp"
+
+namespace pm {
+
+// every call gets a 64-bit ticket of its own: a random salt per process in the upper half, a
+// counter in the lower.  A group is "in" when its flag holds the call's ticket, so the flags need
+// no clearing between calls and whatever an uninitialised workspace holds does not pass for one.
+static unsigned long long next_ticket()
+{
+    static const unsigned long long salt = [] {
+        std::random_device rd;
+        return ((unsigned long long)rd() << 32) ^ 0x9e3779b900000000ull;
+    }();
+    static std::atomic<unsigned long long> count{0};
+    const unsigned long long c = count.fetch_add(1) + 1;
+    return (salt & 0xffffffff00000000ull) | (c & 0xffffffffull);
+}
+
+struct SingleShape { int nmma, rounds, groups; };
+
+// Whether the one-launch kernel serves the shape, and with how many rounds: model_dim 4096 bf16, up to
+// 16 experts, top_k <= 4, and so few tokens that every work-group is resident at once.
+template <int SDT, int CAP, int NMMA, int ROUNDS>
+static bool single_fits(int groups)
+{
+    static int resident[STATIC_SCRATCH_DEVICES_MAX] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_SCRATCH_DEVICES_MAX) return false;
+    if (resident[dev] == 0) {
+        int per_cu = 0, cus = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, forward_single_kernel<SDT, CAP, NMMA, ROUNDS>,
+                                                         FS_THREADS, 0) != hipSuccess) per_cu = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 0;
+        resident[dev] = per_cu * cus > 0 ? per_cu * cus : -1;
+    }
+    return groups <= resident[dev];
+}
+
+template <int SDT, int CAP, int NMMA>
+static int launch_single(int rounds, int groups, hipStream_t st, const void *x, const void *wg, const float *bias,
+                         int samples, int experts, int k, int normalize, int capacity, int32_t *indices,
+                         int32_t *locations, void *gates, int64_t stride, void *logits_out, void *scores_out,
+                         float *l_aux, int32_t *counts, uint8_t *codes, void *bias_out, void *scale_out, void *ws,
+                         int spin_limit, int32_t *gave_up)
+{
+    const unsigned long long ticket = next_ticket();
+#define PM_FS(ROUNDS)                                                                                     \
+    do {                                                                                                  \
+        if (!single_fits<SDT, CAP, NMMA, ROUNDS>(groups)) return 2;                                       \
+        forward_single_kernel<SDT, CAP, NMMA, ROUNDS><<<groups, FS_THREADS, 0, st>>>(                     \
+            (const uint4 *)x, (const uint4 *)wg, bias, samples, experts, k, normalize, capacity, indices, \
+            locations, gates, stride, logits_out, scores_out, l_aux, counts, codes, bias_out, scale_out,  \
+            ws, ticket, spin_limit, gave_up);                                                             \
+    } while (0)
+    switch (rounds) {
+    case 1: PM_FS(1); break;
+    case 2: PM_FS(2); break;
+    case 3: PM_FS(3); break;
+    default: PM_FS(4); break;
+    }
+#undef PM_FS
+    return 0;
+}
+
+// 0: launched; 2: the shape is not served by the one-launch kernel (nothing was enqueued)
+static int run_forward_single(const void *x, const void *wg, int dtype, int fp32_gate, const float *logit_bias,
+                              int samples, int model_dim, int experts, int top_k, int normalize_gate, int capacity,
+                              int32_t *indices, int32_t *locations, void *gates, int64_t stride, void *logits_out,
+                              void *scores_out, float *l_aux, int32_t *counts, uint8_t *codes, void *bias,
+                              void *scale, void *workspace, int spin_limit, int32_t *gave_up, hipStream_t st)
+{
+    const int k = top_k < experts ? top_k : experts;
+    if (dtype != PLANMOE_BF16 || model_dim != 4096 || experts > 16 || k > 4 || samples < 1) return 2;
+    if (!aligned16(codes) && capacity > 0) return 2;
+    int cus = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) return 2;
+    // as few tokens per work-group as it takes to put one work-group on every compute unit
+    const int rounds = (samples + 16 * cus - 1) / (16 * cus);
+    if (rounds > 4) return 2;
+    const int groups = (samples + 16 * rounds - 1) / (16 * rounds);
+#define PM_FS_ARGS rounds, groups, st, x, wg, logit_bias, samples, experts, k, normalize_gate, capacity, indices, \
+                   locations, gates, stride, logits_out, scores_out, l_aux, counts, codes, bias, scale, workspace,   \
+                   spin_limit, gave_up
+    if (fp32_gate) return experts <= 8 ? launch_single<PLANMOE_F32, 8, 16>(PM_FS_ARGS)
+                                       : launch_single<PLANMOE_F32, 16, 16>(PM_FS_ARGS);
+    return experts <= 8 ? launch_single<PLANMOE_BF16, 8, 16>(PM_FS_ARGS) : launch_single<PLANMOE_BF16, 16, 16>(PM_FS_ARGS);
+#undef PM_FS_ARGS
+}
+
+} // namespace pm
+
 using namespace pm;
 
 extern "C" size_t planmoe_forward_workspace_bytes(int samples, int experts, int top_k)
 {
     if (samples <= 0 || experts <= 0 || top_k <= 0) return 256;
     const size_t k = (size_t)(top_k < experts ? top_k : experts);
-    const size_t groups = ((size_t)samples + 31) / 32;      // upper bound over the group sizes
+    const size_t groups = ((size_t)samples + 15) / 16;      // upper bound over the group sizes
+    // + the status word and the 64-bit group tickets of the one-launch kernel
     return round_up(((size_t)experts + FWD_LOSS_PARTS + 2 * groups * k * experts + groups * experts +
-                     (k + 2) * (size_t)samples + (k + 1) * experts * fwd_pad4(groups)) * 4, 256);
+                     (k + 2) * (size_t)samples + (k + 1) * experts * fwd_pad4(groups)) * 4 + 32 + groups * 8, 256);
 }
 
 extern "C" int planmoe_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
@@ -870,12 +967,45 @@ extern "C" int planmoe_forward_int8(const void *x, const void *wg, int dtype, in
     return 0;
 }
 
+extern "C" int planmoe_forward_int8_single(const void *x, const void *wg, int dtype, int fp32_gate,
+                                           const float *logit_bias, int samples, int model_dim, int experts,
+                                           int top_k, int normalize_gate, int capacity, int32_t *indices,
+                                           int32_t *locations, void *gates, int64_t plane_stride,
+                                           void *logits_out, void *scores_out, float *l_aux,
+                                           int32_t *expert_counts, uint8_t *codes, void *bias, void *scale,
+                                           void *workspace, size_t workspace_bytes, int spin_limit,
+                                           int32_t *gave_up, void *stream)
+{
+    PM_REQUIRE(capacity >= 0 && (int64_t)experts * capacity < (1ll << 31), "planmoe_forward_int8_single: bad capacity");
+    if (fused_check("planmoe_forward_int8_single", x, wg, dtype, samples, model_dim, experts, top_k, plane_stride)) return 1;
+    PM_REQUIRE(indices && locations && gates, "planmoe_forward_int8_single: NULL routing output");
+    PM_REQUIRE((codes && bias && scale) || capacity == 0, "planmoe_forward_int8_single: NULL codec output");
+    PM_REQUIRE(workspace && workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
+               "planmoe_forward_int8_single: workspace too small");
+    PM_REQUIRE(spin_limit >= 0, "planmoe_forward_int8_single: spin_limit < 0");
+    const int rc = run_forward_single(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
+                                      normalize_gate, capacity, indices, locations, gates, plane_stride, logits_out,
+                                      scores_out, l_aux, expert_counts, codes, bias, scale, workspace,
+                                      spin_limit > 0 ? spin_limit : (1 << 20), gave_up, (hipStream_t)stream);
+    PM_REQUIRE(rc != 2, "planmoe_forward_int8_single: the one-launch kernel serves bf16 rows of 4096 values, up to 16 "
+               "experts, top_k <= 4 and at most 64 tokens per compute unit; use planmoe_forward_int8");
+    PM_LAUNCH_CHECK("planmoe_forward_int8_single");
+    return rc;
+}
+
+#ifdef PM_FS_TRACE
+extern "C" int planmoe_debug_fs_trace(unsigned long long *out_host)
+{
+    return hipMemcpyFromSymbol(out_host, HIP_SYMBOL(pm::fs_trace), sizeof(unsigned long long) * 1024 * 16) != hipSuccess;
+}
+#endif
+
 // ---- the same entry point for callers that can allocate nothing: its workspace is a file-scope
 // array in device memory.  Host code must not hand `static_scratch` itself to a kernel (on the
 // host the name is a stand-in, not a device address): the address is asked for once per device
 // and kept.
 constexpr size_t STATIC_SCRATCH_BYTES = (size_t)4 << 20;
-constexpr int STATIC_SCRATCH_DEVICES = 64;
+constexpr int STATIC_SCRATCH_DEVICES = STATIC_SCRATCH_DEVICES_MAX;
 static __device__ __align__(256) unsigned char static_scratch[STATIC_SCRATCH_BYTES];
 static void *g_static_scratch[STATIC_SCRATCH_DEVICES];
 static std::mutex g_static_scratch_lock;

@@ -434,6 +434,28 @@ def forward_int8(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, norma
     return out
 
 
+def forward_int8_single(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
+                        want_logits=False, want_scores=False, want_l_aux=True, want_counts=False, spin_limit=0):
+    """forward_int8 in one launch that reads x once (bf16 rows of 4096 values, up to 16 experts,
+    top_k <= 4, at most 64 tokens per compute unit; anything else raises).  Adds `gave_up`, a device
+    int32 that is 1 when a work-group ran out of `spin_limit` polls waiting for the others."""
+    x, wg, T, M, E, k, bias, out, ws = _forward_common(x, wg, top_k, fp32_gate, logit_bias, want_logits,
+                                                       want_scores, want_l_aux, want_counts)
+    R = E * capacity_
+    out["codes"] = torch.empty((R, M), dtype=torch.uint8, device=x.device)
+    out["bias"] = torch.empty((R, 1), dtype=x.dtype, device=x.device)
+    out["scale"] = torch.empty((R, 1), dtype=x.dtype, device=x.device)
+    out["gave_up"] = torch.zeros((), dtype=torch.int32, device=x.device)
+    check(lib.planmoe_forward_int8_single(_ptr(x), _ptr(wg), _dt(x, "forward_int8_single"), int(bool(fp32_gate)),
+                                          _ptr(bias), T, M, E, k, int(bool(normalize_gate)), capacity_,
+                                          _ptr(out["indices"]), _ptr(out["locations"]), _ptr(out["gates"]), max(T, 1),
+                                          _ptr(out["logits"]), _ptr(out["scores"]), _ptr(out["l_aux"]),
+                                          _ptr(out["counts"]), _ptr(out["codes"]), _ptr(out["bias"]),
+                                          _ptr(out["scale"]), _ptr(ws), ws.numel(), int(spin_limit),
+                                          _ptr(out["gave_up"]), _stream(x)))
+    return out
+
+
 def forward_int8_static(x, wg, top_k, capacity_, out, fp32_gate=True, logit_bias=None, normalize_gate=True):
     """forward_int8 through the entry point that allocates nothing: the workspace is the library's
     built-in device buffer and every output is the caller's (`out`: the dict of tensors a

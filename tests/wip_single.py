@@ -1,0 +1,56 @@
+"""planmoe_forward_int8_single (one launch, x read once) against the oracle and the two-launch chain."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import np_raw, raw
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("T,E,k,cf,fp32_gate", [(16384, 8, 2, 1.25, True), (16384, 8, 2, 1.25, False), (16000, 8, 2, 1.25, True),
+                                                (4096, 8, 2, 1.0, True), (100, 4, 2, 1.0, True), (9000, 16, 3, 0.5, True),
+                                                (12288, 8, 1, 1.0, True), (5000, 12, 4, 2.0, False), (1, 3, 2, 1.0, True)])
+def test_single_launch_forward(T, E, k, cf, fp32_gate):
+    from planmoe_amd import ops
+    M = 4096
+    print("case", T, E, k, cf, fp32_gate, flush=True)
+    g = torch.Generator().manual_seed(T + E)
+    x = torch.randn(T, M, generator=g).bfloat16().to(DEV)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
+    C = ops.capacity(T, E, k, cf, 4)
+    out = ops.forward_int8_single(x, wg, k, C, fp32_gate=fp32_gate, want_scores=True, want_counts=True, want_logits=True)
+    torch.cuda.synchronize()
+    assert int(out["gave_up"]) == 0
+    scores = out["scores"].float().cpu().numpy() if fp32_gate else None
+    if fp32_gate:
+        idx, loc, gates, counts = oracle.route_topk(scores, k)
+    else:
+        from helpers import bf16_bits
+        idx, loc, gates, counts = oracle.route_topk(bf16_bits(out["scores"]), k)
+    assert np.array_equal(out["indices"].cpu().numpy(), idx)
+    assert np.array_equal(out["locations"].cpu().numpy(), loc)
+    assert np.array_equal(raw(out["gates"]), np_raw(gates))
+    assert np.array_equal(out["counts"].cpu().numpy(), counts)
+    ref = ops.forward_int8(x, wg, k, C, fp32_gate=fp32_gate, want_scores=True, want_logits=True)
+    assert torch.allclose(out["logits"].float(), ref["logits"].float(), rtol=1e-2 if not fp32_gate else 1e-5, atol=1e-5)
+    want = oracle.gshard_loss(out["scores"].float().cpu().numpy(), idx[0])
+    assert abs(float(out["l_aux"]) - want) <= 1e-5 * abs(want)
+    c2, b2, s2 = ops.dispatch_int8(x, list(out["indices"]), list(out["locations"]), None, E, C)
+    assert torch.equal(out["codes"].view(-1), c2.view(-1))
+    assert np.array_equal(raw(out["bias"]).reshape(-1), raw(b2).reshape(-1))
+    assert np.array_equal(raw(out["scale"]).reshape(-1), raw(s2).reshape(-1))
+
+
+def test_single_launch_gives_up_cleanly_when_told_to():
+    """spin_limit = 1 with more than one group: some group finds the others not in yet, gives up,
+    writes none of its rows and raises the flag; every work-group still exits."""
+    from planmoe_amd import ops
+    T, M, E, k = 16384, 4096, 8, 2
+    x = torch.randn(T, M, device=DEV).bfloat16()
+    wg = (torch.randn(E, M, device=DEV) * M ** -0.5).bfloat16()
+    out = ops.forward_int8_single(x, wg, k, 5120, spin_limit=1)
+    torch.cuda.synchronize()
+    assert int(out["gave_up"]) in (0, 1)
