@@ -818,9 +818,10 @@ static int run_dispatch_routed(const void *x, int dtype, int samples, int model_
 
 namespace pm {
 
-// every call gets a 64-bit ticket of its own: a random salt per process in the upper half, a
-// counter in the lower.  A group is "in" when its flag holds the call's ticket, so the flags need
-// no clearing between calls and whatever an uninitialised workspace holds does not pass for one.
+// every call draws a 64-bit ticket: a random salt per process in the upper half, a counter in the
+// lower.  The kernel mixes it into the tag of the words its work-groups publish (the other part is
+// the workspace's own launch counter), so that what an uninitialised workspace holds, or another
+// process left behind, does not pass for a word of this launch.
 static unsigned long long next_ticket()
 {
     static const unsigned long long salt = [] {
@@ -895,6 +896,7 @@ static int run_forward_single(const void *x, const void *wg, int dtype, int fp32
     const int rounds = (samples + 16 * cus - 1) / (16 * cus);
     if (rounds > 4) return 2;
     const int groups = (samples + 16 * rounds - 1) / (16 * rounds);
+    if (groups > FS_MAX_GROUPS) return 2;
 #define PM_FS_ARGS rounds, groups, st, x, wg, logit_bias, samples, experts, k, normalize_gate, capacity, indices, \
                    locations, gates, stride, logits_out, scores_out, l_aux, counts, codes, bias, scale, workspace,   \
                    spin_limit, gave_up
@@ -913,9 +915,11 @@ extern "C" size_t planmoe_forward_workspace_bytes(int samples, int experts, int 
     if (samples <= 0 || experts <= 0 || top_k <= 0) return 256;
     const size_t k = (size_t)(top_k < experts ? top_k : experts);
     const size_t groups = ((size_t)samples + 15) / 16;      // upper bound over the group sizes
-    // + the status word and the 64-bit group tickets of the one-launch kernel
-    return round_up(((size_t)experts + FWD_LOSS_PARTS + 2 * groups * k * experts + groups * experts +
-                     (k + 2) * (size_t)samples + (k + 1) * experts * fwd_pad4(groups)) * 4 + 32 + groups * 8, 256);
+    const size_t tables = ((size_t)experts + FWD_LOSS_PARTS + 2 * groups * k * experts + groups * experts +
+                           (k + 2) * (size_t)samples + (k + 1) * experts * fwd_pad4(groups)) * 4;
+    // the one-launch kernel keeps the words its work-groups publish in the same space
+    const size_t published = fs_pub_bytes((int)(groups < (size_t)FS_MAX_GROUPS ? groups : (size_t)FS_MAX_GROUPS));
+    return round_up(tables > published ? tables : published, 256);
 }
 
 extern "C" int planmoe_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,

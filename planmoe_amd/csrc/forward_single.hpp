@@ -3,14 +3,24 @@
 // A work-group of 8 waves owns 16 * ROUNDS consecutive tokens and there is one work-group per
 // compute unit, all resident together.  Phase 1 streams the tokens in rounds of 16 (one MFMA
 // M-tile): gate GEMM split-K over the 8 waves, row min / max on the way, softmax / top-k of the
-// round.  A row can be quantised as soon as its own min / max are known, so the rows of the first
-// rounds are turned into codes at once and parked in LDS; the last two rounds simply stay in the
-// registers they were loaded into.  Then the group's expert histogram is published and the
-// work-group waits until every group has done so (the slot of a second choice needs the number of
-// first choices of the whole batch).  Phase 2 adds up the histogram columns it needs, once per
-// work-group, and writes every parked row to its slots straight from LDS in full 4 KB rows, the
-// register rounds being quantised (while the first stores drain) and passed through the same LDS
-// rows; empty slots are zero-filled by all work-groups together.
+// round.  A row can be quantised as soon as its own min / max are known, so every round is turned
+// into codes right away, while the loads of the next rounds are in flight: the codes of the first
+// rounds are parked in LDS, those of the last two stay in registers.  Then the group publishes
+// its expert histogram and waits until every group has done so (the slot of a second choice needs
+// the first-choice counts of the whole batch); the last round is quantised during that wait.
+// Phase 2 only stores: every parked row goes to its slots in full 4 KB rows from LDS (the register
+// rounds pass through the same LDS rows), empty slots are zero-filled by all work-groups together.
+//
+// What the groups tell each other travels in 64-bit words that carry their own validity: the
+// upper half is the launch's tag, the lower half four 8-bit counts (or one float of the score
+// sums).  A word is written by one atomic store and read by one atomic load, so there is no
+// ordering between words to enforce, no cache write-back or invalidation, and nothing to clear
+// between launches: a word of an earlier launch, or whatever an uninitialised workspace holds,
+// does not carry the tag.  The tag is the workspace's launch counter + 1 (mixed with a ticket the
+// host draws per call).  Every work-group reads the counter first thing; the last group stores
+// counter + 1 at its very end, by when every group has published, hence started, hence read the
+// old value.  So the counter needs no initial value, and replays of a captured launch, whose
+// arguments never change, still get a tag of their own each.
 //
 // Replaces gates/top.py:20-26 + moe_layer.py:230-256 + fast_dispatch.py:140-201 +
 // Int8Compressor::compress (int8.cpp:7-44), like the two-launch chain.
@@ -26,27 +36,34 @@ __device__ unsigned long long fs_trace[1024 * 16];
 #define FS_STAMP(i) do { } while (0)
 #endif
 
+#ifdef PM_FS_NT_LOADS
+#define FS_LOAD(p) stream_load(p)
+#else
+#define FS_LOAD(p) (*(p))
+#endif
+
+#ifdef PM_FS_FENCE
+#define FS_SCHED_FENCE __builtin_amdgcn_sched_barrier(0)
+#else
+#define FS_SCHED_FENCE do { } while (0)
+#endif
+
+#ifndef FS_SPLIT
+#define FS_SPLIT 1
+#endif
+
 constexpr int FS_WAVES = 8;
 constexpr int FS_THREADS = FS_WAVES * WAVE;
+constexpr int FS_MAX_GROUPS = 512;          // work-groups the published tables are sized for
 
 // waits for LDS traffic only: loads and stores to global memory that are in flight stay in flight
 // across the barrier (__syncthreads would drain them)
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// per-group tickets and the status word live behind the tables of the two-launch chain
-struct FsSync {
-    unsigned long long *flags;      // [groups]: the ticket of the call whose histogram row is complete
-    uint32_t *status;               // [0]: ticket (low word) of a call that gave up waiting
-};
-__host__ __device__ inline FsSync fs_sync(const FwdWs &w, int samples)
-{
-    FsSync s;
-    uintptr_t p = (uintptr_t)(w.row_max + samples);
-    p = (p + 15) & ~(uintptr_t)15;
-    s.status = (uint32_t *)p;
-    s.flags = (unsigned long long *)(p + 16);
-    return s;
-}
+// the one-launch kernel's part of the workspace: the launch counter, then from byte 256 the
+// published words hist[groups][CAP] (4 planes x CAP experts, four counts per word), me[groups][CAP]
+constexpr size_t FS_PUB_OFFSET = 256;
+__host__ __device__ inline size_t fs_pub_bytes(int groups) { return FS_PUB_OFFSET + (size_t)groups * (16 + 16) * 8; }
 
 template <int NMMA> struct FsGeom {
     static constexpr int M = 256 * NMMA;          // model_dim: every wave owns M / 8 elements of a row
@@ -55,6 +72,13 @@ template <int NMMA> struct FsGeom {
                                                   // rows fall into different banks
     static constexpr int RV = M / 16 / WAVE;      // 16-byte pieces of a code row per lane
 };
+
+// four 8-bit counts -> four 16-bit fields (sums over up to 512 groups of counts up to 64 fit)
+__device__ __forceinline__ unsigned long long fs_spread(uint32_t p)
+{
+    return (unsigned long long)(p & 0xffu) | ((unsigned long long)(p & 0xff00u) << 8) |
+           ((unsigned long long)(p & 0xff0000u) << 16) | ((unsigned long long)(p >> 24) << 48);
+}
 
 template <int SDT, int CAP, int NMMA, int ROUNDS>
 __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
@@ -73,65 +97,49 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
     static_assert(ROUNDS >= 1 && ROUNDS <= 4, "one lane per token in the ranking step");
     static_assert(NMMA % 4 == 0 && G::RV >= 1, "rows are dealt out in 16-byte pieces");
     constexpr int TOK = 16 * ROUNDS;
-    constexpr int REG_ROUNDS = ROUNDS < 2 ? ROUNDS : 2;    // the last rounds stay raw in registers
-    constexpr int LDS_ROUNDS = ROUNDS - REG_ROUNDS;        // the first rounds are parked as codes
+    constexpr int REG_ROUNDS = ROUNDS < 2 ? ROUNDS : 2;    // the last rounds keep their codes in registers
+    constexpr int LDS_ROUNDS = ROUNDS - REG_ROUNDS;        // the first rounds park theirs in LDS
     constexpr int PARK_ROUNDS = LDS_ROUNDS > REG_ROUNDS ? LDS_ROUNDS : REG_ROUNDS;
+    constexpr int HW = CAP;                                // published histogram words per group: 4 planes x CAP / 4
     __shared__ __align__(16) uint8_t park[PARK_ROUNDS * 16 * G::RS];
     __shared__ float part[2][FS_WAVES][16][CAP + 1];
     __shared__ int32_t pstat[2][FS_WAVES][16][3];
     __shared__ uint8_t s_best[4][TOK];
     __shared__ int32_t s_rank[4][TOK];
     __shared__ float s_mn[TOK], s_sc[TOK];
-    __shared__ float s_me[ROUNDS][CAP];
-    __shared__ int32_t s_hist[CAP];
-    __shared__ int32_t s_part[4][CAP], s_full[4][CAP];     // histogram columns: groups before this one / all
-    __shared__ int32_t s_base[4][CAP], s_tot[CAP];
-    __shared__ float s_loss[CAP];
-    __shared__ int s_fail;
+    __shared__ float s_logit[TOK][CAP + 1];
+    constexpr int RPASSES = (TOK * CAP + FS_THREADS - 1) / FS_THREADS;       // routing passes of the 8 waves
+    __shared__ float s_me[RPASSES * FS_WAVES][CAP];
+    __shared__ int32_t s_hist[4][CAP];
+    __shared__ unsigned long long s_before64[HW], s_full64[HW];
+    __shared__ int32_t s_full[4][CAP], s_base[4][CAP], s_tot[CAP];
+    __shared__ float s_mepart[FS_THREADS / CAP][CAP];
+    __shared__ int s_vote[2][FS_WAVES];
 
     const int tid = threadIdx.x, w = tid >> 6, lane = lane_id(), m = lane & 15, g = lane >> 4;
     const int groups = gridDim.x, grp = blockIdx.x, t0 = grp * TOK;
-    const FwdWs ws = fwd_ws(workspace, groups, k, experts, samples);
-    const FsSync sync = fs_sync(ws, samples);
+    unsigned long long *launches = reinterpret_cast<unsigned long long *>(workspace);
+    unsigned long long *pub_hist = reinterpret_cast<unsigned long long *>((char *)workspace + FS_PUB_OFFSET);
+    unsigned long long *pub_me = pub_hist + (size_t)groups * HW;
+    const unsigned long long launch = __hip_atomic_load(launches, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+    const uint32_t tag = (uint32_t)launch ^ (uint32_t)(ticket ^ (ticket >> 32));
     const float eps = SDT == PLANMOE_F32 ? 1.1920928955078125e-07f : SDT == PLANMOE_BF16 ? 0.0078125f : 0.0009765625f;
+    if (tid < HW) { s_before64[tid] = 0; s_full64[tid] = 0; }
 
     // lane (m, g) of wave w holds, of row m of a round, the vectors  w * 4 NMMA + 4 i + g
     const int v0 = w * (4 * NMMA) + g;
     const uint4 *bp = wg + (int64_t)min(m, experts - 1) * G::NV + v0;
-    auto load_x = [&](uint4 (&a)[NMMA], int r) {
-        const uint4 *p = x + (int64_t)min(t0 + 16 * r + m, samples - 1) * G::NV + v0;
-#pragma unroll
-        for (int i = 0; i < NMMA; ++i) a[i] = p[4 * i];
-    };
-    // codes of this lane's share of row `row` of the parking area
-    auto encode_to_park = [&](const uint4 (&a)[NMMA], int row, float mn, float scale) {
-        const RowEncoder<PLANMOE_BF16> enc(mn, scale);
-        uint8_t *dst = park + row * G::RS + v0 * 8;
-        auto body = [&](auto mode) {
-#pragma unroll
-            for (int i = 0; i < NMMA; ++i) {
-                uint32_t wd[2];
-                enc.template encode<decltype(mode)::value>(a[i], wd);
-                *reinterpret_cast<uint2 *>(dst + 32 * i) = make_uint2(wd[0], wd[1]);
-            }
-        };
-        // the mode is a property of the row, i.e. of the lane here: one branch for the wave
-        if (__ballot(!enc.rq.fast) == 0) body(std::true_type{}); else body(std::false_type{});
-    };
+    auto row_ptr = [&](int r) { return x + (int64_t)min(t0 + 16 * r + m, samples - 1) * G::NV + v0; };
+    uint8_t *my_park = park + m * G::RS + v0 * 8;          // this lane's 8 bytes of vector 0 in parked row m
 
     uint4 buf0[NMMA], buf1[NMMA];
-    float keep_mn[2] = {0.f, 0.f}, keep_sc[2] = {0.f, 0.f};       // row min / scale of the rows left in buf0 / buf1
+    uint4 b[NMMA];                                         // this wave's K range of the gate weights, loaded once
+    uint2 kept[REG_ROUNDS][NMMA];                          // codes of the last rounds (phase 2)
 
-    // ---- one round: GEMM + row statistics of 16 tokens, their routing, codes of the early rounds
-    auto round = [&](auto rc, uint4 (&cur)[NMMA], uint4 (&nxt)[NMMA]) {
+    // ---- one round: GEMM + row statistics of 16 tokens, their logits, the codes of the early rounds
+    auto round = [&](auto rc, uint4 (&cur)[NMMA]) {
         constexpr int r = decltype(rc)::value;
         constexpr int par = r & 1;
-        // gate weights of this wave's K range first, then the next round's rows: the MFMAs below
-        // wait for the weights only, the rows stay in flight behind them
-        uint4 b[NMMA];
-#pragma unroll
-        for (int i = 0; i < NMMA; ++i) b[i] = bp[4 * i];
-        if constexpr (r + 1 < ROUNDS) load_x(nxt, r + 1);
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
         RowStats<PLANMOE_BF16, true> st;
         st.init();
@@ -155,7 +163,9 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i) part[par][w][4 * g + i][m] = acc[i];
         }
+        if constexpr (r == 1) FS_STAMP(13);
         lds_barrier();
+        if constexpr (r == 1) FS_STAMP(14);
 
         // min / max of this lane's row over the 8 K ranges
         float mn, mx;
@@ -170,174 +180,238 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
         const float scale = B16::round(mx - mn);
         if (w == 0 && g == 0) { s_mn[16 * r + m] = mn; s_sc[16 * r + m] = scale; }
 
-        // routing of the round's 16 tokens by one wave: CAP lanes share a token, lane el holds expert el
-        if (w == (r + 1) % FS_WAVES) {
-            constexpr int LPT = CAP, TPP = WAVE / LPT;
-            const int el = lane % LPT, tk = lane / LPT;
-            auto token_reduce = [&](auto v, auto op) { return row_allreduce<LPT>(v, op); };
-            float me_acc = 0.f;
+        // logits of the round: the 8 partial sums of every (token, expert), added in wave order
+        if (tid < 16 * CAP) {
+            const int tok16 = tid / CAP, e = tid % CAP;
+            float v = part[par][0][tok16][e];
 #pragma unroll
-            for (int p = 0; p < 16 / TPP; ++p) {
-                const int tok16 = p * TPP + tk, tok = 16 * r + tok16, t = t0 + tok;
-                const bool valid = t < samples;
-                float v = -INFINITY;
-                if (el < experts) {
-                    v = part[par][0][tok16][el];
-#pragma unroll
-                    for (int ww = 1; ww < FS_WAVES; ++ww) v += part[par][ww][tok16][el];
-                    v = S::round(v);
-                    if (logits_out && valid) S::store(logits_out, (int64_t)t * experts + el, v);
-                    if (logit_bias) v = S::round(v + logit_bias[el]);
-                }
-                const float mxl = token_reduce(v, [](float a, float c) { return fmaxf(a, c); });
-                float sc = el < experts ? expf(v - mxl) : 0.f;
-                const float sum = token_reduce(sc, [](float a, float c) { return a + c; });
-                const float inv = 1.0f / sum;
-                if (el < experts) {
-                    sc = S::round(sc * inv);
-                    if (scores_out && valid) S::store(scores_out, (int64_t)t * experts + el, sc);
-                } else {
-                    sc = -INFINITY;
-                }
-                if (l_aux) {
-                    float c = (valid && el < experts) ? sc : 0.f;
-#pragma unroll
-                    for (int off = LPT; off < WAVE; off <<= 1) c += __shfl_xor(c, off, WAVE);
-                    me_acc += c;
-                }
-                // k-fold arg-max, the lower expert id wins among equal scores
-                bool taken = false;
-                float denom = 0.f, my_gate = 0.f;
-                int my_idx = 0;
-                for (int j = 0; j < k; ++j) {
-                    float bv = -INFINITY; int bi = 0x7fffffff;
-                    if (!taken && el < experts) { bv = sc; bi = el; }
-                    auto merge = [&](float ov, int oi) {
-                        const bool better = oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi));
-                        if (better) { bv = ov; bi = oi; }
-                    };
-                    merge(row_partner<1>(bv), row_partner<1>(bi));
-                    merge(row_partner<2>(bv), row_partner<2>(bi));
-                    merge(row_partner<4>(bv), row_partner<4>(bi));
-                    if constexpr (LPT >= 16) merge(row_partner<8>(bv), row_partner<8>(bi));
-                    if (bi == el) taken = true;
-                    denom = (j == 0) ? bv : S::round(denom + bv);
-                    if (el == 0) s_best[j][tok] = (uint8_t)bi;
-                    if (el == j) { my_gate = bv; my_idx = bi; }
-                }
-                if (valid && el < k) {
-                    const bool norm = k > 1 && normalize_gate;
-                    const float d = fmaxf(denom, eps);
-                    indices[(int64_t)el * stride + t] = my_idx;
-                    S::store(gates, (int64_t)el * stride + t, norm ? my_gate / d : my_gate);
-                }
-            }
-            if (l_aux && tk == 0 && el < experts) s_me[r][el] = me_acc;
+            for (int ww = 1; ww < FS_WAVES; ++ww) v += part[par][ww][tok16][e];
+            s_logit[16 * r + tok16][e] = v;
         }
 
+        // codes of the early rounds go to LDS, then their registers take the row two rounds ahead.
+        // The last rounds stay in their registers as they are and are
+        // coded in phase 2, under the stores.  The mode is a property of the row, i.e. of the lane
+        // here: one branch for the wave.
         if constexpr (r < LDS_ROUNDS) {
-            encode_to_park(cur, r * 16 + m, mn, scale);
-        } else {
-            keep_mn[par] = mn; keep_sc[par] = scale;
+            const RowEncoder<PLANMOE_BF16> enc(mn, scale);
+            const uint4 *ahead = row_ptr(r + 2);
+            auto body = [&](auto mode) {
+#pragma unroll
+                for (int h = 0; h < FS_SPLIT; ++h) {
+#pragma unroll
+                    for (int i = h * (NMMA / FS_SPLIT); i < (h + 1) * (NMMA / FS_SPLIT); ++i) {
+                        uint32_t wd[2];
+                        enc.template encode<decltype(mode)::value>(cur[i], wd);
+                        *reinterpret_cast<uint2 *>(my_park + r * 16 * G::RS + 32 * i) = make_uint2(wd[0], wd[1]);
+                    }
+                    // the half just coded takes its share of the row two rounds ahead
+                    FS_SCHED_FENCE;
+#pragma unroll
+                    for (int i = h * (NMMA / FS_SPLIT); i < (h + 1) * (NMMA / FS_SPLIT); ++i) cur[i] = FS_LOAD(ahead + 4 * i);
+                    FS_SCHED_FENCE;
+                }
+            };
+            if (__ballot(!enc.rq.fast) == 0) body(std::true_type{}); else body(std::false_type{});
         }
     };
 
     FS_STAMP(0);
-    load_x(buf0, 0);
-    round(std::integral_constant<int, 0>{}, buf0, buf1);
+    {
+        const uint4 *p0 = row_ptr(0), *p1 = row_ptr(ROUNDS > 1 ? 1 : 0);
+#pragma unroll
+        for (int i = 0; i < NMMA; ++i) buf0[i] = FS_LOAD(p0 + 4 * i);
+#pragma unroll
+        for (int i = 0; i < NMMA; ++i) b[i] = bp[4 * i];
+        if constexpr (ROUNDS > 1) {
+#pragma unroll
+            for (int i = 0; i < NMMA; ++i) buf1[i] = FS_LOAD(p1 + 4 * i);
+        }
+    }
+    round(std::integral_constant<int, 0>{}, buf0);
     FS_STAMP(1);
-    if constexpr (ROUNDS > 1) round(std::integral_constant<int, 1>{}, buf1, buf0);
+    if constexpr (ROUNDS > 1) round(std::integral_constant<int, 1>{}, buf1);
     FS_STAMP(2);
-    if constexpr (ROUNDS > 2) round(std::integral_constant<int, 2>{}, buf0, buf1);
+    if constexpr (ROUNDS > 2) round(std::integral_constant<int, 2>{}, buf0);
     FS_STAMP(3);
-    if constexpr (ROUNDS > 3) round(std::integral_constant<int, 3>{}, buf1, buf0);
+    if constexpr (ROUNDS > 3) round(std::integral_constant<int, 3>{}, buf1);
+    lds_barrier();
+
+    // ---- routing of the group's tokens by all waves at once: CAP lanes share a token, lane el
+    // holds expert el; softmax and the k-fold arg-max are butterflies over those lanes
+    {
+        constexpr int LPT = CAP, TPP = WAVE / LPT;
+        const int el = lane % LPT, tk = lane / LPT;
+        auto token_reduce = [&](auto v, auto op) { return row_allreduce<LPT>(v, op); };
+#pragma unroll
+        for (int p = 0; p < RPASSES; ++p) {
+            const int tok = min((p * FS_WAVES + w) * TPP + tk, TOK - 1), t = t0 + tok;
+            const bool valid = (p * FS_WAVES + w) * TPP + tk < TOK && t < samples;
+            float v = -INFINITY;
+            if (el < experts) {
+                v = S::round(s_logit[tok][el]);
+                if (logits_out && valid) S::store(logits_out, (int64_t)t * experts + el, v);
+                if (logit_bias) v = S::round(v + logit_bias[el]);
+            }
+            const float mxl = token_reduce(v, [](float a, float c) { return fmaxf(a, c); });
+            float sc = el < experts ? expf(v - mxl) : 0.f;
+            const float sum = token_reduce(sc, [](float a, float c) { return a + c; });
+            const float inv = 1.0f / sum;
+            if (el < experts) {
+                sc = S::round(sc * inv);
+                if (scores_out && valid) S::store(scores_out, (int64_t)t * experts + el, sc);
+            } else {
+                sc = -INFINITY;
+            }
+            if (l_aux) {
+                float c = (valid && el < experts) ? sc : 0.f;
+#pragma unroll
+                for (int off = LPT; off < WAVE; off <<= 1) c += __shfl_xor(c, off, WAVE);
+                if (tk == 0) s_me[p * FS_WAVES + w][el] = c;
+            }
+            // k-fold arg-max, the lower expert id wins among equal scores
+            bool taken = false;
+            float denom = 0.f, my_gate = 0.f;
+            int my_idx = 0;
+            for (int j = 0; j < k; ++j) {
+                float bv = -INFINITY; int bi = 0x7fffffff;
+                if (!taken && el < experts) { bv = sc; bi = el; }
+                auto merge = [&](float ov, int oi) {
+                    const bool better = oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi));
+                    if (better) { bv = ov; bi = oi; }
+                };
+                merge(row_partner<1>(bv), row_partner<1>(bi));
+                merge(row_partner<2>(bv), row_partner<2>(bi));
+                merge(row_partner<4>(bv), row_partner<4>(bi));
+                if constexpr (LPT >= 16) merge(row_partner<8>(bv), row_partner<8>(bi));
+                if (bi == el) taken = true;
+                denom = (j == 0) ? bv : S::round(denom + bv);
+                if (el == 0 && valid) s_best[j][tok] = (uint8_t)bi;
+                if (el == j) { my_gate = bv; my_idx = bi; }
+            }
+            if (valid && el < k) {
+                const bool norm = k > 1 && normalize_gate;
+                const float d = fmaxf(denom, eps);
+                indices[(int64_t)el * stride + t] = my_idx;
+                S::store(gates, (int64_t)el * stride + t, norm ? my_gate / d : my_gate);
+            }
+        }
+    }
     lds_barrier();
     FS_STAMP(4);
 
-    // ---- the group's ranks and histogram (wave 0, one lane per token), then its ticket
+    // ---- the group's ranks and histogram (wave 0, one lane per token), published at once
     if (w == 0) {
         const bool valid = lane < TOK && t0 + lane < samples;
-        for (int j = 0; j < k; ++j) {
-            const int best = valid ? (int)s_best[j][lane % TOK] : -1;
+        for (int j = 0; j < 4; ++j) {
+            const int best = (valid && j < k) ? (int)s_best[j][lane % TOK] : -1;
             int rank = 0;
 #pragma unroll
             for (int e = 0; e < CAP; ++e) {
                 const uint64_t mk = __ballot(best == e);
                 if (best == e) rank = __popcll(mk & lanes_below());
-                if (lane == e) s_hist[e] = __popcll(mk);
+                if (lane == e) s_hist[j][e] = __popcll(mk);
             }
             if (lane < TOK) s_rank[j][lane] = rank;
-            __builtin_amdgcn_wave_barrier();
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (lane < HW) {
+            const int32_t *h = &s_hist[0][0] + 4 * lane;
+            const uint32_t payload = (uint32_t)h[0] | ((uint32_t)h[1] << 8) | ((uint32_t)h[2] << 16) | ((uint32_t)h[3] << 24);
+            __hip_atomic_store(pub_hist + (size_t)grp * HW + lane, ((unsigned long long)tag << 32) | payload,
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (l_aux && lane < CAP) {
+            float v = 0.f;
             if (lane < experts) {
-                int32_t *col = ws.hist_t + ((int64_t)j * experts + lane) * ws.gstride;
-                col[grp] = s_hist[lane];
-                if (grp == groups - 1)
-                    for (int p = groups; p < ws.gstride; ++p) col[p] = 0;
-            }
-            __builtin_amdgcn_wave_barrier();
-        }
-        if (l_aux && lane < experts) {
-            float v = s_me[0][lane];
+                v = s_me[0][lane];
 #pragma unroll
-            for (int r = 1; r < ROUNDS; ++r) v += s_me[r][lane];
-            ws.me_t[(int64_t)lane * ws.gstride + grp] = v;
-            if (grp == groups - 1)
-                for (int p = groups; p < ws.gstride; ++p) ws.me_t[(int64_t)lane * ws.gstride + p] = 0.f;
+                for (int i = 1; i < RPASSES * FS_WAVES; ++i) v += s_me[i][lane];
+            }
+            __hip_atomic_store(pub_me + (size_t)grp * CAP + lane, ((unsigned long long)tag << 32) | __float_as_uint(v),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        __threadfence();
-        FS_STAMP(5);
-        if (lane == 0) __hip_atomic_store(sync.flags + grp, ticket, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-
-        // every group's ticket must be in before any slot is final; the wait is bounded
-        bool all = false;
-        for (int spin = 0; spin <= spin_limit; ++spin) {
-            bool ok = true;
-            for (int i = lane; i < groups; i += WAVE)
-                ok = ok && __hip_atomic_load(sync.flags + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ticket;
-            all = __ballot(!ok) == 0;
-            if (all) break;
-            __builtin_amdgcn_s_sleep(4);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        if (lane == 0) s_fail = all ? 0 : 1;
     }
-    lds_barrier();
+    FS_STAMP(5);
+
     FS_STAMP(6);
-    if (s_fail) {
-        // not every group showed up in time: none of this group's rows is written
-        if (tid == 0) {
-            __hip_atomic_store(sync.status, (uint32_t)ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (gave_up) __hip_atomic_store(gave_up, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    // ---- every group's histogram must be in before any slot is final.  Thread (gi, q) reads word q
+    // of the groups gi, gi + GPP, ...; a word counts once its tag is the call's.  The wait is bounded.
+    constexpr int GPP = FS_THREADS / HW;                   // groups per pass
+    constexpr int PASSES = (FS_MAX_GROUPS + GPP - 1) / GPP;
+    const int q = tid % HW, gi = tid / HW;
+    const bool active = 4 * q < k * CAP;                   // words of planes past top_k hold no counts
+    unsigned long long word[PASSES];
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) word[p] = (unsigned long long)tag << 32;
+    bool all = false;
+    for (int spin = 0; spin <= spin_limit; ++spin) {
+        bool ok = true;
+        if (active) {
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                if (p * GPP < groups) {
+                    const int gg = min(gi + p * GPP, groups - 1);
+                    word[p] = __hip_atomic_load(pub_hist + (size_t)gg * HW + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) ok = ok && (uint32_t)(word[p] >> 32) == tag;
         }
+        const int slot = spin & 1;
+        const int wave_bad = __ballot(!ok) != 0;             // (taken by all lanes: a ballot sees active lanes only)
+        if (lane == 0) s_vote[slot][w] = wave_bad;
+        lds_barrier();
+        int bad = 0;
+#pragma unroll
+        for (int ww = 0; ww < FS_WAVES; ++ww) bad |= s_vote[slot][ww];
+        all = bad == 0;
+        if (all) break;
+        __builtin_amdgcn_s_sleep(8);
+    }
+    FS_STAMP(7);
+    if (!all) {
+        // not every group showed up in time: none of this group's rows is written
+        if (tid == 0 && gave_up) __hip_atomic_store(gave_up, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0 && grp == groups - 1) __hip_atomic_store(launches, launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return;
     }
 
-    // ---- phase 2.  Histogram columns: entries of the groups before this one, and of all groups
-    for (int item = w; item < k * experts; item += FS_WAVES) {
-        const int32_t *col = ws.hist_t + (int64_t)item * ws.gstride;
-        int before = 0, full = 0;
-        for (int i = lane * 4; i < groups; i += 4 * WAVE) {
-            const int4 v = *reinterpret_cast<const int4 *>(col + i);
-            const int vv[4] = {v.x, v.y, v.z, v.w};
+    // entries of the groups before this one, and of all groups, for every (plane, expert)
+    {
+        unsigned long long before = 0, full = 0;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                if (i + c < groups) full += vv[c];
-                if (i + c < grp) before += vv[c];
-            }
+        for (int p = 0; p < PASSES; ++p) {
+            const int gg = gi + p * GPP;
+            const unsigned long long sp = fs_spread((uint32_t)word[p]);
+            if (gg < groups) full += sp;
+            if (gg < grp) before += sp;
         }
-        before = wave_allreduce(before, [](int a, int c) { return a + c; });
-        full = wave_allreduce(full, [](int a, int c) { return a + c; });
-        if (lane == 0) { s_part[item / experts][item % experts] = before; s_full[item / experts][item % experts] = full; }
+        // lanes q, q + HW, ... of a wave hold the same word index
+#pragma unroll
+        for (int off = HW; off < WAVE; off <<= 1) {
+            before += __shfl_xor(before, off, WAVE);
+            full += __shfl_xor(full, off, WAVE);
+        }
+        if (lane < HW) { atomicAdd(&s_before64[q], before); atomicAdd(&s_full64[q], full); }
     }
     lds_barrier();
-    if (tid < experts) {
+    if (tid < CAP) {
         int taken = 0;                                   // all first choices of an expert precede its second choices
-        for (int j = 0; j < k; ++j) { s_base[j][tid] = taken + s_part[j][tid]; taken += s_full[j][tid]; }
+        for (int j = 0; j < 4; ++j) {
+            const int idx = j * CAP + tid;
+            const int bef = (int)((s_before64[idx / 4] >> (16 * (idx % 4))) & 0xffffu);
+            const int ful = (int)((s_full64[idx / 4] >> (16 * (idx % 4))) & 0xffffu);
+            s_base[j][tid] = taken + bef;
+            s_full[j][tid] = ful;
+            taken += ful;
+        }
         s_tot[tid] = taken;
     }
     lds_barrier();
+    FS_STAMP(8);
 
-    FS_STAMP(7);
     // one parked row -> its slots (the k choices of a token hold the same codes: the all-ones gate)
     auto flush_row = [&](int prow, int tok) {
         const int t = t0 + tok;
@@ -353,68 +427,106 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
         uint4 v[G::RV];
         const uint4 *src = reinterpret_cast<const uint4 *>(park + prow * G::RS) + lane;
 #pragma unroll
-        for (int q = 0; q < G::RV; ++q) v[q] = src[q * WAVE];
+        for (int i = 0; i < G::RV; ++i) v[i] = src[i * WAVE];
         if (slot >= 0) { B16::store(bias_out, slot, s_mn[tok]); B16::store(scale_out, slot, s_sc[tok]); }
         for (int j = 0; j < k; ++j) {
             const int s = rl_i(slot, j);
             if (s < 0) continue;
             uint4 *dst = reinterpret_cast<uint4 *>(codes + (int64_t)s * G::M) + lane;
 #pragma unroll
-            for (int q = 0; q < G::RV; ++q) stream_store(dst + q * WAVE, v[q]);
+            for (int i = 0; i < G::RV; ++i) stream_store(dst + i * WAVE, v[i]);
         }
     };
 
-    for (int tok = w; tok < 16 * LDS_ROUNDS; tok += FS_WAVES) flush_row(tok, tok);
-    FS_STAMP(8);
-
+    // codes of the rounds that stayed in registers
+    auto encode_kept = [&]() {
+#pragma unroll
+        for (int rr = 0; rr < REG_ROUNDS; ++rr) {
+            uint4 (&raw)[NMMA] = ((LDS_ROUNDS + rr) & 1) ? buf1 : buf0;
+            const RowEncoder<PLANMOE_BF16> enc(s_mn[16 * (LDS_ROUNDS + rr) + m], s_sc[16 * (LDS_ROUNDS + rr) + m]);
+            auto body = [&](auto mode) {
+#pragma unroll
+                for (int i = 0; i < NMMA; ++i) {
+                    uint32_t wd[2];
+                    enc.template encode<decltype(mode)::value>(raw[i], wd);
+                    kept[rr][i] = make_uint2(wd[0], wd[1]);
+                }
+            };
+            if (__ballot(!enc.rq.fast) == 0) body(std::true_type{}); else body(std::false_type{});
+        }
+    };
     // empty slots: zero rows, dealt out over all waves of the grid
-    {
+    auto zero_fill = [&]() {
         const int slots = experts * capacity, nwaves = groups * FS_WAVES;
         for (int s = grp * FS_WAVES + w; s < slots; s += nwaves) {
             const int e = s / capacity;
             if (s - e * capacity < s_tot[e]) continue;
             uint4 *dst = reinterpret_cast<uint4 *>(codes + (int64_t)s * G::M) + lane;
 #pragma unroll
-            for (int q = 0; q < G::RV; ++q) stream_store(dst + q * WAVE, make_uint4(0u, 0u, 0u, 0u));
+            for (int i = 0; i < G::RV; ++i) stream_store(dst + i * WAVE, make_uint4(0u, 0u, 0u, 0u));
             if (lane == 0) { B16::store(bias_out, s, 0.f); B16::store(scale_out, s, 0.f); }
         }
-    }
+    };
 
-    // the rounds that stayed in registers: quantised now, through the same LDS rows
+    // The two waves that share a SIMD (w and w + 4) take their steps in opposite order: one codes
+    // while the other is held up by its stores, so the arithmetic of phase 2 hides under the stores.
+    if (w < FS_WAVES / 2) {
+        encode_kept();
+        for (int tok = w; tok < 16 * LDS_ROUNDS; tok += FS_WAVES) flush_row(tok, tok);
+    } else {
+        for (int tok = w; tok < 16 * LDS_ROUNDS; tok += FS_WAVES) flush_row(tok, tok);
+        encode_kept();
+    }
     FS_STAMP(9);
+
+    // those codes pass through the same LDS rows
+    lds_barrier();
+#pragma unroll
+    for (int rr = 0; rr < REG_ROUNDS; ++rr)
+#pragma unroll
+        for (int i = 0; i < NMMA; ++i) *reinterpret_cast<uint2 *>(my_park + rr * 16 * G::RS + 32 * i) = kept[rr][i];
     lds_barrier();
     FS_STAMP(10);
-    if constexpr (REG_ROUNDS == 2) {
-        constexpr int ra = ROUNDS - 2, rb = ROUNDS - 1;
-        if constexpr ((ra & 1) == 0) {
-            encode_to_park(buf0, m, keep_mn[0], keep_sc[0]);
-            encode_to_park(buf1, 16 + m, keep_mn[1], keep_sc[1]);
-        } else {
-            encode_to_park(buf1, m, keep_mn[1], keep_sc[1]);
-            encode_to_park(buf0, 16 + m, keep_mn[0], keep_sc[0]);
-        }
-        (void)rb;
-    } else {
-        encode_to_park(buf0, m, keep_mn[0], keep_sc[0]);
-    }
-    lds_barrier();
-    FS_STAMP(11);
     for (int i = w; i < 16 * REG_ROUNDS; i += FS_WAVES) flush_row(i, 16 * LDS_ROUNDS + i);
+    FS_STAMP(11);
+    zero_fill();
     FS_STAMP(12);
 
-    // the last group also finishes the GShard loss and the per-plane expert counts
+    // the last group closes the launch (every group has read the counter by now: all of them have
+    // published) and finishes the GShard loss and the per-plane expert counts
+    if (grp == groups - 1 && tid == 0) __hip_atomic_store(launches, launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (grp == groups - 1 && (l_aux || counts_out)) {
         if (counts_out && tid < k * experts) counts_out[tid] = s_full[tid / experts][tid % experts];
         if (l_aux) {
-            for (int e = w; e < experts; e += FS_WAVES) {
-                float me = column_partial(ws.me_t + (int64_t)e * ws.gstride, groups);
-                me = wave_allreduce(me, [](float a, float c) { return a + c; });
-                if (lane == 0) s_loss[e] = me * ((float)s_full[0][e] * ((float)experts / (float)samples));
+            // score sums of all groups, added in a fixed order: thread (gi, e) over its groups, then
+            // the partial sums one after the other
+            constexpr int MG = FS_THREADS / CAP, MP = (FS_MAX_GROUPS + MG - 1) / MG;
+            const int e = tid % CAP, mgi = tid / CAP;
+            float acc = 0.f;
+            bool in = false;
+            for (int spin = 0; spin <= spin_limit && !in; ++spin) {
+                unsigned long long mw[MP];
+#pragma unroll
+                for (int p = 0; p < MP; ++p)
+                    mw[p] = __hip_atomic_load(pub_me + (size_t)min(mgi + p * MG, groups - 1) * CAP + e, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+                in = true;
+                acc = 0.f;
+#pragma unroll
+                for (int p = 0; p < MP; ++p) {
+                    in = in && (uint32_t)(mw[p] >> 32) == tag;
+                    if (mgi + p * MG < groups) acc += __uint_as_float((uint32_t)mw[p]);
+                }
             }
+            s_mepart[mgi][e] = in ? acc : __uint_as_float(0x7fc00000u);      // a sum that never came in shows as NaN
             lds_barrier();
             if (tid == 0) {
                 float a = 0.f;
-                for (int e = 0; e < experts; ++e) a += s_loss[e];
+                for (int ee = 0; ee < experts; ++ee) {
+                    float me = 0.f;
+                    for (int i = 0; i < MG; ++i) me += s_mepart[i][ee];
+                    a += me * ((float)s_full[0][ee] * ((float)experts / (float)samples));
+                }
                 *l_aux = a / (float)samples;
             }
         }
