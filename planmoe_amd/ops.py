@@ -481,7 +481,7 @@ class ForwardInt8Plan:
     C-ABI call that enqueues the two launches (for serving loops that reuse their buffers)."""
 
     def __init__(self, x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
-                 want_l_aux=True, want_counts=False):
+                 want_l_aux=True, want_counts=False, single=False):
         x, wg, T, M, E, k, bias, out, _ = _forward_common(x, wg, top_k, fp32_gate, logit_bias, False,
                                                           False, want_l_aux, want_counts)
         # a workspace of the plan's own: redispatch() reads the routing state run() left in it, which
@@ -496,9 +496,16 @@ class ForwardInt8Plan:
                       int(bool(normalize_gate)), capacity_, _ptr(out["indices"]), _ptr(out["locations"]),
                       _ptr(out["gates"]), max(T, 1), None, None, _ptr(out["l_aux"]), _ptr(out["counts"]),
                       _ptr(out["codes"]), _ptr(out["bias"]), _ptr(out["scale"]), _ptr(ws), ws.numel()]
+        # single: the one-launch kernel that reads x once (planmoe_forward_int8_single; shapes it does
+        # not serve raise at run()); gave_up is its device flag
+        self.single = bool(single)
+        self.gave_up = torch.zeros((), dtype=torch.int32, device=x.device)
 
     def run(self):
-        check(lib.planmoe_forward_int8(*self._args, _stream(self.x)))
+        if self.single:
+            check(lib.planmoe_forward_int8_single(*self._args, 0, _ptr(self.gave_up), _stream(self.x)))
+        else:
+            check(lib.planmoe_forward_int8(*self._args, _stream(self.x)))
         return self.out
 
     def redispatch(self):

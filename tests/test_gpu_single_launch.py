@@ -54,3 +54,31 @@ def test_single_launch_gives_up_cleanly_when_told_to():
     out = ops.forward_int8_single(x, wg, k, 5120, spin_limit=1)
     torch.cuda.synchronize()
     assert int(out["gave_up"]) in (0, 1)
+
+
+def test_single_launch_in_a_graph_replayed_with_fresh_inputs():
+    """The captured launch carries the same arguments on every replay; the words the work-groups
+    publish must still be told apart from those of the replay before (the workspace's launch counter
+    does that).  Replays with fresh inputs, eager work between them, each against the eager result."""
+    from planmoe_amd import ops
+    T, M, E, k = 8192, 4096, 8, 2
+    C = ops.capacity(T, E, k, 1.25, 4)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(T, M, generator=g).bfloat16().to(DEV)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
+    plan = ops.ForwardInt8Plan(x, wg, k, C, single=True)
+    plan.run()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan.run()
+    for it in range(4):
+        x.copy_(torch.randn(T, M, generator=g).bfloat16())
+        graph.replay()
+        torch.cuda.synchronize()
+        got = {key: v.clone() for key, v in plan.out.items() if v is not None}
+        assert int(plan.gave_up) == 0
+        want = ops.forward_int8_single(x, wg, k, C)
+        for key in ("indices", "locations", "gates", "codes", "bias", "scale", "l_aux"):
+            a, b = got[key], want[key]
+            assert torch.equal(a.reshape(-1).view(torch.uint8), b.reshape(-1).view(torch.uint8)), (it, key)
