@@ -5,12 +5,14 @@
 #ifndef PLANMOE_ZFP_COMPRESSOR
 #define PLANMOE_ZFP_COMPRESSOR
 #include "abstract.h"
+#include <hip/hip_runtime_api.h>
 
 class ZfpCompressor : public AbstractCompressor {
 public:
     torch::Tensor compress(const torch::Tensor &) override;
     torch::Tensor decompress(const torch::Tensor &) override;
     void          all_to_all(const torch::Tensor &, const torch::Tensor &) override;
+    void          set_cuda_stream(const hipStream_t &);
     void          set_compress_rate(const double &);
     ZfpCompressor(std::shared_ptr<AbstractComm>, double = 8.0) noexcept;
     ~ZfpCompressor();
@@ -21,5 +23,6 @@ public:
     size_t            last_bufsize;
     std::vector<long> sizes;
     size_t            length;
+    hipStream_t       cuda_stream = nullptr;
 };
 #endif

@@ -5,7 +5,8 @@ custom/custom_kernel.cpp:194-288 (the pybind surface of ``schemoe_custom_kernel`
 Objects are stateful and single use, exactly as in the reference: ``compress`` records what
 ``decompress`` needs.  With one GPU the all-to-all is the identity: ``comm_operation`` hands the
 send buffers over as the receive buffers, or (``SINGLE_RANK_COMM_COPIES``) ``all_to_all`` copies
-the send buffer into ``g_output`` and the per-row state into its receive-side twins."""
+the send buffer into ``g_output`` and the per-row state into its receive-side twins, on a comm
+stream under the reference's event protocol."""
 import torch
 
 from . import ops
@@ -192,21 +193,52 @@ def get_comm(name):
 
 
 # custom_kernel.cpp:226-288 -------------------------------------------------------------------
+# When the comm step copies (SINGLE_RANK_COMM_COPIES), it runs on a comm stream of its own, at the
+# priority of the compute stream, under the reference's event protocol: the event of a slot is
+# recorded behind the compress (custom_kernel.cpp:251-253), the comm stream waits for it, carries
+# the copies and records it again (:269-275), the decompress makes the compute stream wait for it
+# (:281-283).  With a2a_ffn_overlap_degree > 1 a chunk's copy then runs beside the next chunk's
+# compress.  Tensors that the comm stream touches are marked with record_stream, as int8.cpp:25-42
+# does, so that the allocator does not hand their memory out while the copy is in flight.
 _compress_ptr_lst = []
+_events = []
 _comm_cnt = 0
 _decompress_cnt = 0
+_comm_streams = {}
+
+
+def comm_stream(device):
+    """The comm stream of `device` (the reference's g_nccl_stream), created on first use."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    if index not in _comm_streams:
+        _comm_streams[index] = torch.cuda.Stream(device=index)          # default priority
+    return _comm_streams[index]
+
+
+def _tensors_of(c):
+    return [v for v in vars(c).values() if isinstance(v, torch.Tensor) and v.is_cuda]
 
 
 def clear_ptr_lst():
     global _comm_cnt, _decompress_cnt
     _compress_ptr_lst.clear()
+    _events.clear()
     _comm_cnt = 0
     _decompress_cnt = 0
 
 
 def compress_operation(input, name, comm_name):
     _compress_ptr_lst.append(get_compressor(name, get_comm(comm_name)))
-    return _compress_ptr_lst[-1].compress(input)
+    out = _compress_ptr_lst[-1].compress(input)
+    event = None
+    if SINGLE_RANK_COMM_COPIES and out.is_cuda:
+        event = torch.cuda.Event()
+        event.record(torch.cuda.current_stream(out.device))
+        side = comm_stream(out.device)
+        for t in [out] + _tensors_of(_compress_ptr_lst[-1]):
+            t.record_stream(side)
+    _events.append(event)
+    return out
 
 
 def comm_operation(input):
@@ -219,6 +251,12 @@ def comm_operation(input):
     c.pre_comm(None)
     if c.comm_ptr.g_world_size == 1 and not SINGLE_RANK_COMM_COPIES:
         c.adopt(input)
+    elif _events[idx] is not None:
+        side = comm_stream(input.device)
+        side.wait_event(_events[idx])
+        with torch.cuda.stream(side):
+            c.all_to_all(input, c.g_output)
+        _events[idx].record(side)
     else:
         c.all_to_all(input, c.g_output)
     return c.g_output
@@ -230,6 +268,8 @@ def decompress_operation(input):
     if idx >= len(_compress_ptr_lst) or _compress_ptr_lst[idx] is None:
         raise PlanMoEError("decompress_operation: no matching compress_operation")
     _decompress_cnt += 1
+    if _events[idx] is not None and input.is_cuda:
+        torch.cuda.current_stream(input.device).wait_event(_events[idx])
     output = _compress_ptr_lst[idx].decompress(input)
     _compress_ptr_lst[idx] = None
     return output

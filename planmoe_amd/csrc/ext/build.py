@@ -29,7 +29,17 @@ def build():
     cmd += ["-lplanmoe_hip", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python", "-lamdhip64",
             "-Wl,-rpath," + csrc, "-Wl,-rpath,/opt/rocm/lib"] + ["-Wl,-rpath," + p for p in ce.library_paths()]
     subprocess.check_call(cmd)
+    # the example plug-in: a compressor compiled against include/planmoe/compressor/abstract.h with the
+    # same flags and linked against the module just built
+    flags = cmd[1:cmd.index(os.path.join(HERE, NAME + ".cpp"))]
+    libs = [a for a in cmd[cmd.index(target()) + 1:] if a != "-lplanmoe_hip"]
+    subprocess.check_call(["g++"] + flags + [os.path.join(HERE, "example_third_party_compressor.cpp"), "-o", example_target(),
+                                             target(), "-Wl,-rpath," + HERE] + libs)
     return target()
+
+
+def example_target():
+    return os.path.join(HERE, "libexample_third_party_compressor.so")
 
 
 if __name__ == "__main__":

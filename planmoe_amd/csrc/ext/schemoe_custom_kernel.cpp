@@ -3,15 +3,20 @@
 // compress_operation / comm_operation / decompress_operation / clear_ptr_lst, plus
 // torch.ops.tutel_ops.cumsum (custom_kernel.cpp:331-385).  All device work goes through the C
 // ABI of libplanmoe_hip; this file only owns tensors and object lifetimes.
-// One GPU: the comm step copies into g_output on the current stream.
+// One GPU: the comm step is a device copy into g_output, issued on a comm stream of its own (same
+// priority as the compute stream) under the reference's event protocol, so that with
+// a2a_ffn_overlap_degree > 1 a chunk's copy runs beside the next chunk's compress.
 #include "planmoe/compressor/abstract.h"
 #include "planmoe/compressor/int8.h"
 #include "planmoe/compressor/lz.h"
 #include "planmoe/compressor/no.h"
 #include "planmoe/compressor/zfpc.h"
+#include "planmoe/compressor/registry.h"
 #include "planmoe_hip.h"
 
+#include <ATen/hip/HIPEvent.h>
 #include <hip/hip_runtime_api.h>
+#include <map>
 #include <torch/script.h>
 
 static void *current_stream() { return (void *)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
@@ -43,8 +48,11 @@ IdentityComm::IdentityComm(std::vector<PlanMoEStream> *stream, std::vector<ncclC
 void IdentityComm::all_to_all(const torch::Tensor &input, const torch::Tensor &output, size_t length)
 {
     AT_ASSERTM(g_world_size == 1, "IdentityComm is the one-GPU all-to-all");
-    AT_ASSERTM(hipMemcpyAsync(output.data_ptr(), input.data_ptr(), length, hipMemcpyDeviceToDevice,
-                              (hipStream_t)current_stream()) == hipSuccess, "all_to_all copy failed");
+    // on the comm stream (naive.cpp:11-27 issues its send / recv pairs on stream->at(0)); the caller
+    // has made that stream wait for the producer of `input`
+    hipStream_t st = (stream && !stream->empty()) ? (hipStream_t)stream->at(0).stream() : (hipStream_t)current_stream();
+    AT_ASSERTM(hipMemcpyAsync(output.data_ptr(), input.data_ptr(), length, hipMemcpyDeviceToDevice, st) == hipSuccess,
+               "all_to_all copy failed");
 }
 
 // ---------------------------------------------------------------- compressors
@@ -84,6 +92,9 @@ torch::Tensor Int8Compressor::compress(const torch::Tensor &input_)
     g_bias = at::empty_like(bias);
     g_scale = at::empty_like(scale);
     this->g_output = at::empty_like(fp_output);
+    // the comm stream reads bias / scale and writes their receive-side twins (int8.cpp:25-42)
+    for (auto &comm_stream : *comm_ptr->stream)
+        for (const torch::Tensor *t : {&bias, &scale, &g_bias, &g_scale, &g_output}) t->record_stream(comm_stream);
     return fp_output;
 }
 torch::Tensor Int8Compressor::decompress(const torch::Tensor &input)
@@ -112,6 +123,9 @@ ZfpCompressor::ZfpCompressor(std::shared_ptr<AbstractComm> comm_ptr, double comp
     this->last_bufsize = 0;
 }
 ZfpCompressor::~ZfpCompressor() { buffer = nullptr; }
+// zfpc.h:15 -- the reference hands zfp's CUDA back end a stream; here every launch goes to the
+// current stream, the value is only kept
+void ZfpCompressor::set_cuda_stream(const hipStream_t &s) { this->cuda_stream = s; }
 void ZfpCompressor::set_compress_rate(const double &rate) { this->compress_rate = rate; }
 torch::Tensor ZfpCompressor::compress(const torch::Tensor &input_)
 {
@@ -191,10 +205,39 @@ void LzCompressor::all_to_all(const torch::Tensor &, const torch::Tensor &)
 }
 
 // ---------------------------------------------------------------- registry (custom_kernel.cpp:194-288)
-static std::vector<PlanMoEStream> g_streams;          // no comm streams on one GPU
+// one comm stream per device, taken from torch's pool at default priority the first time it is
+// needed (the reference's g_nccl_stream, custom_kernel.cpp:128-153), and one event per
+// compress / comm / decompress triple (g_cuda_events)
+static std::map<int, std::vector<PlanMoEStream>> g_streams_by_device;
+static std::vector<at::cuda::CUDAEvent> g_events;
+
+static std::vector<PlanMoEStream> *comm_streams()
+{
+    const int dev = (int)c10::hip::current_device();
+    auto it = g_streams_by_device.find(dev);
+    if (it == g_streams_by_device.end())
+        it = g_streams_by_device.emplace(dev, std::vector<PlanMoEStream>{
+                 c10::hip::getStreamFromPoolMasqueradingAsCUDA(/*isHighPriority=*/false)}).first;
+    return &it->second;
+}
+
+static std::map<std::string, planmoe::CompressorFactory> &factories()
+{
+    static std::map<std::string, planmoe::CompressorFactory> f;
+    return f;
+}
+void planmoe::register_compressor(const std::string &name, planmoe::CompressorFactory factory) { factories()[name] = factory; }
+std::vector<std::string> planmoe::registered_compressors()
+{
+    std::vector<std::string> names;
+    for (auto &kv : factories()) names.push_back(kv.first);
+    return names;
+}
 
 static AbstractCompressor *get_compressor(const std::string &name, std::shared_ptr<AbstractComm> comm_ptr)
 {
+    auto it = factories().find(name);                       // plug-ins first: they may replace a built-in name
+    if (it != factories().end()) return it->second(comm_ptr);
     if (name == "int8") return new Int8Compressor(comm_ptr);
     if (name == "zfp") return new ZfpCompressor(comm_ptr);
     if (name == "lz") return new LzCompressor(comm_ptr);
@@ -203,7 +246,7 @@ static AbstractCompressor *get_compressor(const std::string &name, std::shared_p
 static std::shared_ptr<AbstractComm> get_comm(const std::string &)
 {
     // naive / pipe / dd / hetu are all the identity on one GPU
-    return std::make_shared<IdentityComm>(&g_streams, std::vector<ncclComm_t>(), 1, 0, 1, 0);
+    return std::make_shared<IdentityComm>(comm_streams(), std::vector<ncclComm_t>(), 1, 0, 1, 0);
 }
 
 static std::vector<AbstractCompressor *> compress_ptr_lst;
@@ -217,11 +260,20 @@ static void clear_ptr_lst()
     comm_cnt = 0;
     decompress_cnt = 0;
 }
+// custom_kernel.cpp:242-258: the event of slot idx is recorded behind the compress on the compute stream
 static torch::Tensor compress_operation(const torch::Tensor &input, const std::string &str, const std::string &comm_name)
 {
+    CHECK_GPU(input);                      // before anything asks the device for a stream
+    const size_t idx = compress_ptr_lst.size();
     compress_ptr_lst.emplace_back(get_compressor(str, get_comm(comm_name)));
-    return compress_ptr_lst.back()->compress(input);
+    torch::Tensor after_compress = compress_ptr_lst.back()->compress(input);
+    if (g_events.size() <= idx) g_events.resize(idx + 1);
+    g_events[idx].record(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
+    for (auto &comm_stream : *comm_streams()) after_compress.record_stream(comm_stream);
+    return after_compress;
 }
+// custom_kernel.cpp:260-277: the comm stream waits for the compress, carries the all-to-all, and
+// records the event again
 static torch::Tensor comm_operation(const torch::Tensor &input)
 {
     AT_ASSERTM(comm_cnt < (int)compress_ptr_lst.size() && compress_ptr_lst[comm_cnt],
@@ -229,14 +281,21 @@ static torch::Tensor comm_operation(const torch::Tensor &input)
     const int idx = comm_cnt++;
     const PlanMoEStream original_stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
     compress_ptr_lst[idx]->pre_comm(&original_stream);
+    for (auto &comm_stream : *comm_streams()) g_events[idx].block(comm_stream);
     compress_ptr_lst[idx]->all_to_all(input, compress_ptr_lst[idx]->g_output);
+    for (auto &comm_stream : *comm_streams()) {
+        g_events[idx].record(comm_stream);
+        compress_ptr_lst[idx]->g_output.record_stream(comm_stream);
+    }
     return compress_ptr_lst[idx]->g_output;
 }
+// custom_kernel.cpp:279-288: the compute stream waits for the all-to-all
 static torch::Tensor decompress_operation(const torch::Tensor &input)
 {
     AT_ASSERTM(decompress_cnt < (int)compress_ptr_lst.size() && compress_ptr_lst[decompress_cnt],
                "decompress_operation: no matching compress_operation");
     const int idx = decompress_cnt++;
+    g_events[idx].block(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
     torch::Tensor output = compress_ptr_lst[idx]->decompress(input);
     delete compress_ptr_lst[idx];
     compress_ptr_lst[idx] = nullptr;
@@ -262,8 +321,23 @@ torch::Tensor warp_cumsum(torch::Tensor x)
     return y;
 }
 
+// the reference's NVRTC entry points (custom_kernel.cpp:295-298, jit.h): the mechanism this build
+// replaces with compiled gfx950 kernels behind typed entry points
+static void jit_unavailable(const char *what)
+{
+    AT_ASSERTM(false, what, ": this build has no run-time kernel compiler; its kernels are compiled into "
+               "libplanmoe_hip.so (see include/planmoe_hip.h for the typed entry points)");
+}
+static void update_sdk_home(const torch::Tensor &) { jit_unavailable("update_sdk_home"); }
+static int inject_source(const std::string &) { jit_unavailable("inject_source"); return -1; }
+static void invoke(const std::vector<torch::Tensor> &, const std::vector<long> &, int) { jit_unavailable("invoke"); }
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
+    m.def("update_sdk_home", &update_sdk_home, "not available in this build");
+    m.def("invoke", &invoke, "not available in this build");
+    m.def("inject_source", &inject_source, "not available in this build");
+    m.def("registered_compressors", &planmoe::registered_compressors, "names of the compressor plug-ins registered from C++");
     m.def("invoke_cpu_fp32", &invoke_cpu_unavailable, "not available in this build");
     m.def("invoke_cpu_fp64", &invoke_cpu_unavailable, "not available in this build");
     m.def("compress_operation", &compress_operation, "Compress Operation");

@@ -32,6 +32,74 @@ def test_module_surface_and_host_side_errors():
     with pytest.raises(RuntimeError, match="GPU tensor"):
         ck.compress_operation(torch.zeros(4, 4, 8), "lz", "naive")
     ck.clear_ptr_lst()
+    # the reference's NVRTC entry points exist and say what replaced them (custom_kernel.cpp:295-298)
+    for call in (lambda: ck.update_sdk_home(torch.zeros(1)), lambda: ck.inject_source("__global__ void f() {}"),
+                 lambda: ck.invoke([torch.zeros(1)], [1], 0)):
+        with pytest.raises(RuntimeError, match="no run-time kernel compiler"):
+            call()
+
+
+def _load_example_plugin():
+    """The example third-party compressor: built against include/planmoe/compressor/abstract.h by
+    ext/build.py, linked against the extension module, registered under the name 'half'."""
+    import ctypes
+    import os
+    from planmoe_amd import ext
+    ck = ext.load()
+    path = os.path.join(os.path.dirname(ext.PATH), "libexample_third_party_compressor.so")
+    assert os.path.exists(path), "run python planmoe_amd/csrc/ext/build.py"
+    ctypes.CDLL(path).register_example_compressor()
+    return ck
+
+
+def test_third_party_compressor_registers():
+    ck = _load_example_plugin()
+    assert "half" in ck.registered_compressors()
+
+
+@pytest.mark.gpu
+def test_third_party_compressor_runs_through_the_registry():
+    """A subclass of AbstractCompressor compiled outside the extension goes through
+    compress_operation / comm_operation / decompress_operation like a built-in one."""
+    ck = _load_example_plugin()
+    x = torch.randn(4, 64, 256, generator=torch.Generator().manual_seed(9)).to(DEV)
+    ck.clear_ptr_lst()
+    sent = ck.compress_operation(x, "half", "naive")
+    assert sent.dtype == torch.float16 and torch.equal(sent, x.half())
+    recv = ck.comm_operation(sent)
+    assert recv.data_ptr() != sent.data_ptr()
+    out = ck.decompress_operation(recv)
+    assert out.dtype == torch.float32 and torch.equal(out, x.half().float())
+    ck.clear_ptr_lst()
+
+
+@pytest.mark.gpu
+def test_comm_runs_on_its_own_stream_under_the_event_protocol():
+    """Two chunks, each compress -> comm, then decompress in order (overlap.py:59-74 with degree 2):
+    the copies are issued on the comm stream, the results equal those of one chunk at a time, and
+    producing the next chunk's input on the compute stream right after cannot overtake a copy."""
+    from planmoe_amd import compressor, ext
+    ck = ext.load()
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(8, 512, 1024, generator=g).bfloat16().to(DEV)
+    for mod in (ck, compressor):
+        old = compressor.SINGLE_RANK_COMM_COPIES
+        compressor.SINGLE_RANK_COMM_COPIES = True
+        try:
+            mod.clear_ptr_lst()
+            whole = mod.decompress_operation(mod.comm_operation(mod.compress_operation(x, "int8", "naive")))
+            mod.clear_ptr_lst()
+            halves = [h.contiguous() for h in x.split(256, dim=1)]
+            recv = []
+            for h in halves:
+                recv.append(mod.comm_operation(mod.compress_operation(h, "int8", "naive")))
+                h.zero_()            # the compute stream moves on and overwrites the chunk it has compressed
+            got = torch.cat([mod.decompress_operation(r) for r in recv], dim=1)
+            torch.cuda.synchronize()
+            assert torch.equal(got, whole)
+            mod.clear_ptr_lst()
+        finally:
+            compressor.SINGLE_RANK_COMM_COPIES = old
 
 
 @pytest.mark.gpu
