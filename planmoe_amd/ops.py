@@ -434,6 +434,15 @@ def forward_int8(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, norma
     return out
 
 
+def forward_int8_single_serves(x, wg, top_k):
+    """The shapes planmoe_forward_int8_single takes: bf16 rows of 4096 values, up to 16 experts,
+    top_k <= 4, at most 64 tokens per compute unit."""
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.shape[1] == 4096 and x.shape[0] >= 1):
+        return False
+    cus = torch.cuda.get_device_properties(x.device).multi_processor_count
+    return wg.shape[0] <= 16 and min(int(top_k), wg.shape[0]) <= 4 and x.shape[0] <= 64 * cus
+
+
 def forward_int8_single(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
                         want_logits=False, want_scores=False, want_l_aux=True, want_counts=False, spin_limit=0):
     """forward_int8 in one launch that reads x once (bf16 rows of 4096 values, up to 16 experts,

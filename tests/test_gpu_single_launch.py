@@ -82,3 +82,43 @@ def test_single_launch_in_a_graph_replayed_with_fresh_inputs():
         for key in ("indices", "locations", "gates", "codes", "bias", "scale", "l_aux"):
             a, b = got[key], want[key]
             assert torch.equal(a.reshape(-1).view(torch.uint8), b.reshape(-1).view(torch.uint8)), (it, key)
+
+
+def test_moe_layer_with_the_single_launch_send_side():
+    """moe_layer (int8 compressor, identity experts) with overlap.FORWARD_SINGLE_LAUNCH: forward and
+    backward against the same layer on the two-launch send side.  The two gate GEMMs add their
+    partial sums in another order, so a token within an ulp of a tie may go elsewhere: all but a
+    sliver of the rows must agree to the bit."""
+    import planmoe_amd
+    from planmoe_amd import overlap
+
+    class Identity(torch.nn.Module):
+        def update(self, ctx):
+            self.dummy = torch.nn.Parameter(torch.zeros(1))
+
+        def forward(self, x, ctx):
+            return x
+
+    T, M, E = 4096, 4096, 8
+    results = []
+    for single in (False, True):
+        overlap.FORWARD_SINGLE_LAUNCH = single
+        try:
+            layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'capacity_factor': 1.25, 'fp32_gate': True}, M,
+                                          experts={'type': 'custom', 'module': Identity(), 'count_per_node': E},
+                                          seeds=(1, 2, 3), compress_name='int8').to(DEV).to(torch.bfloat16)
+            x = torch.randn(T, M, generator=torch.Generator().manual_seed(0)).bfloat16().to(DEV).requires_grad_(True)
+            y = layer(x)
+            (y.float().square().mean() + y.l_aux.float()).backward()
+            torch.cuda.synchronize()
+            results.append((y.detach().float(), x.grad.float(), float(y.l_aux.detach()), layer.gates[0].wg.weight.grad.float()))
+        finally:
+            overlap.FORWARD_SINGLE_LAUNCH = False
+    (y0, g0, l0, w0), (y1, g1, l1, w1) = results
+    same_rows = (y0 == y1).all(dim=1).float().mean().item()
+    assert same_rows > 0.999
+    # x.grad carries the gate's share, which depends on the scores' last bits: bf16 tolerance
+    assert torch.allclose(g0, g1, rtol=2e-2, atol=2e-2 * g0.abs().max().item())
+    assert (g0 == g1).float().mean().item() > 0.99
+    assert abs(l0 - l1) <= 1e-4 * abs(l0)
+    assert torch.allclose(w0, w1, rtol=2e-2, atol=1e-3 * w0.abs().max().item())
