@@ -411,6 +411,203 @@ __global__ __launch_bounds__(256) void zfp_decode1_kernel(const uint32_t *__rest
     reinterpret_cast<float4 *>(field)[b] = make_float4(f[0], f[1], f[2], f[3]);
 }
 
+// ---------------------------------------------------------------- 1-D blocks of 32 bits (rate 8)
+// A block is 4 values and one 32-bit word: 9 header bits and a budget of 23.  Everything a bit
+// plane contributes follows from two small numbers, the count of values that are significant
+// already and the plane's 4 bits, so both directions look their group tests up instead of
+// walking them: the coder in a table of 4 x 16 entries (code, length, newly significant values),
+// the decoder in one of 4 x 128 entries indexed by the next 7 stream bits (the longest group-test
+// code of a plane has 7 bits), and the block's word never leaves its register.
+
+// group-test code of the 4 - nsig values that are not significant yet, whose plane bits are r:
+// code in bits 0..7, its length in bits 8..11, the values that become significant in bits 12..14
+__host__ __device__ constexpr uint32_t gt4_code(int nsig, uint32_t r)
+{
+    uint32_t code = 0, x = r;
+    int len = 0, n = nsig;
+    while (n < 4) {
+        const uint32_t any = x != 0u;
+        code |= any << len; ++len;
+        if (!any) break;
+        while (n < 3) {
+            const uint32_t one = x & 1u;
+            code |= one << len; ++len;
+            if (one) break;
+            x >>= 1; ++n;
+        }
+        x >>= 1; ++n;
+    }
+    return code | ((uint32_t)len << 8) | ((uint32_t)(n - nsig) << 12);
+}
+
+// the inverse, for a stream whose next 7 bits are s and whose budget does not end inside the code:
+// plane bits (at their absolute positions) in bits 0..3, bits used in 4..7, newly significant in 8..10
+__host__ __device__ constexpr uint32_t gt4_parse(int nsig, uint32_t s)
+{
+    uint32_t x = 0;
+    int used = 0, n = nsig;
+    while (n < 4) {
+        const uint32_t any = (s >> used) & 1u; ++used;
+        if (!any) break;
+        while (n < 3) {
+            const uint32_t one = (s >> used) & 1u; ++used;
+            if (one) break;
+            ++n;
+        }
+        x |= 1u << n; ++n;
+    }
+    return x | ((uint32_t)used << 4) | ((uint32_t)(n - nsig) << 8);
+}
+
+// The 32 bit planes of a 1-D block as nibbles: word c holds the planes k = c (mod 4), plane k in
+// bits k - c .. k - c + 3 (bit i of the nibble = bit k of value i).  32 operations for all planes
+// instead of 8 per plane.
+__device__ __forceinline__ void planes_of(const uint32_t (&u)[4], uint32_t (&pl)[4])
+{
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+        pl[c] = ((u[0] >> c) & 0x11111111u) | (((u[1] >> c) & 0x11111111u) << 1) |
+                (((u[2] >> c) & 0x11111111u) << 2) | (((u[3] >> c) & 0x11111111u) << 3);
+}
+__device__ __forceinline__ void values_of(const uint32_t (&pl)[4], uint32_t (&u)[4])
+{
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        u[i] = ((pl[0] >> i) & 0x11111111u) | (((pl[1] >> i) & 0x11111111u) << 1) |
+               (((pl[2] >> i) & 0x11111111u) << 2) | (((pl[3] >> i) & 0x11111111u) << 3);
+}
+
+// both tables worked out by the compiler; a work-group copies them into LDS
+struct Gt4Tables {
+    uint32_t code[64];      // [nsig][plane bits]: code, length, newly significant values, a byte each
+    uint16_t parse[512];    // [nsig][next 7 stream bits]
+    constexpr Gt4Tables() : code(), parse()
+    {
+        for (int i = 0; i < 64; ++i) {
+            const uint32_t e = gt4_code(i >> 4, (uint32_t)i & 15u);
+            code[i] = (e & 0xffu) | (((e >> 8) & 15u) << 8) | ((e >> 12) << 16);
+        }
+        for (int i = 0; i < 512; ++i) parse[i] = (uint16_t)gt4_parse(i >> 7, (uint32_t)i & 127u);
+    }
+};
+__constant__ const Gt4Tables gt4_tables = Gt4Tables();
+
+__global__ __launch_bounds__(256) void zfp_encode1_word_kernel(const float *__restrict__ field, int64_t blocks,
+                                                               uint32_t *__restrict__ out)
+{
+    __shared__ uint32_t tab[64];
+    if (threadIdx.x < 64) tab[threadIdx.x] = gt4_tables.code[threadIdx.x];
+    __syncthreads();
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    if (b == blocks - 1 && (blocks & 1)) out[blocks] = 0u;      // the other half of the last 64-bit stream word
+    const float4 v = reinterpret_cast<const float4 *>(field)[b];
+    const float f[4] = {v.x, v.y, v.z, v.w};
+    const float m = fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3])));
+    if (!(m > 0.f)) { out[b] = 0u; return; }                     // all-zero block: '0' flag and zero padding
+    const int emax = (int)((__float_as_uint(m) >> 23) & 0xffu) - 126;
+    const int se = 30 - emax;
+    const float s = se > 127 ? INFINITY : __uint_as_float((uint32_t)(se + 127) << 23);
+    int32_t q[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float t = f[i] * s;
+        q[i] = fabsf(t) < 2147483648.0f ? (int32_t)t : (int32_t)0x80000000;
+    }
+    fwd_lift(q[0], q[1], q[2], q[3]);
+    const uint32_t u[4] = {to_negabinary(q[0]), to_negabinary(q[1]), to_negabinary(q[2]), to_negabinary(q[3])};
+    uint32_t pl[4];
+    planes_of(u, pl);
+
+    // The word fills from bit 9 up.  What does not fit falls off the top of the 32-bit register, which
+    // is exactly where the budget cuts the stream, so nothing is masked to the remaining budget.
+    uint32_t acc = 2u * (uint32_t)(emax + 127) + 1u;
+    int fill = 9, nsig = 0;
+    uint32_t sigmask = 0u;                                       // (1 << nsig) - 1
+    auto plane = [&](uint32_t x) __attribute__((always_inline)) {
+        acc |= (x & sigmask) << fill;
+        fill += nsig;
+        if (nsig < 4 && fill < 32) {
+            const uint32_t e = tab[nsig * 16 + (int)(x >> nsig)];
+            acc |= (e & 0xffu) << fill;
+            fill += (int)((e >> 8) & 0xffu);
+            nsig += (int)(e >> 16);
+            sigmask = (1u << nsig) - 1u;
+        }
+    };
+    for (int kb = 28; kb >= 0 && fill < 32; kb -= 4) {
+        plane((pl[3] >> kb) & 15u);
+        if (fill < 32) plane((pl[2] >> kb) & 15u);
+        if (fill < 32) plane((pl[1] >> kb) & 15u);
+        if (fill < 32) plane((pl[0] >> kb) & 15u);
+    }
+    out[b] = acc;
+}
+
+__global__ __launch_bounds__(256) void zfp_decode1_word_kernel(const uint32_t *__restrict__ in, int64_t blocks,
+                                                               float *__restrict__ field)
+{
+    __shared__ uint16_t tab[512];
+    for (int i = threadIdx.x; i < 512; i += 256) tab[i] = gt4_tables.parse[i];
+    __syncthreads();
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    const uint32_t w = in[b];
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (w & 1u) {
+        const int emax = (int)((w >> 1) & 0xffu) - 127;
+        uint32_t s = w >> 9;                                     // the 23 coded bits, zeros above them
+        uint32_t pl[4] = {0u, 0u, 0u, 0u};
+        int bits = 23, nsig = 0;
+        uint32_t sigmask = 0u;
+        // plane bits of one plane; reading past the budget reads zeros, as the budget's end demands
+        auto plane = [&]() __attribute__((always_inline)) {
+            uint32_t x = s & sigmask;
+            s >>= nsig; bits -= nsig;
+            if (nsig < 4 && bits > 0) {
+                const uint32_t e = tab[nsig * 128 + (int)(s & 127u)];
+                const int used = (int)((e >> 4) & 15u);
+                if (used <= bits) {                             // every bit the table looked at is the block's own
+                    x |= e & 15u;
+                    s >>= used; bits -= used;
+                    nsig += (int)(e >> 8);
+                } else {
+                    // the budget may end inside the code: bit by bit
+                    while (nsig < 4 && bits > 0) {
+                        --bits;
+                        const uint32_t any = s & 1u; s >>= 1;
+                        if (!any) break;
+                        while (nsig < 3 && bits > 0) {
+                            --bits;
+                            const uint32_t one = s & 1u; s >>= 1;
+                            if (one) break;
+                            ++nsig;
+                        }
+                        x |= 1u << nsig; ++nsig;
+                    }
+                }
+                sigmask = (1u << nsig) - 1u;
+            }
+            return x;
+        };
+        for (int kb = 28; kb >= 0 && bits > 0; kb -= 4) {
+            pl[3] |= plane() << kb;
+            if (bits > 0) pl[2] |= plane() << kb;
+            if (bits > 0) pl[1] |= plane() << kb;
+            if (bits > 0) pl[0] |= plane() << kb;
+        }
+        uint32_t u[4];
+        values_of(pl, u);
+        int32_t q0 = from_negabinary(u[0]), q1 = from_negabinary(u[1]), q2 = from_negabinary(u[2]), q3 = from_negabinary(u[3]);
+        inv_lift(q0, q1, q2, q3);
+        // 2^(emax - 30): a normal number unless the block's values are next to the denormals
+        const int se = emax - 30 + 127;
+        const float sc = se >= 1 ? __uint_as_float((uint32_t)se << 23) : ldexpf(1.0f, emax - 30);
+        o = make_float4((float)q0 * sc, (float)q1 * sc, (float)q2 * sc, (float)q3 * sc);
+    }
+    reinterpret_cast<float4 *>(field)[b] = o;
+}
+
 template <int NW>
 __global__ __launch_bounds__(256) void zfp_encode2_kernel(const float *__restrict__ field, int64_t nx,
                                                           int64_t nbx, int64_t blocks,
@@ -722,6 +919,11 @@ extern "C" int planmoe_zfp_compress(const float *field, int dims, int64_t nx, in
                stream_capacity, need);
     hipStream_t st = (hipStream_t)stream;
     const unsigned grid = (unsigned)((blocks + 255) / 256);
+    if (dims == 1 && nw == 1) {
+        zfp_encode1_word_kernel<<<grid, 256, 0, st>>>(field, blocks, (uint32_t *)stream_out);
+        PM_LAUNCH_CHECK("planmoe_zfp_compress");
+        return 0;
+    }
     PM_NW_SWITCH(nw, NW, {
         if (dims == 1) zfp_encode1_kernel<NW><<<grid, 256, 0, st>>>(field, blocks, (uint32_t *)stream_out);
         else zfp_encode2_kernel<NW><<<grid, 256, 0, st>>>(field, nx, nx / 4, blocks, (uint32_t *)stream_out);
@@ -740,6 +942,11 @@ extern "C" int planmoe_zfp_decompress(const void *stream_in, int dims, int64_t n
     PM_REQUIRE(aligned16(field) && aligned16(stream_in), "planmoe_zfp_decompress: buffers must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
     const unsigned grid = (unsigned)((blocks + 255) / 256);
+    if (dims == 1 && nw == 1) {
+        zfp_decode1_word_kernel<<<grid, 256, 0, st>>>((const uint32_t *)stream_in, blocks, field);
+        PM_LAUNCH_CHECK("planmoe_zfp_decompress");
+        return 0;
+    }
     PM_NW_SWITCH(nw, NW, {
         if (dims == 1) zfp_decode1_kernel<NW><<<grid, 256, 0, st>>>((const uint32_t *)stream_in, blocks, field);
         else zfp_decode2_kernel<NW><<<grid, 256, 0, st>>>((const uint32_t *)stream_in, nx, nx / 4, blocks, field);
