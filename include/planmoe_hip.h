@@ -310,6 +310,20 @@ int planmoe_forward_int8_redispatch(const void *x, int dtype, int samples, int m
                                     void *bias, void *scale, void *workspace, size_t workspace_bytes,
                                     void *stream);
 
+/* ---------------------------------------------------------------- expert FFN on int8 codes
+ * The first batched GEMM of FusedExpertsNetwork.forward (experts/ffn.py:77) with the receive
+ * side's Int8Compressor::decompress (int8.cpp:46-60, reached from overlap.py:66) as its prologue:
+ *   out[e][r][n] = bf16( bf16( sum_k dec(e, r, k) * w[e][n][k] ) + fc_bias[e][n] )
+ * where dec(e, r, k) is the bf16 value planmoe_int8_decompress would have stored for code
+ * codes[e][r][k] with bias[e][r], scale[e][r].  The decoded [experts, rows, model_dim] tensor
+ * never exists in memory.  weight_k_major is the layer's batched_fc1_w [experts, model_dim,
+ * hidden] transposed to [experts, hidden, model_dim] (k fastest: what both MFMA operands want);
+ * fc_bias [experts, hidden] may be NULL.  bf16 only; model_dim a multiple of 64, hidden of 128.
+ * Results equal torch.matmul on the decompressed tensor up to the order of the fp32 sums. */
+int planmoe_ffn_fc1_int8(const uint8_t *codes, const void *bias, const void *scale, int dtype,
+                         const void *weight_k_major, const void *fc_bias, int experts, int rows,
+                         int model_dim, int hidden, void *out, void *stream);
+
 /* ---------------------------------------------------------------- zfp fixed-rate codec
  * Replaces ZfpCompressor::compress / ::decompress (custom/compressor/zfpc.cpp:23-86), i.e.
  * zfp_compress / zfp_decompress of the third-party zfp library in fixed-rate mode on fp32.

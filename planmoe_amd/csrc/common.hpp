@@ -70,47 +70,27 @@ typedef uint32_t pm_u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t pm_u32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ void stream_store(uint4 *p, const uint4 &v)
 {
-#ifdef PM_NO_STREAM_STORES
-    *p = v;
-#else
     __builtin_nontemporal_store(pm_u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<pm_u32x4 *>(p));
-#endif
 }
 __device__ __forceinline__ void stream_store(uint2 *p, const uint2 &v)
 {
-#ifdef PM_NO_STREAM_STORES
-    *p = v;
-#else
     __builtin_nontemporal_store(pm_u32x2{v.x, v.y}, reinterpret_cast<pm_u32x2 *>(p));
-#endif
 }
 __device__ __forceinline__ void stream_store(uint32_t *p, uint32_t v)
 {
-#ifdef PM_NO_STREAM_STORES
-    *p = v;
-#else
     __builtin_nontemporal_store(v, p);
-#endif
 }
 
 // Streaming loads for inputs read exactly once; used where measurement showed a gain.
 __device__ __forceinline__ uint4 stream_load(const uint4 *p)
 {
-#ifdef PM_NO_STREAM_LOADS
-    return *p;
-#else
     const pm_u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const pm_u32x4 *>(p));
     return make_uint4(v.x, v.y, v.z, v.w);
-#endif
 }
 __device__ __forceinline__ uint2 stream_load(const uint2 *p)
 {
-#ifdef PM_NO_STREAM_LOADS
-    return *p;
-#else
     const pm_u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const pm_u32x2 *>(p));
     return make_uint2(v.x, v.y);
-#endif
 }
 
 template <int DT> struct Elem;

@@ -36,22 +36,6 @@ __device__ unsigned long long fs_trace[1024 * 16];
 #define FS_STAMP(i) do { } while (0)
 #endif
 
-#ifdef PM_FS_NT_LOADS
-#define FS_LOAD(p) stream_load(p)
-#else
-#define FS_LOAD(p) (*(p))
-#endif
-
-#ifdef PM_FS_FENCE
-#define FS_SCHED_FENCE __builtin_amdgcn_sched_barrier(0)
-#else
-#define FS_SCHED_FENCE do { } while (0)
-#endif
-
-#ifndef FS_SPLIT
-#define FS_SPLIT 1
-#endif
-
 constexpr int FS_WAVES = 8;
 constexpr int FS_THREADS = FS_WAVES * WAVE;
 constexpr int FS_MAX_GROUPS = 512;          // work-groups the published tables are sized for
@@ -198,19 +182,15 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
             const uint4 *ahead = row_ptr(r + 2);
             auto body = [&](auto mode) {
 #pragma unroll
-                for (int h = 0; h < FS_SPLIT; ++h) {
-#pragma unroll
-                    for (int i = h * (NMMA / FS_SPLIT); i < (h + 1) * (NMMA / FS_SPLIT); ++i) {
-                        uint32_t wd[2];
-                        enc.template encode<decltype(mode)::value>(cur[i], wd);
-                        *reinterpret_cast<uint2 *>(my_park + r * 16 * G::RS + 32 * i) = make_uint2(wd[0], wd[1]);
-                    }
-                    // the half just coded takes its share of the row two rounds ahead
-                    FS_SCHED_FENCE;
-#pragma unroll
-                    for (int i = h * (NMMA / FS_SPLIT); i < (h + 1) * (NMMA / FS_SPLIT); ++i) cur[i] = FS_LOAD(ahead + 4 * i);
-                    FS_SCHED_FENCE;
+                for (int i = 0; i < NMMA; ++i) {
+                    uint32_t wd[2];
+                    enc.template encode<decltype(mode)::value>(cur[i], wd);
+                    *reinterpret_cast<uint2 *>(my_park + r * 16 * G::RS + 32 * i) = make_uint2(wd[0], wd[1]);
                 }
+                // (issuing these loads piecewise between the pieces of the encode costs registers
+                // that the compiler then takes from the resident gate weights)
+#pragma unroll
+                for (int i = 0; i < NMMA; ++i) cur[i] = ahead[4 * i];
             };
             if (__ballot(!enc.rq.fast) == 0) body(std::true_type{}); else body(std::false_type{});
         }
@@ -220,12 +200,12 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
     {
         const uint4 *p0 = row_ptr(0), *p1 = row_ptr(ROUNDS > 1 ? 1 : 0);
 #pragma unroll
-        for (int i = 0; i < NMMA; ++i) buf0[i] = FS_LOAD(p0 + 4 * i);
+        for (int i = 0; i < NMMA; ++i) buf0[i] = p0[4 * i];
 #pragma unroll
         for (int i = 0; i < NMMA; ++i) b[i] = bp[4 * i];
         if constexpr (ROUNDS > 1) {
 #pragma unroll
-            for (int i = 0; i < NMMA; ++i) buf1[i] = FS_LOAD(p1 + 4 * i);
+            for (int i = 0; i < NMMA; ++i) buf1[i] = p1[4 * i];
         }
     }
     round(std::integral_constant<int, 0>{}, buf0);

@@ -1,6 +1,6 @@
-"""Fused expert FFN -- mirror of the reference's experts/ffn.py (two batched library GEMMs
-with bias and activation).  It sits between dispatch and combine and is kept as a torch
-composite: only the data path around it is hand-written here."""
+"""Fused expert FFN -- mirror of the reference's experts/ffn.py (two batched GEMMs with bias and
+activation between dispatch and combine).  forward() is the torch composite of the reference;
+forward_from_codes() takes the int8 codes of the receive buffer straight into the first GEMM."""
 import torch
 
 
@@ -23,26 +23,42 @@ class FusedExpertsNetwork(torch.nn.Module):
         local_experts = ctx.num_local_experts
         hidden = self.hidden_size_per_expert
         out = self.output_dim or model_dim
-        fc1_w = torch.empty(1, local_experts, hidden, model_dim)
-        fc2_w = torch.empty(1, local_experts, hidden, out)
-        fc1_b = torch.empty(1, local_experts, hidden)
-        fc2_b = torch.empty(1, local_experts, out)
+        # parameter names and shapes as the reference's (ffn.py:33-56): fc1 [E, model_dim, hidden],
+        # fc2 [E, hidden, out], so that its state dicts load here
+        fc1_w = torch.empty(local_experts, model_dim, hidden)
+        fc2_w = torch.empty(local_experts, hidden, out)
+        fc1_b = torch.empty(local_experts, hidden)
+        fc2_b = torch.empty(local_experts, out)
         for i in range(local_experts):
             fc1 = torch.nn.Linear(model_dim, hidden)
             fc2 = torch.nn.Linear(hidden, out)
-            fc1_w[0, i], fc1_b[0, i] = fc1.weight, fc1.bias
-            fc2_w[0, i], fc2_b[0, i] = fc2.weight.t(), fc2.bias
-        self.batched_fc1_w = torch.nn.Parameter(fc1_w.squeeze(0))
-        self.batched_fc2_w = torch.nn.Parameter(fc2_w.squeeze(0))
-        self.batched_fc1_bias = torch.nn.Parameter(fc1_b.squeeze(0))
-        self.batched_fc2_bias = torch.nn.Parameter(fc2_b.squeeze(0))
+            fc1_w[i], fc1_b[i] = fc1.weight.t(), fc1.bias
+            fc2_w[i], fc2_b[i] = fc2.weight.t(), fc2.bias
+        self.batched_fc1_w = torch.nn.Parameter(fc1_w)
+        self.batched_fc2_w = torch.nn.Parameter(fc2_w)
+        self.batched_fc1_bias = torch.nn.Parameter(fc1_b)
+        self.batched_fc2_bias = torch.nn.Parameter(fc2_b)
+        self._fc1_k_major = None
 
     def forward(self, x, ctx):
-        w1 = self.batched_fc1_w.permute(0, 2, 1)
-        y = torch.add(torch.matmul(x, w1), self.batched_fc1_bias.unsqueeze(1))
+        y = torch.add(torch.matmul(x, self.batched_fc1_w), self.batched_fc1_bias.unsqueeze(1))
         y = self.activation_fn(y)
         y = torch.add(torch.matmul(y, self.batched_fc2_w), self.batched_fc2_bias.unsqueeze(1))
         return y
+
+    def forward_from_codes(self, codes, bias, scale):
+        """The same forward with the int8 codes of the receive buffer as input (inference: no autograd
+        through the first GEMM): planmoe_ffn_fc1_int8 decodes them inside the GEMM, so the decompressed
+        [E, C, model_dim] tensor is never written.  bf16; model_dim % 64 == 0, hidden % 128 == 0."""
+        from . import ops
+        w = self.batched_fc1_w
+        cached = self._fc1_k_major
+        if cached is None or cached[0] != w._version or cached[1].device != w.device or cached[1].dtype != w.dtype:
+            cached = (w._version, w.detach().transpose(1, 2).contiguous())      # [E, hidden, model_dim]
+            self._fc1_k_major = cached
+        y = ops.ffn_fc1_int8(codes, bias, scale, cached[1], self.batched_fc1_bias.detach())
+        y = self.activation_fn(y)
+        return torch.add(torch.matmul(y, self.batched_fc2_w), self.batched_fc2_bias.unsqueeze(1))
 
 
 ExpertModule = FusedExpertsNetwork

@@ -525,6 +525,31 @@ class ForwardInt8Plan:
         return self.out
 
 
+# ------------------------------------------------------------------------------ expert FFN on codes
+def ffn_fc1_int8(codes, bias, scale, weight_k_major, fc_bias=None, out=None):
+    """First GEMM of the expert FFN straight from int8 codes: codes uint8 [E, C, M], bias / scale
+    bf16 [E, C, 1] (what int8_compress returned), weight_k_major bf16 [E, H, M], fc_bias bf16
+    [E, H] or None -> bf16 [E, C, H] = decompress(codes) @ weight_k_major^T (+ fc_bias)."""
+    _need_gpu(codes, "ffn_fc1_int8")
+    E, C, M = codes.shape
+    H = weight_k_major.shape[1]
+    if bias.dtype != torch.bfloat16 or weight_k_major.dtype != torch.bfloat16:
+        raise PlanMoEError("ffn_fc1_int8: bf16 only")
+    if tuple(weight_k_major.shape) != (E, H, M):
+        raise PlanMoEError("ffn_fc1_int8: weight must be [experts, hidden, model_dim]")
+    codes, weight_k_major = _contig(codes, "ffn_fc1_int8"), _contig(weight_k_major, "ffn_fc1_int8")
+    bias, scale = _contig(bias, "ffn_fc1_int8"), _contig(scale, "ffn_fc1_int8")
+    if fc_bias is not None:
+        fc_bias = _contig(fc_bias.to(torch.bfloat16), "ffn_fc1_int8")
+    if out is None:
+        out = torch.empty((E, C, H), dtype=torch.bfloat16, device=codes.device)
+    elif tuple(out.shape) != (E, C, H) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise PlanMoEError("ffn_fc1_int8: out must be a contiguous bf16 [experts, rows, hidden] tensor")
+    check(lib.planmoe_ffn_fc1_int8(_ptr(codes), _ptr(bias), _ptr(scale), 1, _ptr(weight_k_major), _ptr(fc_bias),
+                                   E, C, M, H, _ptr(out), _stream(codes)))
+    return out
+
+
 # ------------------------------------------------------------------------------ zfp codec
 def zfp_stream_bytes(dims, nx, ny, rate=8.0):
     return int(lib.planmoe_zfp_stream_bytes(dims, nx, ny, float(rate)))
