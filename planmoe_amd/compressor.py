@@ -176,8 +176,25 @@ class LzCompressor(AbstractCompressor):
         self.g_flagArrGlobal, self.g_compressedDataGlobal = self.flagArrGlobal, self.compressedDataGlobal
 
 
+_registered = {}
+
+
+def register(name, factory):
+    """Add a compressor under `name`: factory(comm_ptr) -> AbstractCompressor.  Registered names
+    are looked up before the built-in ones, as in the C++ extension's registry."""
+    if not callable(factory):
+        raise TypeError("register: factory must be callable (a subclass of AbstractCompressor or a function of comm_ptr)")
+    _registered[str(name)] = factory
+
+
+def registered():
+    return sorted(_registered)
+
+
 def get_compressor(name, comm_ptr):
     # custom_kernel.cpp:194-207
+    if name in _registered:
+        return _registered[name](comm_ptr)
     if name == "int8":
         return Int8Compressor(comm_ptr)
     if name == "zfp":

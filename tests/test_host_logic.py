@@ -69,6 +69,31 @@ def test_registry_protocol_errors():
         lz.compress(torch.zeros(4, 4, 8, dtype=torch.bfloat16))
 
 
+def test_registered_compressor_is_found_before_the_built_in_names():
+    """A third-party subclass of the mirror's AbstractCompressor, added by name (the Python twin of
+    the C++ extension's registry), goes through compress / comm / decompress_operation."""
+    class Negate(compressor.NoCompressor):
+        def compress(self, input):
+            return super().compress(-input)
+
+        def decompress(self, input):
+            return -super().decompress(input)
+
+    compressor.clear_ptr_lst()
+    compressor.register("negate", Negate)
+    try:
+        assert "negate" in compressor.registered()
+        x = torch.arange(6.0)
+        sent = compressor.compress_operation(x, "negate", "naive")
+        assert torch.equal(sent, -x)
+        assert torch.equal(compressor.decompress_operation(compressor.comm_operation(sent)), x)
+        with pytest.raises(TypeError):
+            compressor.register("bad", 3)
+    finally:
+        compressor._registered.pop("negate", None)
+        compressor.clear_ptr_lst()
+
+
 def test_zfp_compressor_shape_check():
     c = compressor.ZfpCompressor(compressor.get_comm("naive"))
     assert c.compress_rate == 8.0
