@@ -818,19 +818,16 @@ static int run_dispatch_routed(const void *x, int dtype, int samples, int model_
 
 namespace pm {
 
-// every call draws a 64-bit ticket: a random salt per process in the upper half, a counter in the
-// lower.  The kernel mixes it into the tag of the words its work-groups publish (the other part is
-// the workspace's own launch counter), so that what an uninitialised workspace holds, or another
-// process left behind, does not pass for a word of this launch.
-static unsigned long long next_ticket()
+// a random number per process: the kernel adds it to the workspace's launch counter to form the tag
+// of the words its work-groups publish, so that what an uninitialised workspace holds, or another
+// process left behind, is unlikely to pass for a word of this launch
+static unsigned long long process_salt()
 {
     static const unsigned long long salt = [] {
         std::random_device rd;
-        return ((unsigned long long)rd() << 32) ^ 0x9e3779b900000000ull;
+        return ((unsigned long long)rd() << 32) | (unsigned long long)rd();
     }();
-    static std::atomic<unsigned long long> count{0};
-    const unsigned long long c = count.fetch_add(1) + 1;
-    return (salt & 0xffffffff00000000ull) | (c & 0xffffffffull);
+    return salt;
 }
 
 struct SingleShape { int nmma, rounds, groups; };
@@ -860,14 +857,14 @@ static int launch_single(int rounds, int groups, hipStream_t st, const void *x, 
                          float *l_aux, int32_t *counts, uint8_t *codes, void *bias_out, void *scale_out, void *ws,
                          int spin_limit, int32_t *gave_up)
 {
-    const unsigned long long ticket = next_ticket();
+    const unsigned long long salt = process_salt();
 #define PM_FS(ROUNDS)                                                                                     \
     do {                                                                                                  \
         if (!single_fits<SDT, CAP, NMMA, ROUNDS>(groups)) return 2;                                       \
         forward_single_kernel<SDT, CAP, NMMA, ROUNDS><<<groups, FS_THREADS, 0, st>>>(                     \
             (const uint4 *)x, (const uint4 *)wg, bias, samples, experts, k, normalize, capacity, indices, \
             locations, gates, stride, logits_out, scores_out, l_aux, counts, codes, bias_out, scale_out,  \
-            ws, ticket, spin_limit, gave_up);                                                             \
+            ws, salt, spin_limit, gave_up);                                                               \
     } while (0)
     switch (rounds) {
     case 1: PM_FS(1); break;

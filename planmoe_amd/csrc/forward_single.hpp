@@ -16,11 +16,14 @@
 // sums).  A word is written by one atomic store and read by one atomic load, so there is no
 // ordering between words to enforce, no cache write-back or invalidation, and nothing to clear
 // between launches: a word of an earlier launch, or whatever an uninitialised workspace holds,
-// does not carry the tag.  The tag is the workspace's launch counter + 1 (mixed with a ticket the
-// host draws per call).  Every work-group reads the counter first thing; the last group stores
-// counter + 1 at its very end, by when every group has published, hence started, hence read the
-// old value.  So the counter needs no initial value, and replays of a captured launch, whose
-// arguments never change, still get a tag of their own each.
+// does not carry the tag.  The tag is the workspace's launch counter + 1, plus a salt the host
+// draws once per process.  Launches on one workspace follow each other in stream order and each
+// adds one to the counter, so no two of them share a tag, whatever mixture of eager calls and
+// replays of a captured launch they are (a per-call number mixed in would break exactly that: two
+// numbers that both grow by one can cancel).  Every work-group reads the counter first thing; the
+// last group stores counter + 1 at its very end, by when every group has published, hence
+// started, hence read the old value.  So the counter needs no initial value, and replays of a
+// captured launch, whose arguments never change, still get a tag of their own each.
 //
 // Replaces gates/top.py:20-26 + moe_layer.py:230-256 + fast_dispatch.py:140-201 +
 // Int8Compressor::compress (int8.cpp:7-44), like the two-launch chain.
@@ -39,14 +42,20 @@ __device__ unsigned long long fs_trace[1024 * 16];
 constexpr int FS_WAVES = 8;
 constexpr int FS_THREADS = FS_WAVES * WAVE;
 constexpr int FS_MAX_GROUPS = 512;          // work-groups the published tables are sized for
+constexpr int FS_ZERO_ROWS = 8;             // empty slots per ticket
+constexpr int FS_SHARE = 8;                 // work-groups that share a ticket counter
+constexpr int FS_COUNTER_STRIDE = 128;      // bytes between ticket counters (a cache line each)
 
 // waits for LDS traffic only: loads and stores to global memory that are in flight stay in flight
 // across the barrier (__syncthreads would drain them)
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// the one-launch kernel's part of the workspace: the launch counter, then from byte 256 the
-// published words hist[groups][CAP] (4 planes x CAP experts, four counts per word), me[groups][CAP]
-constexpr size_t FS_PUB_OFFSET = 256;
+// the one-launch kernel's part of the workspace: the launch counter at byte 0, from byte 256 the
+// ticket counters of the empty slots, one per FS_SHARE work-groups (none of these needs an initial
+// value), then the published words hist[groups][CAP] (4 planes x CAP experts, four counts per
+// word), me[groups][CAP]
+constexpr size_t FS_COUNTER_OFFSET = 256;
+constexpr size_t FS_PUB_OFFSET = FS_COUNTER_OFFSET + (size_t)(FS_MAX_GROUPS / FS_SHARE) * FS_COUNTER_STRIDE;
 __host__ __device__ inline size_t fs_pub_bytes(int groups) { return FS_PUB_OFFSET + (size_t)groups * (16 + 16) * 8; }
 
 template <int NMMA> struct FsGeom {
@@ -71,7 +80,7 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
     int32_t *__restrict__ indices, int32_t *__restrict__ locations, void *__restrict__ gates, int64_t stride,
     void *__restrict__ logits_out, void *__restrict__ scores_out, float *__restrict__ l_aux,
     int32_t *__restrict__ counts_out, uint8_t *__restrict__ codes, void *__restrict__ bias_out,
-    void *__restrict__ scale_out, void *__restrict__ workspace, unsigned long long ticket, int spin_limit,
+    void *__restrict__ scale_out, void *__restrict__ workspace, unsigned long long salt, int spin_limit,
     int32_t *__restrict__ gave_up)
 {
     using S = Elem<SDT>;
@@ -99,6 +108,8 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
     __shared__ int32_t s_full[4][CAP], s_base[4][CAP], s_tot[CAP];
     __shared__ float s_mepart[FS_THREADS / CAP][CAP];
     __shared__ int s_vote[2][FS_WAVES];
+    __shared__ int32_t s_zbeg[CAP + 1], s_used[CAP];       // empty slots: first list index and first slot per expert
+    __shared__ int s_zdone;
 
     const int tid = threadIdx.x, w = tid >> 6, lane = lane_id(), m = lane & 15, g = lane >> 4;
     const int groups = gridDim.x, grp = blockIdx.x, t0 = grp * TOK;
@@ -106,9 +117,16 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
     unsigned long long *pub_hist = reinterpret_cast<unsigned long long *>((char *)workspace + FS_PUB_OFFSET);
     unsigned long long *pub_me = pub_hist + (size_t)groups * HW;
     const unsigned long long launch = __hip_atomic_load(launches, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
-    const uint32_t tag = (uint32_t)launch ^ (uint32_t)(ticket ^ (ticket >> 32));
+    const uint32_t tag = (uint32_t)launch + (uint32_t)(salt ^ (salt >> 32));
+    // tickets for the empty slots are drawn from a counter that only ever grows: what it holds now
+    // is this launch's zero (no group draws before every group has published, i.e. has been here)
+    // (32 bits, used modulo 2^32: only differences to the value read here matter)
+    uint32_t *zero_tickets = reinterpret_cast<uint32_t *>((char *)workspace + FS_COUNTER_OFFSET +
+                                                          (size_t)(grp / FS_SHARE) * FS_COUNTER_STRIDE);
+    const uint32_t zero_base = __hip_atomic_load(zero_tickets, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const float eps = SDT == PLANMOE_F32 ? 1.1920928955078125e-07f : SDT == PLANMOE_BF16 ? 0.0078125f : 0.0009765625f;
     if (tid < HW) { s_before64[tid] = 0; s_full64[tid] = 0; }
+    if (tid == 0) s_zdone = 0;
 
     // lane (m, g) of wave w holds, of row m of a round, the vectors  w * 4 NMMA + 4 i + g
     const int v0 = w * (4 * NMMA) + g;
@@ -388,6 +406,21 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
             taken += ful;
         }
         s_tot[tid] = taken;
+        // the empty slots of all experts as one list, expert after expert
+        int zbefore = 0, zown = 0;
+        for (int ee = 0; ee < CAP; ++ee) {
+            int tt = 0;
+            for (int j = 0; j < 4; ++j) {
+                const int idx = j * CAP + ee;
+                tt += (int)((s_full64[idx / 4] >> (16 * (idx % 4))) & 0xffffu);
+            }
+            const int z = ee < experts ? capacity - min(tt, capacity) : 0;
+            if (ee < tid) zbefore += z;
+            if (ee == tid) zown = z;
+        }
+        s_zbeg[tid] = zbefore;
+        s_used[tid] = capacity - zown;
+        if (tid == CAP - 1) s_zbeg[CAP] = zbefore + zown;
     }
     lds_barrier();
     FS_STAMP(8);
@@ -435,16 +468,50 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
             if (__ballot(!enc.rq.fast) == 0) body(std::true_type{}); else body(std::false_type{});
         }
     };
-    // empty slots: zero rows, dealt out over all waves of the grid
-    auto zero_fill = [&]() {
-        const int slots = experts * capacity, nwaves = groups * FS_WAVES;
-        for (int s = grp * FS_WAVES + w; s < slots; s += nwaves) {
-            const int e = s / capacity;
-            if (s - e * capacity < s_tot[e]) continue;
-            uint4 *dst = reinterpret_cast<uint4 *>(codes + (int64_t)s * G::M) + lane;
+    // empty slots: zero rows.  Which compute units get their rows out first differs by several
+    // microseconds, mostly from one XCD to the next, so the list of empty slots is dealt out by
+    // tickets, FS_ZERO_ROWS rows each, to whoever is done with its own rows: FS_SHARE consecutive
+    // work-groups (one per XCD) share a counter and a stretch of the list.  A ticket is drawn before
+    // the rows of the one before are written; the first wave of a group that finds the stretch
+    // exhausted tells the others, who then need not ask.  (One counter for the whole grid does not
+    // do: a few thousand additions to one address take longer than the stores.)
+    // The pointer is passed through a vector register: with an address it can prove uniform the
+    // compiler rewrites the addition into its own one-lane form, which waits for the answer on the spot.
+    typedef __attribute__((address_space(1))) uint32_t global_u32;
+    global_u32 *zero_tickets_v = (global_u32 *)zero_tickets;
+    asm volatile("" : "+v"(zero_tickets_v));
+    auto draw = [&]() {
+        uint32_t got = 0;
+        if (lane == 0) got = __hip_atomic_fetch_add(zero_tickets_v, (uint32_t)FS_ZERO_ROWS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return got;
+    };
+    // the answer to a draw is looked at only after the stores that follow it have been issued
+    auto drawn = [&](uint32_t got) {
+        asm volatile("" : "+v"(got) : : "memory");
+        return (uint32_t)__builtin_amdgcn_readfirstlane((int)got) - zero_base;
+    };
+    auto zero_row = [&](uint32_t idx) {
+        const int e = __popcll(__ballot(lane >= 1 && lane < CAP && (uint32_t)s_zbeg[min(lane, CAP)] <= idx));
+        const int slot = e * capacity + s_used[e] + (int)(idx - (uint32_t)s_zbeg[e]);
+        uint4 *dst = reinterpret_cast<uint4 *>(codes + (int64_t)slot * G::M) + lane;
 #pragma unroll
-            for (int i = 0; i < G::RV; ++i) stream_store(dst + i * WAVE, make_uint4(0u, 0u, 0u, 0u));
-            if (lane == 0) { B16::store(bias_out, s, 0.f); B16::store(scale_out, s, 0.f); }
+        for (int i = 0; i < G::RV; ++i) stream_store(dst + i * WAVE, make_uint4(0u, 0u, 0u, 0u));
+        if (lane == 0) { B16::store(bias_out, slot, 0.f); B16::store(scale_out, slot, 0.f); }
+    };
+    auto zero_fill = [&]() {
+        const uint32_t total = (uint32_t)s_zbeg[CAP];
+        const uint32_t shares = (uint32_t)(groups + FS_SHARE - 1) / FS_SHARE, per = (total + shares - 1) / shares;
+        const uint32_t lo = (uint32_t)(grp / FS_SHARE) * per, hi = min(lo + per, total);
+        if (lo >= hi) return;
+        uint32_t cur = lo + drawn(draw());
+        while (cur < hi) {
+            const bool ask = __hip_atomic_load(&s_zdone, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == 0;
+            uint32_t ticket = 0;
+            if (ask) ticket = draw();
+#pragma unroll
+            for (int r = 0; r < FS_ZERO_ROWS; ++r) zero_row(min(cur + r, hi - 1));      // past the end: the last row once more
+            cur = ask ? lo + drawn(ticket) : hi;
+            if (cur >= hi && lane == 0) __hip_atomic_store(&s_zdone, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
     };
 
