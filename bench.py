@@ -418,6 +418,46 @@ def layer_table():
         print("%-4s %-6s %-9s %14.3f %14.3f" % (cfg, codec, str(dtype).replace("torch.", ""), times[0], times[1]))
 
 
+def overlap_run(passes=6):
+    """The reference's pipeline (one entry point per step) around identity experts with the comm
+    step copying on the comm stream, at a2a_ffn_overlap_degree 1 and 2, forward only, config 2 with
+    the int8 compressor.  Meant to be run under `rocprofv3 --kernel-trace --memory-copy-trace`: at
+    degree 2 the copy of a chunk (comm stream) lies beside the compress of the next chunk."""
+    import torch
+    import planmoe_amd
+    from planmoe_amd import overlap, compressor
+    dev = "cuda:0"
+
+    class Identity(torch.nn.Module):
+        def update(self, ctx):
+            self.dummy = torch.nn.Parameter(torch.zeros(1))
+
+        def forward(self, x, ctx):
+            return x
+
+    T, M, E, k, cf = 16384, 4096, 8, 2, 1.25
+    overlap.FUSE_INT8 = overlap.FUSE_GATE = overlap.FUSE_ZFP = False
+    compressor.SINGLE_RANK_COMM_COPIES = True
+    x = torch.randn(T, M, generator=torch.Generator().manual_seed(0)).bfloat16().to(dev)
+    outs = []
+    for degree in (1, 2):
+        layer = planmoe_amd.moe_layer({'type': 'top', 'k': k, 'capacity_factor': cf, 'fp32_gate': True}, M,
+                                      experts={'type': 'custom', 'module': Identity(), 'count_per_node': E},
+                                      seeds=(1, 2, 3), compress_name="int8", a2a_ffn_overlap_degree=degree).to(dev).to(torch.bfloat16)
+        scrub = torch.zeros((1 << 28,), dtype=torch.int32, device=dev)
+        with torch.no_grad():
+            def step():
+                # two passes over 1 GiB first: while the GPU is busy with them the host enqueues the whole
+                # layer, so that the trace shows what the streams allow and not how fast Python is
+                torch.max(scrub), torch.max(scrub)
+                return layer(x)
+            avg, med, best = event_time_us(step, passes, 2, rounds=3)
+            outs.append(step())
+        torch.cuda.synchronize()
+        print("a2a_ffn_overlap_degree %d: 2 GiB of reads + forward %.1f us (median of 3 rounds of %d passes)" % (degree, med, passes), flush=True)
+    print("outputs of degree 2 equal to degree 1:", bool(torch.equal(outs[0], outs[1])))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -434,6 +474,9 @@ def main():
     ap.add_argument("--layer", action="store_true",
                     help="instead of the JSON line, time moe_layer forward + backward with identity experts for "
                          "every compressor, with and without the fused entry points")
+    ap.add_argument("--overlap", action="store_true",
+                    help="instead of the JSON line, run the step-by-step int8 pipeline with the comm copy on the "
+                         "comm stream at a2a_ffn_overlap_degree 1 and 2 (to be traced with rocprofv3)")
     ap.add_argument("--cpu-stages", action="store_true",
                     help="instead of the JSON line, time the CPU oracle (one thread) stage by stage on bounded "
                          "samples of the same workloads; needs no GPU")
@@ -447,13 +490,15 @@ def main():
         __graft_entry__.ensure_built()
         cpu_stage_table()
         return
-    if args.kernels or args.layer:
+    if args.kernels or args.layer or args.overlap:
         import __graft_entry__
         __graft_entry__.ensure_built()
         if args.kernels:
             kernel_table(args.only)
-        else:
+        elif args.layer:
             layer_table()
+        else:
+            overlap_run()
         return
 
     import __graft_entry__
