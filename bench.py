@@ -202,7 +202,10 @@ def kernel_table(only=None):
     fb = torch.zeros(E, Hf, dtype=torch.bfloat16, device=dev)
     fout = torch.empty(E, C, Hf, dtype=torch.bfloat16, device=dev)
     add("ffn_fc1_int8 (GEMM from codes)", "2", R * M + R * 4 + E * Hf * M * 2 + R * Hf * 2,
-        lambda: ops.ffn_fc1_int8(codes, b, s_, wk, fb, out=fout), iters=5)
+        lambda: ops.ffn_fc1_int8(codes.view(E, C, M), b.view(E, C, 1), s_.view(E, C, 1), wk, fb, out=fout), iters=5)
+    wcs = ops.ffn_weight_colsum(wk)
+    add("ffn_fc1_int8_affine (GEMM on codes)", "2", R * M + R * 4 + E * Hf * M * 2 + R * Hf * 2,
+        lambda: ops.ffn_fc1_int8_affine(codes.view(E, C, M), b.view(E, C, 1), s_.view(E, C, 1), wk, wcs, fb, out=fout), iters=5)
     ffn_flops = 2.0 * R * M * Hf
     del d, dc, codes, plan, plan1, wk, fout
 
@@ -275,14 +278,14 @@ def kernel_table(only=None):
         out = torch.empty_like(buf)
         add("lz_decompress %s" % label, "5", buf.numel() * 4 + used, lambda: ops.lz_decompress(out, fo, do, fl, da), iters=5)
 
-    print("%-30s %-4s %10s %9s %9s %8s %6s %10s %10s" % ("entry point", "cfg", "alg MB", "avg us", "best us", "GB/s", "frac",
+    print("%-36s %-4s %10s %9s %9s %8s %6s %10s %10s" % ("entry point", "cfg", "alg MB", "avg us", "best us", "GB/s", "frac",
                                                          "cold-r us", "cold-w us"))
     for name, cfg, nbytes, avg, best, cold_r, cold_w in rows:
         gbs = nbytes / avg / 1e3
-        print("%-30s %-4s %10.1f %9.1f %9.1f %8.0f %6.2f %10.1f %10.1f" % (name, cfg, nbytes / 1e6, avg, best, gbs,
+        print("%-36s %-4s %10.1f %9.1f %9.1f %8.0f %6.2f %10.1f %10.1f" % (name, cfg, nbytes / 1e6, avg, best, gbs,
                                                                          gbs / HBM_PEAK_GBS, cold_r, cold_w))
         if name.startswith("ffn_fc1_int8"):
-            print("%-30s %-4s %10s %9s %9s %8.0f TFLOP/s = %.3f of the %.0f TFLOP/s dense bf16 MFMA peak" % (
+            print("%-36s %-4s %10s %9s %9s %8.0f TFLOP/s = %.3f of the %.0f TFLOP/s dense bf16 MFMA peak" % (
                 "  ^ as a GEMM", cfg, "", "", "", ffn_flops / avg / 1e6, ffn_flops / avg / 1e6 / 2500.0, 2500.0))
 
 

@@ -324,6 +324,20 @@ int planmoe_ffn_fc1_int8(const uint8_t *codes, const void *bias, const void *sca
                          const void *weight_k_major, const void *fc_bias, int experts, int rows,
                          int model_dim, int hidden, void *out, void *stream);
 
+/* The same step (int8.cpp:46-60 + experts/ffn.py:77) with the row's affine map taken out of the
+ * sum: the matrix cores multiply the codes themselves and the epilogue applies
+ *   out[e][r][n] = bf16( bf16( scale[e][r] / 255 * sum_k code[e][r][k] w[e][n][k]
+ *                              + bias[e][r] * weight_colsum[e][n] ) + fc_bias[e][n] )
+ * weight_colsum [experts, hidden] fp32 = sum over model_dim of weight_k_major, computed by the
+ * caller once per weight.  Skips the three bf16 roundings Int8Compressor::decompress applies to
+ * every element (and their arithmetic: fifteen instructions per two codes against three), so it
+ * agrees with decompress + GEMM to about one ulp of the bf16 result (tolerance-level parity) and is
+ * the faster of the two.  Same shape limits as planmoe_ffn_fc1_int8. */
+int planmoe_ffn_fc1_int8_affine(const uint8_t *codes, const void *bias, const void *scale, int dtype,
+                                const void *weight_k_major, const float *weight_colsum,
+                                const void *fc_bias, int experts, int rows, int model_dim, int hidden,
+                                void *out, void *stream);
+
 /* ---------------------------------------------------------------- zfp fixed-rate codec
  * Replaces ZfpCompressor::compress / ::decompress (custom/compressor/zfpc.cpp:23-86), i.e.
  * zfp_compress / zfp_decompress of the third-party zfp library in fixed-rate mode on fp32.

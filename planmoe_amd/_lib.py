@@ -76,6 +76,8 @@ SIGNATURES = {
                                                 c_size_t, c_void_p]),
     "planmoe_ffn_fc1_int8": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
                                      c_int, c_void_p, c_void_p]),
+    "planmoe_ffn_fc1_int8_affine": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                            c_int, c_int, c_void_p, c_void_p]),
     "planmoe_zfp_max_bytes": (c_size_t, [c_int, c_int64, c_int64, c_double]),
     "planmoe_zfp_stream_bytes": (c_size_t, [c_int, c_int64, c_int64, c_double]),
     "planmoe_zfp_compress": (c_int, [c_void_p, c_int, c_int64, c_int64, c_double, c_void_p, c_size_t,

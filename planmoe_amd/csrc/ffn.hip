@@ -21,10 +21,28 @@ namespace pm {
 
 constexpr int FFN_BM = 128, FFN_BN = 128, FFN_BK = 64;
 
+__device__ __forceinline__ uint32_t codes_to_bf16x2(uint32_t w, int first)
+{
+    // bf16 of two bytes of w: the upper halves of their fp32 conversions
+    const float lo = (float)((w >> (first ? 16 : 0)) & 0xffu), hi = (float)((w >> (first ? 24 : 8)) & 0xffu);
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+
+// AFFINE: the row's affine map is taken out of the sum,
+//   sum_k dec(r, k) w[n][k]  ~  (scale_r / 255) * sum_k code[r][k] w[n][k]  +  bias_r * sum_k w[n][k]
+// so the matrix cores multiply the codes themselves (0 .. 255 are exact in bf16; two instructions
+// per four codes instead of the decompressor's fifteen per two) and the epilogue applies scale, bias
+// and the column sums of the weights, which the caller computes once per weight.  What is lost are
+// the three bf16 roundings the decompressor applies to every element: the result differs by about an
+// ulp of the bf16 output (tolerance-level parity), where the other form multiplies exactly the
+// decompressor's values.  (A 256 x 256 tile with 128 x 128 per wave, which would halve the LDS
+// traffic per MFMA, was tried and is slower as compiled: the 256 accumulator registers per lane
+// end up half in the other register file and are copied in every step.)
+template <bool AFFINE>
 __global__ __launch_bounds__(256) void ffn_fc1_int8_kernel(
     const uint8_t *__restrict__ codes, const uint16_t *__restrict__ qbias, const uint16_t *__restrict__ qscale,
-    const uint16_t *__restrict__ w, const uint16_t *__restrict__ fc_bias, int rows, int K, int N,
-    uint16_t *__restrict__ out)
+    const uint16_t *__restrict__ w, const float *__restrict__ colsum, const uint16_t *__restrict__ fc_bias,
+    int rows, int K, int N, uint16_t *__restrict__ out)
 {
     using B16 = Elem<PLANMOE_BF16>;
     __shared__ uint4 smem[(FFN_BM + FFN_BN) * FFN_BK * 2 / 16];          // A tile, then B tile: 32 KB
@@ -56,10 +74,15 @@ __global__ __launch_bounds__(256) void ffn_fc1_int8_kernel(
         cb3 = *reinterpret_cast<const uint4 *>(bsrc + 3 * bstep + k0);
     };
     auto decode_chunk = [&](uint32_t lo, uint32_t hi, int j) {
-        float f[8];
-        dec.word(lo, f);
-        dec.word(hi, f + 4);
-        sA[ar * 8 + ((ah * 4 + j) ^ (ar & 7))] = B16::pack(f);
+        if constexpr (AFFINE) {
+            sA[ar * 8 + ((ah * 4 + j) ^ (ar & 7))] = make_uint4(codes_to_bf16x2(lo, 0), codes_to_bf16x2(lo, 1),
+                                                                 codes_to_bf16x2(hi, 0), codes_to_bf16x2(hi, 1));
+        } else {
+            float f[8];
+            dec.word(lo, f);
+            dec.word(hi, f + 4);
+            sA[ar * 8 + ((ah * 4 + j) ^ (ar & 7))] = B16::pack(f);
+        }
     };
     auto store_tile = [&]() {
         // 32 codes -> 32 bf16 values = 4 chunks of this row
@@ -115,12 +138,18 @@ __global__ __launch_bounds__(256) void ffn_fc1_int8_kernel(
     for (int j = 0; j < 4; ++j) {
         const int col = wn * 64 + j * 16 + m;
         const float fb = fc_bias ? B16::load(fc_bias, (int64_t)e * N + n0 + col) : 0.f;
+        const float cs = AFFINE ? colsum[(int64_t)e * N + n0 + col] : 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int row = wm * 64 + i * 16 + 4 * g + q;
-                float v = B16::round(acc[i][j][q]);                 // the matmul's own rounding
+                float v = acc[i][j][q];
+                if constexpr (AFFINE) {
+                    const int64_t gr = (int64_t)e * rows + min(r0 + row, rows - 1);
+                    v = B16::load(qscale, gr) * (1.0f / 255.0f) * v + B16::load(qbias, gr) * cs;
+                }
+                v = B16::round(v);                                  // the matmul's own rounding
                 if (fc_bias) v = v + fb;                            // torch.add in bf16
                 sC[row * FFN_BN + col] = (uint16_t)f32_to_bf16(v);
             }
@@ -139,6 +168,27 @@ __global__ __launch_bounds__(256) void ffn_fc1_int8_kernel(
 
 using namespace pm;
 
+extern "C" int planmoe_ffn_fc1_int8_affine(const uint8_t *codes, const void *bias, const void *scale, int dtype,
+                                           const void *weight_k_major, const float *weight_colsum, const void *fc_bias,
+                                           int experts, int rows, int model_dim, int hidden, void *out, void *stream)
+{
+    PM_REQUIRE(dtype == PLANMOE_BF16, "planmoe_ffn_fc1_int8_affine: bf16 only (got dtype tag %d)", dtype);
+    PM_REQUIRE(experts >= 0 && rows >= 0 && model_dim >= 1 && hidden >= 1, "planmoe_ffn_fc1_int8_affine: bad shape");
+    if (experts == 0 || rows == 0) return 0;
+    PM_REQUIRE(model_dim % FFN_BK == 0 && hidden % FFN_BN == 0,
+               "planmoe_ffn_fc1_int8_affine: model_dim must be a multiple of %d and hidden of %d (got %d, %d)", FFN_BK, FFN_BN,
+               model_dim, hidden);
+    PM_REQUIRE(codes && bias && scale && weight_k_major && weight_colsum && out, "planmoe_ffn_fc1_int8_affine: NULL argument");
+    PM_REQUIRE(aligned16(codes) && aligned16(weight_k_major) && aligned16(out), "planmoe_ffn_fc1_int8_affine: buffers must be 16-byte aligned");
+    PM_REQUIRE((rows + FFN_BM - 1) / FFN_BM <= 65535 && experts <= 65535, "planmoe_ffn_fc1_int8_affine: too many row tiles or experts");
+    const dim3 grid((unsigned)(hidden / FFN_BN), (unsigned)((rows + FFN_BM - 1) / FFN_BM), (unsigned)experts);
+    ffn_fc1_int8_kernel<true><<<grid, 256, 0, (hipStream_t)stream>>>(
+        codes, (const uint16_t *)bias, (const uint16_t *)scale, (const uint16_t *)weight_k_major, weight_colsum,
+        (const uint16_t *)fc_bias, rows, model_dim, hidden, (uint16_t *)out);
+    PM_LAUNCH_CHECK("planmoe_ffn_fc1_int8_affine");
+    return 0;
+}
+
 extern "C" int planmoe_ffn_fc1_int8(const uint8_t *codes, const void *bias, const void *scale, int dtype,
                                     const void *weight_k_major, const void *fc_bias, int experts, int rows,
                                     int model_dim, int hidden, void *out, void *stream)
@@ -153,9 +203,9 @@ extern "C" int planmoe_ffn_fc1_int8(const uint8_t *codes, const void *bias, cons
     PM_REQUIRE(aligned16(codes) && aligned16(weight_k_major) && aligned16(out), "planmoe_ffn_fc1_int8: buffers must be 16-byte aligned");
     PM_REQUIRE((rows + FFN_BM - 1) / FFN_BM <= 65535 && experts <= 65535, "planmoe_ffn_fc1_int8: too many row tiles or experts");
     const dim3 grid((unsigned)(hidden / FFN_BN), (unsigned)((rows + FFN_BM - 1) / FFN_BM), (unsigned)experts);
-    ffn_fc1_int8_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(codes, (const uint16_t *)bias, (const uint16_t *)scale,
-                                                                 (const uint16_t *)weight_k_major, (const uint16_t *)fc_bias,
-                                                                 rows, model_dim, hidden, (uint16_t *)out);
+    ffn_fc1_int8_kernel<false><<<grid, 256, 0, (hipStream_t)stream>>>(
+        codes, (const uint16_t *)bias, (const uint16_t *)scale, (const uint16_t *)weight_k_major, nullptr,
+        (const uint16_t *)fc_bias, rows, model_dim, hidden, (uint16_t *)out);
     PM_LAUNCH_CHECK("planmoe_ffn_fc1_int8");
     return 0;
 }

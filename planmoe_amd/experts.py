@@ -46,17 +46,23 @@ class FusedExpertsNetwork(torch.nn.Module):
         y = torch.add(torch.matmul(y, self.batched_fc2_w), self.batched_fc2_bias.unsqueeze(1))
         return y
 
-    def forward_from_codes(self, codes, bias, scale):
+    def forward_from_codes(self, codes, bias, scale, exact=False):
         """The same forward with the int8 codes of the receive buffer as input (inference: no autograd
-        through the first GEMM): planmoe_ffn_fc1_int8 decodes them inside the GEMM, so the decompressed
-        [E, C, model_dim] tensor is never written.  bf16; model_dim % 64 == 0, hidden % 128 == 0."""
+        through the first GEMM): the GEMM reads the codes, so the decompressed [E, C, model_dim]
+        tensor is never written.  exact=False: planmoe_ffn_fc1_int8_affine (scale / bias in the
+        epilogue, about an ulp from decompress + GEMM); exact=True: planmoe_ffn_fc1_int8 (multiplies
+        the decompressor's very values).  bf16; model_dim % 64 == 0, hidden % 128 == 0."""
         from . import ops
         w = self.batched_fc1_w
         cached = self._fc1_k_major
         if cached is None or cached[0] != w._version or cached[1].device != w.device or cached[1].dtype != w.dtype:
-            cached = (w._version, w.detach().transpose(1, 2).contiguous())      # [E, hidden, model_dim]
+            wk = w.detach().transpose(1, 2).contiguous()                        # [E, hidden, model_dim]
+            cached = (w._version, wk, ops.ffn_weight_colsum(wk))
             self._fc1_k_major = cached
-        y = ops.ffn_fc1_int8(codes, bias, scale, cached[1], self.batched_fc1_bias.detach())
+        if exact:
+            y = ops.ffn_fc1_int8(codes, bias, scale, cached[1], self.batched_fc1_bias.detach())
+        else:
+            y = ops.ffn_fc1_int8_affine(codes, bias, scale, cached[1], cached[2], self.batched_fc1_bias.detach())
         y = self.activation_fn(y)
         return torch.add(torch.matmul(y, self.batched_fc2_w), self.batched_fc2_bias.unsqueeze(1))
 

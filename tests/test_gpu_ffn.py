@@ -81,4 +81,55 @@ def test_ffn_module_from_codes_equals_decompress_then_forward():
     with torch.no_grad():
         want = ffn(ops.int8_decompress(codes, bias, scale), layer)
         got = ffn.forward_from_codes(codes, bias, scale)
+        got_exact = ffn.forward_from_codes(codes, bias, scale, exact=True)
     assert torch.allclose(got.float(), want.float(), rtol=2e-2, atol=2e-2 * float(want.float().abs().max()))
+    assert torch.allclose(got_exact.float(), want.float(), rtol=2e-2, atol=2e-2 * float(want.float().abs().max()))
+
+
+@pytest.mark.parametrize("E,C,M,H,with_bias", [(2, 200, 256, 128, True), (3, 256, 64, 512, False), (1, 1, 512, 256, True),
+                                               (2, 700, 1024, 384, True)])
+def test_fc1_affine_against_the_oracle(E, C, M, H, with_bias):
+    """planmoe_ffn_fc1_int8_affine: codes on the matrix cores, scale / bias in the epilogue.  Against the
+    oracle's decode + fp64 product with the same bf16 tolerance as the exact-decode kernel (the three
+    roundings of the decompressor that it skips are of that size), and against that kernel."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(E * 1000 + C)
+    x = torch.randn(E, C, M, generator=g).bfloat16()
+    x[0, 0] = 0.0
+    w = (torch.randn(E, H, M, generator=g) * M ** -0.5).bfloat16()
+    fb = torch.randn(E, H, generator=g).bfloat16() if with_bias else None
+    codes, bias, scale = ops.int8_compress(x.to(DEV))
+    wd = w.to(DEV)
+    got = ops.ffn_fc1_int8_affine(codes, bias, scale, wd, ops.ffn_weight_colsum(wd), fb.to(DEV) if with_bias else None).float().cpu()
+    rc, rb, rs = oracle.int8_compress(bf16_bits(x))
+    dec = from_bf16_bits(oracle.int8_decompress(rc, rb, rs)).double()
+    ref = torch.einsum("ecm,ehm->ech", dec, w.double())
+    mag = torch.einsum("ecm,ehm->ech", dec.abs(), w.double().abs())
+    if with_bias:
+        ref = ref + fb.double()[:, None, :]
+        mag = mag + fb.double().abs()[:, None, :]
+    assert ((got.double() - ref).abs() <= 1e-2 * ref.abs() + 2.0 ** -7 * mag + 1e-30).all()
+    exact = ops.ffn_fc1_int8(codes, bias, scale, wd, fb.to(DEV) if with_bias else None).float().cpu()
+    assert ((got - exact).abs().double() <= 1e-2 * ref.abs() + 2.0 ** -7 * mag + 1e-30).all()
+    assert float((got[0, 0] - (fb[0].float() if with_bias else 0.0)).abs().max()) == 0.0     # the empty slot: bias only
+
+
+def test_fc1_affine_config2_shape():
+    from planmoe_amd import ops
+    E, C, M, H = 8, 5120, 4096, 4096
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(E, C, M, generator=g).bfloat16()
+    w = (torch.randn(E, H, M, generator=g) * M ** -0.5).bfloat16()
+    fb = torch.randn(E, H, generator=g).bfloat16()
+    codes, bias, scale = ops.int8_compress(x.to(DEV))
+    wd = w.to(DEV)
+    got = ops.ffn_fc1_int8_affine(codes, bias, scale, wd, None, fb.to(DEV))
+    torch.cuda.synchronize()
+    rows = torch.tensor([0, 1, 127, 128, 255, 256, 2559, 2560, 4000, 5118, 5119])
+    sample = got[:, rows].float().cpu().double()
+    rc, rb, rs = oracle.int8_compress(bf16_bits(x[:, rows].contiguous()))
+    dec = from_bf16_bits(oracle.int8_decompress(rc, rb, rs)).double()
+    ref = torch.einsum("ecm,ehm->ech", dec, w.double()) + fb.double()[:, None, :]
+    mag = torch.einsum("ecm,ehm->ech", dec.abs(), w.double().abs()) + fb.double().abs()[:, None, :]
+    assert ((sample - ref).abs() <= 1e-2 * ref.abs() + 2.0 ** -7 * mag).all()
+    assert bool(torch.isfinite(got.float()).all()) and float(got.float().abs().sum(dim=2).min()) > 0
