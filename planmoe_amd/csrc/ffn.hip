@@ -35,9 +35,10 @@ __device__ __forceinline__ uint32_t codes_to_bf16x2(uint32_t w, int first)
 // and the column sums of the weights, which the caller computes once per weight.  What is lost are
 // the three bf16 roundings the decompressor applies to every element: the result differs by about an
 // ulp of the bf16 output (tolerance-level parity), where the other form multiplies exactly the
-// decompressor's values.  (A 256 x 256 tile with 128 x 128 per wave, which would halve the LDS
-// traffic per MFMA, was tried and is slower as compiled: the 256 accumulator registers per lane
-// end up half in the other register file and are copied in every step.)
+// decompressor's values.  (Larger tiles, which would cut the LDS traffic per MFMA, were tried and
+// are slower as compiled: 256 x 256 with 128 x 128 per wave keeps half of its 256 accumulator
+// registers in the other register file and copies them in every step, 340 TFLOP/s; 256 x 128 with
+// 128 x 64 per wave takes 304 registers, one wave per SIMD, 476 TFLOP/s.)
 template <bool AFFINE>
 __global__ __launch_bounds__(256) void ffn_fc1_int8_kernel(
     const uint8_t *__restrict__ codes, const uint16_t *__restrict__ qbias, const uint16_t *__restrict__ qscale,
