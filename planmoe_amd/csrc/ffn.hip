@@ -40,7 +40,7 @@ __device__ __forceinline__ uint32_t codes_to_bf16x2(uint32_t w, int first)
 // registers in the other register file and copies them in every step, 340 TFLOP/s; 256 x 128 with
 // 128 x 64 per wave takes 304 registers, one wave per SIMD, 476 TFLOP/s.)
 template <bool AFFINE>
-__global__ __launch_bounds__(256) void ffn_fc1_int8_kernel(
+__global__ __launch_bounds__(256, 3) void ffn_fc1_int8_kernel(
     const uint8_t *__restrict__ codes, const uint16_t *__restrict__ qbias, const uint16_t *__restrict__ qscale,
     const uint16_t *__restrict__ w, const float *__restrict__ colsum, const uint16_t *__restrict__ fc_bias,
     int rows, int K, int N, uint16_t *__restrict__ out)
@@ -59,20 +59,21 @@ __global__ __launch_bounds__(256) void ffn_fc1_int8_kernel(
     const RowDecoder<PLANMOE_BF16> dec(B16::load(qbias, (int64_t)e * rows + arow), B16::load(qscale, (int64_t)e * rows + arow));
     const uint16_t *wp = w + ((int64_t)e * N + n0) * K;
 
-    // (four named registers for the weight chunks: an array indexed inside these helpers ends up in
-    // private memory)
-    uint4 ca0, ca1, cb0, cb1, cb2, cb3;
+    // What a thread fetches of one k-tile.  Two sets: the loads of a tile are issued two tiles ahead,
+    // since one tile's MFMAs (512 cycles per wave, three work-groups per CU) do not cover the latency
+    // of a load.  (Named members: an array indexed inside these helpers ends up in private memory.)
+    struct Fetched { uint4 ca0, ca1, cb0, cb1, cb2, cb3; } f0, f1;
     const int brow = tid >> 3, bc = tid & 7;                         // chunk tid + 256 i: row brow + 32 i, chunk bc
     const uint16_t *bsrc = wp + (int64_t)brow * K + bc * 8;
     const int64_t bstep = (int64_t)32 * K;
-    auto load_tile = [&](int kt) {
+    auto load_tile = [&](Fetched &f, int kt) {
         const int k0 = kt * FFN_BK;
-        ca0 = *reinterpret_cast<const uint4 *>(ap + k0);
-        ca1 = *reinterpret_cast<const uint4 *>(ap + k0 + 16);
-        cb0 = *reinterpret_cast<const uint4 *>(bsrc + k0);
-        cb1 = *reinterpret_cast<const uint4 *>(bsrc + bstep + k0);
-        cb2 = *reinterpret_cast<const uint4 *>(bsrc + 2 * bstep + k0);
-        cb3 = *reinterpret_cast<const uint4 *>(bsrc + 3 * bstep + k0);
+        f.ca0 = *reinterpret_cast<const uint4 *>(ap + k0);
+        f.ca1 = *reinterpret_cast<const uint4 *>(ap + k0 + 16);
+        f.cb0 = *reinterpret_cast<const uint4 *>(bsrc + k0);
+        f.cb1 = *reinterpret_cast<const uint4 *>(bsrc + bstep + k0);
+        f.cb2 = *reinterpret_cast<const uint4 *>(bsrc + 2 * bstep + k0);
+        f.cb3 = *reinterpret_cast<const uint4 *>(bsrc + 3 * bstep + k0);
     };
     auto decode_chunk = [&](uint32_t lo, uint32_t hi, int j) {
         if constexpr (AFFINE) {
@@ -85,32 +86,28 @@ __global__ __launch_bounds__(256) void ffn_fc1_int8_kernel(
             sA[ar * 8 + ((ah * 4 + j) ^ (ar & 7))] = B16::pack(f);
         }
     };
-    auto store_tile = [&]() {
+    auto store_tile = [&](const Fetched &f) {
         // 32 codes -> 32 bf16 values = 4 chunks of this row
-        decode_chunk(ca0.x, ca0.y, 0);
-        decode_chunk(ca0.z, ca0.w, 1);
-        decode_chunk(ca1.x, ca1.y, 2);
-        decode_chunk(ca1.z, ca1.w, 3);
+        decode_chunk(f.ca0.x, f.ca0.y, 0);
+        decode_chunk(f.ca0.z, f.ca0.w, 1);
+        decode_chunk(f.ca1.x, f.ca1.y, 2);
+        decode_chunk(f.ca1.z, f.ca1.w, 3);
         // rows brow + 32 i share brow & 7, hence the chunk's place
         const int place = bc ^ (brow & 7);
-        sB[brow * 8 + place] = cb0;
-        sB[(brow + 32) * 8 + place] = cb1;
-        sB[(brow + 64) * 8 + place] = cb2;
-        sB[(brow + 96) * 8 + place] = cb3;
+        sB[brow * 8 + place] = f.cb0;
+        sB[(brow + 32) * 8 + place] = f.cb1;
+        sB[(brow + 64) * 8 + place] = f.cb2;
+        sB[(brow + 96) * 8 + place] = f.cb3;
     };
 
+    const int KT = K / FFN_BK;
     f32x4 acc[4][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int KT = K / FFN_BK;
-    load_tile(0);
-    for (int kt = 0; kt < KT; ++kt) {
-        store_tile();
-        __syncthreads();
-        if (kt + 1 < KT) load_tile(kt + 1);
+    auto multiply = [&]() {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             uint4 af[4], bf[4];
@@ -129,7 +126,20 @@ __global__ __launch_bounds__(256) void ffn_fc1_int8_kernel(
 #pragma unroll
                 for (int j = 0; j < 4; ++j) Mma<PLANMOE_BF16>::run(af[i], bf[j], acc[i][j]);
         }
+    };
+    auto step = [&](Fetched &f, int kt) {
+        store_tile(f);
         __syncthreads();
+        load_tile(f, min(kt + 2, KT - 1));          // (past the end: the last tile once more, never used)
+        multiply();
+        __syncthreads();
+    };
+
+    load_tile(f0, 0);
+    load_tile(f1, min(1, KT - 1));
+    for (int kt = 0; kt < KT; kt += 2) {
+        step(f0, kt);
+        if (kt + 1 < KT) step(f1, kt + 1);
     }
 
     // epilogue: the tile goes through LDS (the operand space, 128 x 128 bf16) so that it leaves in
