@@ -41,13 +41,15 @@ struct BitWriter {
     }
 };
 
-// The decoder looks at the stream by bit position: the block's words sit in LDS (NW + 1 words per
-// thread, the last one zero) and a look is two neighbouring words funnel-shifted, so there is no
-// refill state to carry and no branch in the reader.  Streams of one or two words stay in a
-// register pair that is shifted as bits are consumed.
+// The decoder looks at the stream by bit position: the block's words sit in LDS (NW words per
+// thread and three zero words behind them: an odd stride) and a look is neighbouring words
+// funnel-shifted, so there is no refill state to carry and no branch in the reader.  A bit plane
+// takes one look of 64 bits (a plane never uses more than 48) and is then parsed in registers.
+// Streams of one or two words stay in a register pair that is shifted as bits are consumed.
 template <int NW>
 struct BitReader {
-    const uint32_t *words;      // this thread's NW + 1 words in LDS
+    static constexpr int STRIDE = NW + 3;
+    const uint32_t *words;      // this thread's NW + 3 words in LDS
     int pos;
     uint64_t small;             // NW <= 2: the whole stream in a register pair instead
     __device__ __forceinline__ void init(uint32_t *lds, const uint32_t *w)
@@ -58,10 +60,12 @@ struct BitReader {
             if constexpr (NW == 2) small |= (uint64_t)w[1] << 32;
             words = nullptr;
         } else {
-            uint32_t *mine = lds + threadIdx.x * (NW + 1);
+            uint32_t *mine = lds + threadIdx.x * STRIDE;
 #pragma unroll
             for (int i = 0; i < NW; ++i) mine[i] = w[i];
             mine[NW] = 0u;
+            mine[NW + 1] = 0u;
+            mine[NW + 2] = 0u;
             words = mine;
             small = 0;
         }
@@ -76,7 +80,18 @@ struct BitReader {
             return __builtin_amdgcn_alignbit(words[i + 1], words[i], pos & 31);
         }
     }
-    __device__ __forceinline__ void skip(int n)      // n <= 32
+    // the next 64 bits
+    __device__ __forceinline__ uint64_t peek64() const
+    {
+        if constexpr (NW <= 2) {
+            return small;
+        } else {
+            const int i = pos >> 5, sh = pos & 31;
+            const uint32_t w0 = words[i], w1 = words[i + 1], w2 = words[i + 2];
+            return (uint64_t)__builtin_amdgcn_alignbit(w1, w0, sh) | ((uint64_t)__builtin_amdgcn_alignbit(w2, w1, sh) << 32);
+        }
+    }
+    __device__ __forceinline__ void skip(int n)      // n <= 32 (NW <= 2), any n otherwise
     {
         if constexpr (NW <= 2) small >>= n;
         else pos += n;
@@ -277,11 +292,11 @@ __device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f)
     int bits = 32 * NW - 9;
     int nsig = 0;
     auto read_plane = [&]() __attribute__((always_inline)) {
-        const int mm = min(nsig, bits);
-        bits -= mm;
-        uint32_t x = br.get(mm);
-        while (nsig < N && bits > 0) {
-            if constexpr (N == 4) {
+        if constexpr (N == 4) {
+            const int mm = min(nsig, bits);
+            bits -= mm;
+            uint32_t x = br.get(mm);
+            while (nsig < N && bits > 0) {
                 // tiny blocks: test bit and run are read separately (measured faster here)
                 --bits;
                 if (!br.get(1)) break;
@@ -292,21 +307,32 @@ __device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f)
                 br.skip(used); bits -= used; nsig += z;
                 x |= 1u << nsig;
                 ++nsig;
-                continue;
             }
-            // one look per segment: the test bit, then the zeros up to the next one bit (cut short
-            // by the budget or by the block's last value, whose one is implied)
-            const uint32_t look = br.peek();
-            if (!(look & 1u)) { br.skip(1); --bits; break; }
-            const int lim = min(N - 1 - nsig, bits - 1);
-            const uint32_t win = (look >> 1) & ((1u << lim) - 1u);
-            const int z = win != 0u ? __builtin_ctz(win) : lim;       // zeros read
-            const int used = 1 + (win != 0u ? z + 1 : lim);
-            br.skip(used); bits -= used; nsig += z;
-            x |= 1u << nsig;
-            ++nsig;
+            return x;
+        } else {
+            // one look at the stream per plane: nsig verbatim bits, then segment by segment the test
+            // bit and the zeros up to the next one bit (cut short by the budget or by the block's
+            // last value, whose one is implied), at most 16 + 32 bits in all
+            uint64_t look = br.peek64();
+            const int before = bits;
+            const int mm = min(nsig, bits);
+            bits -= mm;
+            uint32_t x = (uint32_t)look & ((1u << mm) - 1u);
+            look >>= mm;
+            while (nsig < N && bits > 0) {
+                const uint32_t lo = (uint32_t)look;
+                if (!(lo & 1u)) { --bits; break; }
+                const int lim = min(N - 1 - nsig, bits - 1);
+                const uint32_t win = (lo >> 1) & ((1u << lim) - 1u);
+                const int z = win != 0u ? __builtin_ctz(win) : lim;       // zeros read
+                const int used = 1 + (win != 0u ? z + 1 : lim);
+                look >>= used; bits -= used; nsig += z;
+                x |= 1u << nsig;
+                ++nsig;
+            }
+            br.skip(before - bits);
+            return x;
         }
-        return x;
     };
     if constexpr (N == 16) {
         // planes 31..16 are collected as rows and transposed into the coefficients' upper halves
@@ -401,7 +427,7 @@ __global__ __launch_bounds__(256) void zfp_decode1_kernel(const uint32_t *__rest
 {
     const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (b >= blocks) return;
-    __shared__ uint32_t lds[NW <= 2 ? 1 : (NW + 1) * 256];
+    __shared__ uint32_t lds[NW <= 2 ? 1 : BitReader<NW>::STRIDE * 256];
     uint32_t w[NW];
     load_words<NW>(in + b * NW, w);
     BitReader<NW> br;
@@ -640,7 +666,7 @@ __global__ __launch_bounds__(256) void zfp_decode2_kernel(const uint32_t *__rest
 {
     const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (b >= blocks) return;
-    __shared__ uint32_t lds[NW <= 2 ? 1 : (NW + 1) * 256];
+    __shared__ uint32_t lds[NW <= 2 ? 1 : BitReader<NW>::STRIDE * 256];
     uint32_t w[NW];
     load_words<NW>(in + b * NW, w);
     BitReader<NW> br;
@@ -738,7 +764,7 @@ __global__ __launch_bounds__(256) void combine_zfp2_kernel(const uint32_t *__res
 {
     const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (b >= blocks) return;
-    __shared__ uint32_t lds[NW <= 2 ? 1 : (NW + 1) * 256];
+    __shared__ uint32_t lds[NW <= 2 ? 1 : BitReader<NW>::STRIDE * 256];
     const int64_t by = b / nbx, bx = b - by * nbx;
     const int4 tok = *reinterpret_cast<const int4 *>(src + 4 * by);
     const int4 pl = *reinterpret_cast<const int4 *>(splane + 4 * by);
@@ -787,7 +813,7 @@ __global__ __launch_bounds__(256) void bwd_gate_zfp2_kernel(const uint32_t *__re
                                                            int64_t model_dim, int64_t nbx,
                                                            float *__restrict__ grad_gates)
 {
-    __shared__ uint32_t lds[NW <= 2 ? 1 : (NW + 1) * 256];
+    __shared__ uint32_t lds[NW <= 2 ? 1 : BitReader<NW>::STRIDE * 256];
     __shared__ float s_part[4][4];
     const int64_t by = blockIdx.x;
     const int4 tok = *reinterpret_cast<const int4 *>(src + 4 * by);
