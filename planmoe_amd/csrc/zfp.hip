@@ -466,16 +466,20 @@ __host__ __device__ constexpr uint32_t gt4_code(int nsig, uint32_t r)
     return code | ((uint32_t)len << 8) | ((uint32_t)(n - nsig) << 12);
 }
 
-// the inverse, for a stream whose next 7 bits are s and whose budget does not end inside the code:
-// plane bits (at their absolute positions) in bits 0..3, bits used in 4..7, newly significant in 8..10
-__host__ __device__ constexpr uint32_t gt4_parse(int nsig, uint32_t s)
+// the inverse, for a stream whose next 7 bits are s and of which `budget` >= 1 bits are left (7
+// stands for "7 or more": the longest code has 7 bits); the walk is zfp's own, budget checks
+// included.  Plane bits (at their absolute positions) in bits 0..3, bits used in 4..7, newly
+// significant values in 8..10
+__host__ __device__ constexpr uint32_t gt4_parse(int nsig, uint32_t s, int budget)
 {
     uint32_t x = 0;
-    int used = 0, n = nsig;
-    while (n < 4) {
+    int used = 0, n = nsig, bits = budget;
+    while (n < 4 && bits > 0) {
+        --bits;
         const uint32_t any = (s >> used) & 1u; ++used;
         if (!any) break;
-        while (n < 3) {
+        while (n < 3 && bits > 0) {
+            --bits;
             const uint32_t one = (s >> used) & 1u; ++used;
             if (one) break;
             ++n;
@@ -506,14 +510,14 @@ __device__ __forceinline__ void values_of(const uint32_t (&pl)[4], uint32_t (&u)
 // both tables worked out by the compiler; a work-group copies them into LDS
 struct Gt4Tables {
     uint32_t code[64];      // [nsig][plane bits]: code, length, newly significant values, a byte each
-    uint16_t parse[512];    // [nsig][next 7 stream bits]
+    uint16_t parse[7 * 512];    // [min(budget, 7) - 1][nsig][next 7 stream bits]
     constexpr Gt4Tables() : code(), parse()
     {
         for (int i = 0; i < 64; ++i) {
             const uint32_t e = gt4_code(i >> 4, (uint32_t)i & 15u);
             code[i] = (e & 0xffu) | (((e >> 8) & 15u) << 8) | ((e >> 12) << 16);
         }
-        for (int i = 0; i < 512; ++i) parse[i] = (uint16_t)gt4_parse(i >> 7, (uint32_t)i & 127u);
+        for (int i = 0; i < 7 * 512; ++i) parse[i] = (uint16_t)gt4_parse((i >> 7) & 3, (uint32_t)i & 127u, (i >> 9) + 1);
     }
 };
 __constant__ const Gt4Tables gt4_tables = Gt4Tables();
@@ -570,68 +574,68 @@ __global__ __launch_bounds__(256) void zfp_encode1_word_kernel(const float *__re
     out[b] = acc;
 }
 
+// blocks per thread: the parse table (7 KB) is copied into LDS once per work-group
+constexpr int ZD1_PER_THREAD = 4;
+
 __global__ __launch_bounds__(256) void zfp_decode1_word_kernel(const uint32_t *__restrict__ in, int64_t blocks,
                                                                float *__restrict__ field)
 {
-    __shared__ uint16_t tab[512];
-    for (int i = threadIdx.x; i < 512; i += 256) tab[i] = gt4_tables.parse[i];
+    __shared__ uint16_t tab[7 * 512];
+    {
+        const uint32_t *src = reinterpret_cast<const uint32_t *>(gt4_tables.parse);
+        uint32_t *dst = reinterpret_cast<uint32_t *>(tab);
+#pragma unroll
+        for (int i = 0; i < 7; ++i) dst[threadIdx.x + 256 * i] = src[threadIdx.x + 256 * i];
+    }
     __syncthreads();
-    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (b >= blocks) return;
-    const uint32_t w = in[b];
-    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (w & 1u) {
-        const int emax = (int)((w >> 1) & 0xffu) - 127;
-        uint32_t s = w >> 9;                                     // the 23 coded bits, zeros above them
-        uint32_t pl[4] = {0u, 0u, 0u, 0u};
-        int bits = 23, nsig = 0;
-        uint32_t sigmask = 0u;
-        // plane bits of one plane; reading past the budget reads zeros, as the budget's end demands
-        auto plane = [&]() __attribute__((always_inline)) {
-            uint32_t x = s & sigmask;
-            s >>= nsig; bits -= nsig;
-            if (nsig < 4 && bits > 0) {
-                const uint32_t e = tab[nsig * 128 + (int)(s & 127u)];
-                const int used = (int)((e >> 4) & 15u);
-                if (used <= bits) {                             // every bit the table looked at is the block's own
+    const int64_t b0 = (int64_t)blockIdx.x * (256 * ZD1_PER_THREAD) + threadIdx.x;
+    uint32_t win[ZD1_PER_THREAD];
+#pragma unroll
+    for (int it = 0; it < ZD1_PER_THREAD; ++it) win[it] = in[min(b0 + 256 * it, blocks - 1)];
+#pragma unroll
+    for (int it = 0; it < ZD1_PER_THREAD; ++it) {
+        const int64_t b = b0 + 256 * it;
+        if (b >= blocks) break;
+        const uint32_t w = win[it];
+        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (w & 1u) {
+            const int emax = (int)((w >> 1) & 0xffu) - 127;
+            uint32_t s = w >> 9;                                     // the 23 coded bits, zeros above them
+            uint32_t pl[4] = {0u, 0u, 0u, 0u};
+            int bits = 23, nsig = 0;
+            uint32_t sigmask = 0u;
+            // the bits of one plane: the verbatim ones (past the budget the register holds zeros, as the
+            // budget's end demands), then the group tests by table, whatever is left of the budget
+            auto plane = [&]() __attribute__((always_inline)) {
+                uint32_t x = s & sigmask;
+                s >>= nsig; bits -= nsig;
+                if (nsig < 4 && bits > 0) {
+                    const uint32_t e = tab[(min(bits, 7) - 1) * 512 + nsig * 128 + (int)(s & 127u)];
+                    const int used = (int)((e >> 4) & 15u);
                     x |= e & 15u;
                     s >>= used; bits -= used;
                     nsig += (int)(e >> 8);
-                } else {
-                    // the budget may end inside the code: bit by bit
-                    while (nsig < 4 && bits > 0) {
-                        --bits;
-                        const uint32_t any = s & 1u; s >>= 1;
-                        if (!any) break;
-                        while (nsig < 3 && bits > 0) {
-                            --bits;
-                            const uint32_t one = s & 1u; s >>= 1;
-                            if (one) break;
-                            ++nsig;
-                        }
-                        x |= 1u << nsig; ++nsig;
-                    }
+                    sigmask = (1u << nsig) - 1u;
                 }
-                sigmask = (1u << nsig) - 1u;
+                return x;
+            };
+            for (int kb = 28; kb >= 0 && bits > 0; kb -= 4) {
+                pl[3] |= plane() << kb;
+                if (bits > 0) pl[2] |= plane() << kb;
+                if (bits > 0) pl[1] |= plane() << kb;
+                if (bits > 0) pl[0] |= plane() << kb;
             }
-            return x;
-        };
-        for (int kb = 28; kb >= 0 && bits > 0; kb -= 4) {
-            pl[3] |= plane() << kb;
-            if (bits > 0) pl[2] |= plane() << kb;
-            if (bits > 0) pl[1] |= plane() << kb;
-            if (bits > 0) pl[0] |= plane() << kb;
+            uint32_t u[4];
+            values_of(pl, u);
+            int32_t q0 = from_negabinary(u[0]), q1 = from_negabinary(u[1]), q2 = from_negabinary(u[2]), q3 = from_negabinary(u[3]);
+            inv_lift(q0, q1, q2, q3);
+            // 2^(emax - 30): a normal number unless the block's values are next to the denormals
+            const int se = emax - 30 + 127;
+            const float sc = se >= 1 ? __uint_as_float((uint32_t)se << 23) : ldexpf(1.0f, emax - 30);
+            o = make_float4((float)q0 * sc, (float)q1 * sc, (float)q2 * sc, (float)q3 * sc);
         }
-        uint32_t u[4];
-        values_of(pl, u);
-        int32_t q0 = from_negabinary(u[0]), q1 = from_negabinary(u[1]), q2 = from_negabinary(u[2]), q3 = from_negabinary(u[3]);
-        inv_lift(q0, q1, q2, q3);
-        // 2^(emax - 30): a normal number unless the block's values are next to the denormals
-        const int se = emax - 30 + 127;
-        const float sc = se >= 1 ? __uint_as_float((uint32_t)se << 23) : ldexpf(1.0f, emax - 30);
-        o = make_float4((float)q0 * sc, (float)q1 * sc, (float)q2 * sc, (float)q3 * sc);
+        reinterpret_cast<float4 *>(field)[b] = o;
     }
-    reinterpret_cast<float4 *>(field)[b] = o;
 }
 
 template <int NW>
@@ -969,7 +973,8 @@ extern "C" int planmoe_zfp_decompress(const void *stream_in, int dims, int64_t n
     hipStream_t st = (hipStream_t)stream;
     const unsigned grid = (unsigned)((blocks + 255) / 256);
     if (dims == 1 && nw == 1) {
-        zfp_decode1_word_kernel<<<grid, 256, 0, st>>>((const uint32_t *)stream_in, blocks, field);
+        const unsigned grid1 = (unsigned)((blocks + 256 * ZD1_PER_THREAD - 1) / (256 * ZD1_PER_THREAD));
+        zfp_decode1_word_kernel<<<grid1, 256, 0, st>>>((const uint32_t *)stream_in, blocks, field);
         PM_LAUNCH_CHECK("planmoe_zfp_decompress");
         return 0;
     }
