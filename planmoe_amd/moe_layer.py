@@ -198,7 +198,8 @@ class MOELayer(torch.nn.Module):
                                                                    self.is_postscore):
                 # gate GEMM, routing, encode and compress as one call; decompress + decode in one pass
                 count_step()
-                y, l_aux = _overlap.fused_gate_forward(x, gate, kk, cap, self.normalize_gate, expert_fn, degree)
+                y, l_aux = _overlap.fused_gate_forward(x, gate, kk, cap, self.normalize_gate, expert_fn, degree,
+                                                       _overlap.ffn_from_codes_fn(self.experts, x, degree, reserve_dims))
                 return self._deliver(y, l_aux.to(loss_dtype), shape, dtype)
             if _overlap.gate_route_eligible(x, gate, E, self.is_postscore):
                 # gate GEMM + routing as one call and one node of the graph together with the encode
@@ -219,7 +220,8 @@ class MOELayer(torch.nn.Module):
         if _overlap.fused_int8_eligible(x, self.compress_name, degree, self.is_postscore):
             # encode + compress and decompress + decode in one pass each
             count_step()
-            return self._deliver(_overlap.fused_int8_forward(x, crit, expert_fn, degree), l_aux, shape, dtype)
+            codes_fn = _overlap.ffn_from_codes_fn(self.experts, x, degree, reserve_dims)
+            return self._deliver(_overlap.fused_int8_forward(x, crit, expert_fn, degree, codes_fn), l_aux, shape, dtype)
         if _overlap.fused_zfp_eligible(x, self.compress_name, degree, self.is_postscore, crit[0], crit[4]):
             count_step()
             return self._deliver(_overlap.fused_zfp_forward(x, crit, expert_fn, degree), l_aux, shape, dtype)

@@ -115,6 +115,22 @@ FUSE_GATE = True
 # work-groups from becoming resident until their bounded wait runs out; the backward pass of the
 # layer then raises.  Safe, and 5 us faster at 16384 x 4096, when one stream runs the layers.
 FORWARD_SINGLE_LAUNCH = False
+# inference (no autograd) with the built-in expert FFN in bf16: the receive side hands the int8
+# codes straight to the experts' first GEMM (planmoe_ffn_fc1_int8_affine) instead of decompressing
+# them into a tensor first
+FFN_FROM_CODES = True
+
+
+def ffn_from_codes_fn(module, x, degree, reserve_dims):
+    """The experts as a function of (codes, bias, scale) [E, C, ...] when the layer's receive side
+    may skip the decompress, else None."""
+    from .experts import FusedExpertsNetwork
+    if not (FFN_FROM_CODES and not torch.is_grad_enabled() and type(module) is FusedExpertsNetwork and degree == 1 and
+            reserve_dims == 1 and x.is_cuda and x.dtype == torch.bfloat16 and x.shape[-1] % 64 == 0 and
+            module.hidden_size_per_expert % 128 == 0 and module.batched_fc1_w.dtype == torch.bfloat16 and
+            module.output_dim in (None, x.shape[-1])):
+        return None
+    return module.forward_from_codes
 
 
 class _EncodeInt8(torch.autograd.Function):
@@ -290,14 +306,27 @@ def fused_gate_eligible(x, gate, experts, compress_name, degree, is_postscore):
             experts <= 64 and x.shape[0] >= 1 and gate_weight_fits(gate, x))
 
 
-def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn, degree=1):
+def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn, degree=1, codes_fn=None):
     """moe_layer's forward from the gate to the combine for the int8 compressor, the GShard loss
-    and plain routing.  Returns (output [T, M], l_aux)."""
+    and plain routing.  Returns (output [T, M], l_aux).  codes_fn (inference only): the experts as a
+    function of the codes, see ffn_from_codes_fn."""
     w = gate.wg.weight
     if w.dtype != x.dtype:
         w = w.to(x.dtype)
     experts = w.shape[0]
     x = x.contiguous()
+    if codes_fn is not None and not torch.is_grad_enabled():
+        single = FORWARD_SINGLE_LAUNCH and ops.forward_int8_single_serves(x, w, top_k)
+        out = (ops.forward_int8_single if single else ops.forward_int8)(
+            x, w.contiguous(), top_k, capacity, fp32_gate=bool(gate.fp32_gate), normalize_gate=bool(normalize_gate))
+        M = x.shape[-1]
+        y = codes_fn(out["codes"].view(experts, capacity, M), out["bias"].view(experts, capacity, 1),
+                     out["scale"].view(experts, capacity, 1))
+        codes, bias, scale = ops.int8_compress(y.reshape(experts * capacity, -1).to(x.dtype).contiguous())
+        k = out["indices"].shape[0]
+        res = ops.combine_int8(codes, bias, scale, list(out["indices"]), list(out["locations"]),
+                               [out["gates"][j].float() for j in range(k)], x.shape[0], capacity)
+        return res, out["l_aux"]
     y, gates, l_aux, indices, locations = _GateRouteEncodeInt8.apply(x, w.contiguous(), top_k, capacity,
                                                                      bool(gate.fp32_gate), bool(normalize_gate))
     y = _experts_in_chunks(expert_fn, y.view(experts, capacity, x.shape[-1]), degree)
@@ -398,12 +427,21 @@ def fused_int8_eligible(x, compress_name, degree, is_postscore):
             x.dtype in (torch.float32, torch.bfloat16, torch.float16) and x.shape[-1] % vec == 0)
 
 
-def fused_int8_forward(x, crit, expert_fn, degree=1):
+def fused_int8_forward(x, crit, expert_fn, degree=1, codes_fn=None):
     """encode -> [codec, comm, codec] -> experts -> [codec, comm, codec] -> decode for the
-    int8 compressor.  crit = (experts, indices_s, locations_s, gates_s, capacity)."""
+    int8 compressor.  crit = (experts, indices_s, locations_s, gates_s, capacity).  codes_fn
+    (inference only): the experts as a function of the codes, see ffn_from_codes_fn."""
     experts, indices_s, locations_s, gates_s, capacity = crit
     indices = torch.stack([t.reshape(-1) for t in indices_s]).to(torch.int32).contiguous()     # [k, T]
     locations = torch.stack([t.reshape(-1) for t in locations_s]).to(torch.int32).contiguous()
+    if codes_fn is not None and not torch.is_grad_enabled():
+        x = x.contiguous()
+        M = x.shape[-1]
+        codes, bias, scale = ops.dispatch_int8(x, list(indices), list(locations), None, experts, capacity)
+        y = codes_fn(codes.view(experts, capacity, M), bias.view(experts, capacity, 1), scale.view(experts, capacity, 1))
+        codes, bias, scale = ops.int8_compress(y.reshape(experts * capacity, -1).to(x.dtype).contiguous())
+        return ops.combine_int8(codes, bias, scale, list(indices), list(locations), [g.float() for g in gates_s],
+                                x.shape[0], capacity)
     y = _EncodeInt8.apply(x.contiguous(), indices, locations, experts, capacity)
     y = _experts_in_chunks(expert_fn, y.view(experts, capacity, x.shape[-1]), degree)
     y = y.reshape(experts * capacity, -1).to(x.dtype)

@@ -133,3 +133,39 @@ def test_fc1_affine_config2_shape():
     mag = torch.einsum("ecm,ehm->ech", dec.abs(), w.double().abs()) + fb.double().abs()[:, None, :]
     assert ((sample - ref).abs() <= 1e-2 * ref.abs() + 2.0 ** -7 * mag).all()
     assert bool(torch.isfinite(got.float()).all()) and float(got.float().abs().sum(dim=2).min()) > 0
+
+
+def test_layer_inference_feeds_the_codes_to_the_experts(monkeypatch):
+    """moe_layer under no_grad with the built-in FFN in bf16 and the int8 compressor: the receive
+    side skips the decompress (experts.forward_from_codes is called) and the output agrees with the
+    layer that decompresses first, to bf16 tolerance; with autograd on the usual path runs."""
+    import planmoe_amd
+    from planmoe_amd import overlap, experts
+    T, M, E, H = 1024, 256, 4, 384
+    layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'capacity_factor': 1.25}, M,
+                                  experts={'type': 'ffn', 'count_per_node': E, 'hidden_size_per_expert': H},
+                                  seeds=(1, 2, 3), compress_name='int8').to(DEV).to(torch.bfloat16)
+    x = torch.randn(T, M, generator=torch.Generator().manual_seed(5)).bfloat16().to(DEV)
+    calls = []
+    real = experts.FusedExpertsNetwork.forward_from_codes
+
+    def spy(self, *a, **kw):
+        calls.append(1)
+        return real(self, *a, **kw)
+    monkeypatch.setattr(experts.FusedExpertsNetwork, "forward_from_codes", spy)
+    with torch.no_grad():
+        got = layer(x)
+        assert len(calls) == 1
+        monkeypatch.setattr(overlap, "FFN_FROM_CODES", False)
+        want = layer(x)
+        assert len(calls) == 1
+    assert torch.allclose(got.float(), want.float(), rtol=3e-2, atol=3e-2 * float(want.float().abs().max()))
+    monkeypatch.setattr(overlap, "FFN_FROM_CODES", True)
+    y = layer(x.clone().requires_grad_(True))                     # autograd on: the training path
+    assert len(calls) == 1 and y.requires_grad
+    for fuse_gate in (False,):                                    # and the path with a separate gate + routing
+        monkeypatch.setattr(overlap, "FUSE_GATE", fuse_gate)
+        with torch.no_grad():
+            got2 = layer(x)
+        assert len(calls) == 2
+        assert torch.allclose(got2.float(), want.float(), rtol=3e-2, atol=3e-2 * float(want.float().abs().max()))
