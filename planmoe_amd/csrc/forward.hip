@@ -983,6 +983,7 @@ extern "C" int planmoe_forward_int8_single(const void *x, const void *wg, int dt
     PM_REQUIRE((codes && bias && scale) || capacity == 0, "planmoe_forward_int8_single: NULL codec output");
     PM_REQUIRE(workspace && workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
                "planmoe_forward_int8_single: workspace too small");
+    PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7u) == 0, "planmoe_forward_int8_single: workspace must be 8-byte aligned");
     PM_REQUIRE(spin_limit >= 0, "planmoe_forward_int8_single: spin_limit < 0");
     const int rc = run_forward_single(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
                                       normalize_gate, capacity, indices, locations, gates, plane_stride, logits_out,
