@@ -302,11 +302,95 @@ static torch::Tensor decompress_operation(const torch::Tensor &input)
     return output;
 }
 
-// the reference's CPU kernels are not part of this build: a CPU path would void the parity claim
-static void invoke_cpu_unavailable(const std::vector<torch::Tensor> &, const std::vector<int> &, int)
+// ---- invoke_cpu_fp32 / invoke_cpu_fp64 (custom_kernel.cpp:57-112, called from jit_compiler.py:41-45 for
+// tensors that live on the host).  These are the reference's own entry points for CPU tensors, kept as what
+// they are: a separate call for host tensors, single-threaded, in the tensors' dtype.  Nothing on
+// the GPU path reaches them (every GPU entry point refuses a CPU tensor and these refuse a GPU
+// tensor), and they share no code with the test oracle.
+//   inputs = {gates [T], indices int32 [T], locations int32 [T], rows [T, hidden], slots [E * capacity, hidden]},
+//   extra = {samples, hidden, capacity};  kernel_type 0: slots += gate * row (the caller zeroes slots),
+//   1: rows = gate * slot row, zero rows for pairs without a slot,  2: gates = <slot row, row> or 0.
+// A pair has a slot when index >= 0 and location < capacity (the reference's test, kept to the letter).
+namespace {
+
+template <typename T>
+struct HostPair {                       // one choice plane laid over host memory
+    T *gates; const int32_t *index; const int32_t *location; T *rows; T *slots;
+    int64_t hidden, capacity;
+    T *row(int64_t t) const { return rows + t * hidden; }
+    T *slot(int64_t t) const
+    {
+        if (index[t] < 0 || location[t] >= capacity) return nullptr;
+        return slots + ((int64_t)index[t] * capacity + location[t]) * hidden;
+    }
+};
+
+template <typename T>
+void host_scatter(const HostPair<T> &p, int64_t samples)
 {
-    AT_ASSERTM(false, "invoke_cpu_fp32/fp64: this build has no CPU kernels; pass GPU tensors");
+    for (int64_t t = 0; t < samples; ++t)
+        if (T *dst = p.slot(t)) {
+            const T g = p.gates[t], *src = p.row(t);
+            for (int64_t j = 0; j < p.hidden; ++j) dst[j] += g * src[j];
+        }
 }
+
+template <typename T>
+void host_gather(const HostPair<T> &p, int64_t samples)
+{
+    for (int64_t t = 0; t < samples; ++t) {
+        T *dst = p.row(t);
+        if (const T *src = p.slot(t)) {
+            const T g = p.gates[t];
+            for (int64_t j = 0; j < p.hidden; ++j) dst[j] = g * src[j];
+        } else {
+            std::fill(dst, dst + p.hidden, T(0));
+        }
+    }
+}
+
+template <typename T>
+void host_gate_gradient(const HostPair<T> &p, int64_t samples)
+{
+    for (int64_t t = 0; t < samples; ++t) {
+        T sum = 0;                                              // summed in the tensors' dtype, left to right
+        if (const T *a = p.slot(t)) {
+            const T *b = p.row(t);
+            for (int64_t j = 0; j < p.hidden; ++j) sum += a[j] * b[j];
+        }
+        p.gates[t] = sum;
+    }
+}
+
+template <typename T>
+void invoke_cpu(const std::vector<torch::Tensor> &ts, const std::vector<int> &extra, int kernel_type)
+{
+    const auto want = c10::CppTypeToScalarType<T>::value;
+    AT_ASSERTM(ts.size() >= 5 && extra.size() >= 3, "invoke_cpu: expects 5 tensors and {samples, hidden, capacity}");
+    for (size_t i = 0; i < ts.size(); ++i) {
+        AT_ASSERTM(!ts[i].is_cuda(), "invoke_cpu: tensor must be a CPU tensor (GPU tensors take the GPU entry points)");
+        AT_ASSERTM(ts[i].is_contiguous(), "invoke_cpu: tensor must be contiguous");
+    }
+    AT_ASSERTM(ts[0].scalar_type() == want && ts[3].scalar_type() == want && ts[4].scalar_type() == want,
+               "invoke_cpu: gates, rows and slots must have the dtype of the entry point");
+    AT_ASSERTM(ts[1].scalar_type() == at::kInt && ts[2].scalar_type() == at::kInt, "invoke_cpu: indices and locations must be int32");
+    const int64_t samples = extra[0], hidden = extra[1], capacity = extra[2];
+    AT_ASSERTM(samples >= 0 && hidden >= 0 && capacity >= 0, "invoke_cpu: negative size");
+    AT_ASSERTM(ts[0].numel() >= samples && ts[1].numel() >= samples && ts[2].numel() >= samples &&
+                   ts[3].numel() >= samples * hidden, "invoke_cpu: tensors smaller than {samples, hidden} say");
+    const HostPair<T> p{ts[0].data_ptr<T>(), ts[1].data_ptr<int32_t>(), ts[2].data_ptr<int32_t>(), ts[3].data_ptr<T>(),
+                        ts[4].data_ptr<T>(), hidden, capacity};
+    // every slot a live pair names must lie inside the slots tensor
+    for (int64_t t = 0; t < samples; ++t)
+        if (p.index[t] >= 0 && p.location[t] < capacity)
+            AT_ASSERTM(p.location[t] >= 0 && ((int64_t)p.index[t] * capacity + p.location[t] + 1) * hidden <= ts[4].numel(),
+                       "invoke_cpu: a pair addresses a slot outside the slots tensor");
+    if (kernel_type == 0) host_scatter(p, samples);
+    else if (kernel_type == 1) host_gather(p, samples);
+    else host_gate_gradient(p, samples);
+}
+
+} // namespace
 
 torch::Tensor warp_cumsum(torch::Tensor x)
 {
@@ -338,8 +422,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("invoke", &invoke, "not available in this build");
     m.def("inject_source", &inject_source, "not available in this build");
     m.def("registered_compressors", &planmoe::registered_compressors, "names of the compressor plug-ins registered from C++");
-    m.def("invoke_cpu_fp32", &invoke_cpu_unavailable, "not available in this build");
-    m.def("invoke_cpu_fp64", &invoke_cpu_unavailable, "not available in this build");
+    m.def("invoke_cpu_fp32", &invoke_cpu<float>, "Invoke for Sparse Ops (CPU)");
+    m.def("invoke_cpu_fp64", &invoke_cpu<double>, "Invoke for Sparse Ops (CPU)");
     m.def("compress_operation", &compress_operation, "Compress Operation");
     m.def("comm_operation", &comm_operation, "Comm Operation");
     m.def("decompress_operation", &decompress_operation, "Decompress Operation");

@@ -27,7 +27,7 @@ def test_module_surface_and_host_side_errors():
     with pytest.raises(RuntimeError, match="GPU tensor"):
         ck.compress_operation(torch.zeros(4, 4, 8), "int8", "naive")
     ck.clear_ptr_lst()
-    with pytest.raises(RuntimeError, match="no CPU kernels"):
+    with pytest.raises(RuntimeError, match="expects 5 tensors"):
         ck.invoke_cpu_fp32([torch.zeros(1)], [1, 1, 1], 0)
     with pytest.raises(RuntimeError, match="GPU tensor"):
         ck.compress_operation(torch.zeros(4, 4, 8), "lz", "naive")
@@ -171,3 +171,58 @@ def test_tutel_ops_cumsum():
     m = (torch.rand(3000, 8, generator=torch.Generator().manual_seed(0)) < 0.3).to(torch.int64)
     out = torch.ops.tutel_ops.cumsum(m.to(DEV))
     assert out.dtype == torch.int32 and np.array_equal(out.cpu().numpy(), oracle.cumsum_sub_one(m.numpy()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_invoke_cpu_against_the_oracle_and_closed_forms(dtype):
+    """invoke_cpu_fp32 / fp64 (custom_kernel.cpp:57-112): the reference's calls for host tensors.  The three
+    kernel types against the oracle's restatement (bit for bit: same products, same order of sums)
+    and against what torch computes for the same thing; dropped pairs (index < 0, location >=
+    capacity), errors for GPU-side misuse."""
+    from planmoe_amd import ext
+    ck = ext.load()
+    fn = ck.invoke_cpu_fp32 if dtype == torch.float32 else ck.invoke_cpu_fp64
+    T, H, E, C = 37, 24, 5, 8
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(T, H, generator=g, dtype=dtype)
+    gate = torch.rand(T, generator=g, dtype=dtype)
+    idx = torch.randint(0, E, (T,), generator=g, dtype=torch.int32)
+    # distinct slots for the live pairs, some pairs dropped either way
+    perm = torch.randperm(E * C, generator=g)[:T]
+    idx, loc = (perm // C).to(torch.int32), (perm % C).to(torch.int32)
+    loc[3] = C + 2
+    idx[5] = -1
+    loc[8] = C
+    live = (idx >= 0) & (loc < C)
+    # 0: scatter into zeroed slots
+    slots = torch.zeros(E * C, H, dtype=dtype)
+    fn([gate, idx, loc, x, slots], [T, H, C], 0)
+    want = oracle.dispatch(gate.numpy(), idx.numpy(), loc.numpy(), x.numpy(), np.zeros((E * C, H), dtype=x.numpy().dtype), C)
+    assert np.array_equal(slots.numpy(), want)
+    ref = torch.zeros(E * C, H, dtype=dtype)
+    ref[(idx[live].long() * C + loc[live].long())] = gate[live, None] * x[live]
+    assert torch.equal(slots, ref)
+    fn([gate, idx, loc, x, slots], [T, H, C], 0)                  # it accumulates, as the reference does
+    assert torch.equal(slots, ref + ref)
+    # 1: gather back
+    slots = torch.randn(E * C, H, generator=g, dtype=dtype)
+    rows = torch.full((T, H), 7.0, dtype=dtype)
+    fn([gate, idx, loc, rows, slots], [T, H, C], 1)
+    assert np.array_equal(rows.numpy(), oracle.gather(gate.numpy(), idx.numpy(), loc.numpy(), slots.numpy(), T, C))
+    assert bool((rows[~live] == 0).all()) and torch.equal(rows[live], gate[live, None] * slots[idx[live].long() * C + loc[live].long()])
+    # 2: gate gradients
+    gg = torch.full((T,), 9.0, dtype=dtype)
+    fn([gg, idx, loc, x, slots], [T, H, C], 2)
+    assert np.array_equal(gg.numpy(), oracle.bwd_gate(idx.numpy(), loc.numpy(), x.numpy(), slots.numpy(), C))
+    assert bool((gg[~live] == 0).all())
+    full = (slots[idx[live].long() * C + loc[live].long()].double() * x[live].double()).sum(1)
+    assert torch.allclose(gg[live].double(), full, rtol=1e-5 if dtype == torch.float32 else 1e-12)
+    # misuse
+    with pytest.raises(RuntimeError, match="dtype of the entry point"):
+        fn([gate.to(torch.float16), idx, loc, x, slots], [T, H, C], 0)
+    with pytest.raises(RuntimeError, match="int32"):
+        fn([gate, idx.long(), loc, x, slots], [T, H, C], 0)
+    with pytest.raises(RuntimeError, match="outside the slots tensor"):
+        fn([gate, idx + E, loc, x, slots], [T, H, C], 0)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        fn([gate, idx, loc, x.t().contiguous().t(), slots], [T, H, C], 0)
