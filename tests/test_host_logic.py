@@ -131,3 +131,15 @@ def test_overlap_degree_checks():
         a2a_ffn_overlap_forward(torch.zeros(2, 8, 4), lambda t: t, 3, False, None, "no", "naive")
     y = a2a_ffn_overlap_forward(torch.arange(64.0).view(2, 8, 4), lambda t: t * 2, 2, False, None, "no", "naive")
     assert torch.equal(y, torch.arange(64.0).view(2, 8, 4) * 2)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU's share of the path: --gpus N with N > 1 exits with a message that says
+    so (before anything touches a device)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "--gpus 2 is not supported" in (r.stderr + r.stdout)
