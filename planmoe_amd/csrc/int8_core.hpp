@@ -249,8 +249,13 @@ struct RowEncoder<PLANMOE_BF16> {
         uint32_t pk = f32x2_to_bf16x2(f0 - rq.bias, f1 - rq.bias);
         const float d0 = __uint_as_float(pk << 16), d1 = __uint_as_float(pk & 0xffff0000u);
         pk = f32x2_to_bf16x2(d0 * rq.inv, d1 * rq.inv);
-        const float q0 = __uint_as_float(pk << 16), q1 = __uint_as_float(pk & 0xffff0000u);
-        pk = f32x2_to_bf16x2(q0 * 255.0f, q1 * 255.0f);
+        // bf16(255 q) without multiplying: for q = a 2^e with an 8-bit a in [128, 255] the product
+        // 255 a = 256 a - a has 16 bits and rounds to a - 1 (its fraction a / 256 lies strictly between
+        // 1/2 and 1) for a >= 129, and is 255 2^7 for a = 128: in both cases the bit pattern of
+        // q plus 8 exponent steps minus one, i.e. 256 times the bf16 value just below q.  A zero
+        // or denormal q lands on a value below 2^-100 and a NaN q (0 / 0 rows) on a negative one:
+        // the truncation below makes 0 of both, as it does of their true products.
+        pk += 0x03ff03ffu;
         const float m0 = __uint_as_float(pk << 16), m1 = __uint_as_float(pk & 0xffff0000u);
         // truncation; the conversion saturates NaN (0/0 rows) and negatives to 0, m <= 255
         return __float2uint_rz(m0) | (__float2uint_rz(m1) << 8);
