@@ -246,9 +246,11 @@ struct RowEncoder<PLANMOE_BF16> {
     __device__ __forceinline__ uint32_t pair_values(float f0, float f1) const
     {
         if constexpr (!FAST) return quantise<PLANMOE_BF16>(0.f + f0, rq.bias, rq.scale) | (quantise<PLANMOE_BF16>(0.f + f1, rq.bias, rq.scale) << 8);
-        uint32_t pk = f32x2_to_bf16x2(f0 - rq.bias, f1 - rq.bias);
-        const float d0 = __uint_as_float(pk << 16), d1 = __uint_as_float(pk & 0xffff0000u);
-        pk = f32x2_to_bf16x2(d0 * rq.inv, d1 * rq.inv);
+        // (each difference rounded on its own, into the upper half of a word with zeros below: the
+        // rounded value is a float right away, one conversion per value instead of one per pair
+        // and an unpacking of both)
+        const float d0 = __uint_as_float(f32x2_to_bf16x2(0.f, f0 - rq.bias)), d1 = __uint_as_float(f32x2_to_bf16x2(0.f, f1 - rq.bias));
+        uint32_t pk = f32x2_to_bf16x2(d0 * rq.inv, d1 * rq.inv);
         // bf16(255 q) without multiplying: for q = a 2^e with an 8-bit a in [128, 255] the product
         // 255 a = 256 a - a has 16 bits and rounds to a - 1 (its fraction a / 256 lies strictly between
         // 1/2 and 1) for a >= 129, and is 255 2^7 for a = 128: in both cases the bit pattern of
@@ -256,7 +258,10 @@ struct RowEncoder<PLANMOE_BF16> {
         // or denormal q lands on a value below 2^-100 and a NaN q (0 / 0 rows) on a negative one:
         // the truncation below makes 0 of both, as it does of their true products.
         pk += 0x03ff03ffu;
-        const float m0 = __uint_as_float(pk << 16), m1 = __uint_as_float(pk & 0xffff0000u);
+        // (the upper value keeps the lower one's bits below its own: less than one bf16 step on top
+        // of a value below 256, whose steps are 1 / 2^k, so no integer lies in between and the
+        // truncation does not see them)
+        const float m0 = __uint_as_float(pk << 16), m1 = __uint_as_float(pk);
         // truncation; the conversion saturates NaN (0/0 rows) and negatives to 0, m <= 255
         return __float2uint_rz(m0) | (__float2uint_rz(m1) << 8);
     }
