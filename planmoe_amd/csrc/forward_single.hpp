@@ -108,7 +108,6 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
     __shared__ int32_t s_full[4][CAP], s_base[4][CAP], s_tot[CAP];
     __shared__ float s_mepart[FS_THREADS / CAP][CAP];
     __shared__ int s_vote[2][FS_WAVES];
-    __shared__ int32_t s_zbeg[CAP + 1], s_used[CAP];       // empty slots: first list index and first slot per expert
     __shared__ int s_zdone;
 
     const int tid = threadIdx.x, w = tid >> 6, lane = lane_id(), m = lane & 15, g = lane >> 4;
@@ -406,21 +405,6 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
             taken += ful;
         }
         s_tot[tid] = taken;
-        // the empty slots of all experts as one list, expert after expert
-        int zbefore = 0, zown = 0;
-        for (int ee = 0; ee < CAP; ++ee) {
-            int tt = 0;
-            for (int j = 0; j < 4; ++j) {
-                const int idx = j * CAP + ee;
-                tt += (int)((s_full64[idx / 4] >> (16 * (idx % 4))) & 0xffffu);
-            }
-            const int z = ee < experts ? capacity - min(tt, capacity) : 0;
-            if (ee < tid) zbefore += z;
-            if (ee == tid) zown = z;
-        }
-        s_zbeg[tid] = zbefore;
-        s_used[tid] = capacity - zown;
-        if (tid == CAP - 1) s_zbeg[CAP] = zbefore + zown;
     }
     lds_barrier();
     FS_STAMP(8);
@@ -490,16 +474,27 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
         asm volatile("" : "+v"(got) : : "memory");
         return (uint32_t)__builtin_amdgcn_readfirstlane((int)got) - zero_base;
     };
-    auto zero_row = [&](uint32_t idx) {
-        const int e = __popcll(__ballot(lane >= 1 && lane < CAP && (uint32_t)s_zbeg[min(lane, CAP)] <= idx));
-        const int slot = e * capacity + s_used[e] + (int)(idx - (uint32_t)s_zbeg[e]);
-        uint4 *dst = reinterpret_cast<uint4 *>(codes + (int64_t)slot * G::M) + lane;
-#pragma unroll
-        for (int i = 0; i < G::RV; ++i) stream_store(dst + i * WAVE, make_uint4(0u, 0u, 0u, 0u));
-        if (lane == 0) { B16::store(bias_out, slot, 0.f); B16::store(scale_out, slot, 0.f); }
-    };
     auto zero_fill = [&]() {
-        const uint32_t total = (uint32_t)s_zbeg[CAP];
+        // the empty slots of all experts as one list, expert after expert: lane e < CAP of every wave holds
+        // where expert e's stretch of the list begins and the first empty slot of e (a prefix over the
+        // lanes; worked out here, off the path from the slot bases to the first stores)
+        const int z_used = lane < experts && lane < CAP ? min(s_tot[min(lane, CAP - 1)], capacity) : capacity;
+        int z_upto = capacity - z_used;                          // empty slots of the experts up to this lane's
+#pragma unroll
+        for (int off = 1; off < CAP; off <<= 1) {
+            const int below = __shfl_up(z_upto, off, WAVE);
+            if (lane >= off) z_upto += below;
+        }
+        const int z_beg = z_upto - (capacity - z_used);
+        auto zero_row = [&](uint32_t idx) {
+            const int e = __popcll(__ballot(lane >= 1 && lane < CAP && (uint32_t)z_beg <= idx));
+            const int slot = e * capacity + __builtin_amdgcn_readlane(z_used, e) + (int)(idx - (uint32_t)__builtin_amdgcn_readlane(z_beg, e));
+            uint4 *dst = reinterpret_cast<uint4 *>(codes + (int64_t)slot * G::M) + lane;
+#pragma unroll
+            for (int i = 0; i < G::RV; ++i) stream_store(dst + i * WAVE, make_uint4(0u, 0u, 0u, 0u));
+            if (lane == 0) { B16::store(bias_out, slot, 0.f); B16::store(scale_out, slot, 0.f); }
+        };
+        const uint32_t total = (uint32_t)__builtin_amdgcn_readlane(z_upto, CAP - 1);
         const uint32_t shares = (uint32_t)(groups + FS_SHARE - 1) / FS_SHARE, per = (total + shares - 1) / shares;
         const uint32_t lo = (uint32_t)(grp / FS_SHARE) * per, hi = min(lo + per, total);
         if (lo >= hi) return;
