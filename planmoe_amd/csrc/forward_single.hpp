@@ -297,37 +297,36 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
     lds_barrier();
     FS_STAMP(4);
 
-    // ---- the group's ranks and histogram (wave 0, one lane per token), published at once
-    if (w == 0) {
+    // ---- the group's ranks and histogram, one lane per token: wave j takes choice plane j and
+    // publishes that plane's words itself, wave 4 the score sums
+    if (w < 4) {
+        const int j = w;
         const bool valid = lane < TOK && t0 + lane < samples;
-        for (int j = 0; j < 4; ++j) {
-            const int best = (valid && j < k) ? (int)s_best[j][lane % TOK] : -1;
-            int rank = 0;
+        const int best = (valid && j < k) ? (int)s_best[j][lane % TOK] : -1;
+        int rank = 0;
 #pragma unroll
-            for (int e = 0; e < CAP; ++e) {
-                const uint64_t mk = __ballot(best == e);
-                if (best == e) rank = __popcll(mk & lanes_below());
-                if (lane == e) s_hist[j][e] = __popcll(mk);
-            }
-            if (lane < TOK) s_rank[j][lane] = rank;
+        for (int e = 0; e < CAP; ++e) {
+            const uint64_t mk = __ballot(best == e);
+            if (best == e) rank = __popcll(mk & lanes_below());
+            if (lane == e) s_hist[j][e] = __popcll(mk);
         }
+        if (lane < TOK) s_rank[j][lane] = rank;
         __builtin_amdgcn_wave_barrier();
-        if (lane < HW) {
-            const int32_t *h = &s_hist[0][0] + 4 * lane;
+        if (lane < CAP / 4) {
+            const int32_t *h = &s_hist[j][4 * lane];
             const uint32_t payload = (uint32_t)h[0] | ((uint32_t)h[1] << 8) | ((uint32_t)h[2] << 16) | ((uint32_t)h[3] << 24);
-            __hip_atomic_store(pub_hist + (size_t)grp * HW + lane, ((unsigned long long)tag << 32) | payload,
+            __hip_atomic_store(pub_hist + (size_t)grp * HW + j * (CAP / 4) + lane, ((unsigned long long)tag << 32) | payload,
                                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        if (l_aux && lane < CAP) {
-            float v = 0.f;
-            if (lane < experts) {
-                v = s_me[0][lane];
+    } else if (w == 4 && l_aux && lane < CAP) {
+        float v = 0.f;
+        if (lane < experts) {
+            v = s_me[0][lane];
 #pragma unroll
-                for (int i = 1; i < RPASSES * FS_WAVES; ++i) v += s_me[i][lane];
-            }
-            __hip_atomic_store(pub_me + (size_t)grp * CAP + lane, ((unsigned long long)tag << 32) | __float_as_uint(v),
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int i = 1; i < RPASSES * FS_WAVES; ++i) v += s_me[i][lane];
         }
+        __hip_atomic_store(pub_me + (size_t)grp * CAP + lane, ((unsigned long long)tag << 32) | __float_as_uint(v),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     FS_STAMP(5);
 
