@@ -560,6 +560,14 @@ def main():
     plan2.run()
     stages["dispatch_int8_routed (second launch of the two-launch chain, alone)"] = event_time_us(plan2.redispatch, 30, 5)
     chain2_ev = event_time_us(plan2.run, 30, 5)
+    # the measuring stick: the chain's grid, loads, exchange and stores without its arithmetic (the
+    # floor under this kernel's structure), and the same with nobody waiting at the exchange (the
+    # floor under any arrangement of these loads and stores: what the dependency costs is the difference)
+    ceiling = ops.ForwardCeiling(xd, E, k, C)
+    ceil_ev = {mode: event_time_us(lambda mode=mode: ceiling.run(mode), 30, 5) for mode in (0, 1, 2)}
+    chain_ev_again = event_time_us(chain, 30, 5)
+    if int(ceiling.gave_up) != 0:
+        sys.exit("bench.py: a work-group of the ceiling kernel gave up waiting for the others")
 
     # the chains with none of their operands in the L2s or the 256 MB memory-side cache: a reduction
     # over 1 GiB of other data before every call, one event pair per call, median of 9
@@ -600,7 +608,14 @@ def main():
                      "algorithmic_bytes": chain_bytes, "avg_us": chain_ev[0], "min_us": chain_ev[2],
                      "cold_us": cold_us, "cold_achieved": chain_bytes / cold_us / 1e3,
                      "cold_frac": chain_bytes / cold_us / 1e3 / HBM_PEAK_GBS,
-                     "target_frac": 0.70, "target_met": achieved / HBM_PEAK_GBS >= 0.70},
+                     "target_frac": 0.70, "target_met": achieved / HBM_PEAK_GBS >= 0.70,
+                     # planmoe_forward_int8_single_ceiling in the same run: same grid, loads, exchange and
+                     # stores, no arithmetic
+                     "ceiling_us": ceil_ev[0][0], "ceiling_frac": chain_bytes / ceil_ev[0][0] / 1e3 / HBM_PEAK_GBS,
+                     "ceiling_no_exchange_us": ceil_ev[1][0],
+                     "ceiling_no_exchange_frac": chain_bytes / ceil_ev[1][0] / 1e3 / HBM_PEAK_GBS,
+                     "ceiling_two_halves_us": ceil_ev[2][0],
+                     "avg_us_after_ceilings": chain_ev_again[0]},
         "two_launch_chain": {"entry_point": "planmoe_forward_int8 (x read by both launches)",
                              "algorithmic_bytes": chain_bytes, "device_us_avg": chain2_ev[0],
                              "device_us_min": chain2_ev[2], "GBps": chain_bytes / chain2_ev[0] / 1e3,

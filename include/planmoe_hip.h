@@ -269,9 +269,16 @@ int planmoe_forward_int8(const void *x, const void *wg, int dtype, int fp32_gate
  * an error here (planmoe_forward_int8 picks between the two on its own).  Outputs as
  * planmoe_forward_int8 (logits may differ from it in the last bit: another summation order).
  * The wait between the work-groups is bounded: spin_limit polls (0 = the default, about a second);
- * a work-group that gives up writes none of its rows and sets *gave_up to 1 (optional device
- * word, cleared by the caller).  Two such launches that run at the same time on one GPU can keep
- * each other's work-groups from becoming resident: run them one after the other.
+ * a work-group that gives up writes none of its rows, marks its tokens dropped (locations =
+ * capacity), makes *l_aux NaN and sets *gave_up to 1 (device word, cleared by the caller): the
+ * caller reads that word before it uses any output and, if it is set, runs planmoe_forward_int8.
+ * Two such launches that run at the same time on one GPU could keep each other's work-groups from
+ * becoming resident, so the library puts them in a row: a launch on another stream than the one
+ * before it on the same device first waits (on the device) for that launch's event.  Launches
+ * recorded into a HIP graph are outside that order: keep replays of such graphs apart.
+ * The first FWD region of the workspace (its launch counter and published words) is written by
+ * this entry point alone; the other entry points that take a forward workspace keep their tables
+ * behind it, so one workspace may serve all of them in turn, whatever the shapes.
  * It has no counterpart in the reference. */
 int planmoe_forward_int8_single(const void *x, const void *wg, int dtype, int fp32_gate,
                                 const float *logit_bias, int samples, int model_dim, int experts,
@@ -281,6 +288,24 @@ int planmoe_forward_int8_single(const void *x, const void *wg, int dtype, int fp
                                 int32_t *expert_counts, uint8_t *codes, void *bias, void *scale,
                                 void *workspace, size_t workspace_bytes, int spin_limit,
                                 int32_t *gave_up, void *stream);
+
+/* A measuring stick for planmoe_forward_int8_single, not a product path: one launch with that
+ * kernel's grid, its loads of x, one exchange of tagged words between all work-groups and its
+ * streaming stores (every row of codes [experts*capacity, 4096], bias, scale, and planes =
+ * 3 x [2][samples] int32 standing for indices / locations / gates), and none of its arithmetic.
+ * What it writes means nothing; what it takes is the floor under that way of moving the bytes on
+ * the GPU at hand.  mode 0: read everything, exchange, store everything (the structure of
+ * planmoe_forward_int8_single); mode 1: the same with nobody waiting at the exchange, i.e. what the
+ * loads and stores alone cost when no slot depends on another work-group (the floor under any
+ * arrangement of them); mode 2: tokens dealt in two halves, the first-choice rows of the first
+ * half stored while the second half is read, one more exchange.  Serves model_dim 4096 bf16,
+ * 8 experts, top-2, samples a multiple of 128, capacity >= samples / 4.  Workspace, spin_limit,
+ * gave_up and the ordering of launches as for planmoe_forward_int8_single (it uses the same
+ * region of the workspace).  It has no counterpart in the reference. */
+int planmoe_forward_int8_single_ceiling(const void *x, int samples, int model_dim, int experts, int top_k,
+                                        int capacity, uint8_t *codes, void *bias, void *scale,
+                                        int32_t *planes, void *workspace, size_t workspace_bytes,
+                                        int mode, int spin_limit, int32_t *gave_up, void *stream);
 
 /* planmoe_forward_int8 for callers that cannot allocate device memory or carry a workspace
  * around (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):

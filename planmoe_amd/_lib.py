@@ -67,6 +67,8 @@ SIGNATURES = {
                                             c_int, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
+    "planmoe_forward_int8_single_ceiling": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                                    c_void_p, c_void_p, c_size_t, c_int, c_int, c_void_p, c_void_p]),
     "planmoe_forward_int8_static": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
                                             c_int, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,
                                             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,

@@ -42,6 +42,12 @@ inline int fwd_group_tokens(int experts, int samples)
     return (experts <= 16 && samples < 64 * 256) ? 32 : 64;
 }
 constexpr int FWD_LOSS_PARTS = 64;
+// The first bytes of a forward workspace belong to the one-launch kernel alone (its launch counter,
+// ticket counters and published words, forward_single.hpp): its tags are unique only while that
+// counter grows by one per launch, so no other entry point may write there.  The tables of the
+// two-launch chain and of the stand-alone routing start behind it, whatever the shape.
+constexpr size_t FWD_TABLES_OFFSET = 139520;
+inline void *fwd_tables(void *workspace) { return (char *)workspace + FWD_TABLES_OFFSET; }
 
 // hist_t / me_t are the transposes of hist / me with the group index running fastest (rows of
 // gstride = groups rounded up to 4 entries, the padding zero): a column of the histogram, which
@@ -744,6 +750,7 @@ int route_groups(const void *input, int dtype, int is_logits, const float *logit
     plan.experts_per_block = go_experts_per_block(experts, plan.k);
     plan.blocks = (experts + plan.experts_per_block - 1) / plan.experts_per_block;
     plan.merged = false;
+    workspace = fwd_tables(workspace);
     plan.ws = fwd_ws(workspace, plan.groups, plan.k, experts, samples);
     const int mode = is_logits ? 1 : 2;
     PM_DTYPE_SWITCH(dtype, SDT, (launch_route_groups<SDT>(experts, plan.groups, mode, st, input, is_logits ? logit_bias : nullptr,
@@ -815,6 +822,7 @@ static int run_dispatch_routed(const void *x, int dtype, int samples, int model_
 } // namespace pm
 
 #include "forward_single.hpp"
+#include "forward_ceiling.hpp"
 
 namespace pm {
 
@@ -830,7 +838,27 @@ static unsigned long long process_salt()
     return salt;
 }
 
-struct SingleShape { int nmma, rounds, groups; };
+// Two one-launch kernels that run at the same time on one GPU can keep each other's work-groups
+// from becoming resident, and then both wait until their bound.  So launches of the kernel on one
+// device are put in a row on the host: behind every launch an event is recorded, and a launch on
+// another stream first makes its stream wait for the event of the launch before it.  (Launches on
+// one stream follow each other anyway.  A stream that is being captured into a graph is left
+// alone: neither the wait nor the record belongs into the caller's graph; replays of such graphs
+// are the caller's to keep apart.)
+struct SingleOrder {
+    std::mutex lock;
+    hipEvent_t done = nullptr;
+    hipStream_t last = nullptr;
+    bool recorded = false;
+};
+static SingleOrder g_single_order[STATIC_SCRATCH_DEVICES_MAX];
+
+static bool stream_is_capturing(hipStream_t st)
+{
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &status) != hipSuccess) { (void)hipGetLastError(); return false; }
+    return status != hipStreamCaptureStatusNone;
+}
 
 // Whether the one-launch kernel serves the shape, and with how many rounds: model_dim 4096 bf16, up to
 // 16 experts, top_k <= 4, and so few tokens that every work-group is resident at once.
@@ -909,14 +937,13 @@ using namespace pm;
 
 extern "C" size_t planmoe_forward_workspace_bytes(int samples, int experts, int top_k)
 {
-    if (samples <= 0 || experts <= 0 || top_k <= 0) return 256;
+    if (samples <= 0 || experts <= 0 || top_k <= 0) return FWD_TABLES_OFFSET + 256;
     const size_t k = (size_t)(top_k < experts ? top_k : experts);
     const size_t groups = ((size_t)samples + 15) / 16;      // upper bound over the group sizes
     const size_t tables = ((size_t)experts + FWD_LOSS_PARTS + 2 * groups * k * experts + groups * experts +
                            (k + 2) * (size_t)samples + (k + 1) * experts * fwd_pad4(groups)) * 4;
-    // the one-launch kernel keeps the words its work-groups publish in the same space
-    const size_t published = fs_pub_bytes((int)(groups < (size_t)FS_MAX_GROUPS ? groups : (size_t)FS_MAX_GROUPS));
-    return round_up(tables > published ? tables : published, 256);
+    // in front of the tables: the one-launch kernel's own region
+    return FWD_TABLES_OFFSET + round_up(tables, 256);
 }
 
 extern "C" int planmoe_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
@@ -931,6 +958,7 @@ extern "C" int planmoe_gate_route(const void *x, const void *wg, int dtype, int 
     PM_REQUIRE(indices && locations && gates, "planmoe_gate_route: NULL output");
     PM_REQUIRE(workspace && workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
                "planmoe_gate_route: workspace too small");
+    workspace = fwd_tables(workspace);
     hipStream_t st = (hipStream_t)stream;
     FwdPlan plan;
     if (run_gate_route(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
@@ -956,6 +984,7 @@ extern "C" int planmoe_forward_int8(const void *x, const void *wg, int dtype, in
     PM_REQUIRE((uintptr_t)codes % 8 == 0, "planmoe_forward_int8: codes must be 8-byte aligned");
     PM_REQUIRE(workspace && workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
                "planmoe_forward_int8: workspace too small");
+    workspace = fwd_tables(workspace);
     hipStream_t st = (hipStream_t)stream;
     FwdPlan plan;
     fwd_plan(plan, workspace, samples, experts, top_k);
@@ -985,14 +1014,88 @@ extern "C" int planmoe_forward_int8_single(const void *x, const void *wg, int dt
                "planmoe_forward_int8_single: workspace too small");
     PM_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 7u) == 0, "planmoe_forward_int8_single: workspace must be 8-byte aligned");
     PM_REQUIRE(spin_limit >= 0, "planmoe_forward_int8_single: spin_limit < 0");
+    hipStream_t st = (hipStream_t)stream;
+    int dev = 0;
+    PM_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < STATIC_SCRATCH_DEVICES_MAX,
+               "planmoe_forward_int8_single: no current device");
+    SingleOrder &order = g_single_order[dev];
+    const bool ordered = !stream_is_capturing(st);
+    std::unique_lock<std::mutex> hold(order.lock);
+    if (ordered) {
+        if (!order.done)
+            PM_REQUIRE(hipEventCreateWithFlags(&order.done, hipEventDisableTiming) == hipSuccess,
+                       "planmoe_forward_int8_single: cannot create an event");
+        if (order.recorded && order.last != st)
+            PM_REQUIRE(hipStreamWaitEvent(st, order.done, 0) == hipSuccess,
+                       "planmoe_forward_int8_single: cannot wait for the launch before this one");
+    }
     const int rc = run_forward_single(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
                                       normalize_gate, capacity, indices, locations, gates, plane_stride, logits_out,
                                       scores_out, l_aux, expert_counts, codes, bias, scale, workspace,
-                                      spin_limit > 0 ? spin_limit : (1 << 20), gave_up, (hipStream_t)stream);
+                                      spin_limit > 0 ? spin_limit : (1 << 20), gave_up, st);
+    if (ordered && rc == 0) {
+        PM_REQUIRE(hipEventRecord(order.done, st) == hipSuccess, "planmoe_forward_int8_single: cannot record an event");
+        order.last = st;
+        order.recorded = true;
+    }
+    hold.unlock();
     PM_REQUIRE(rc != 2, "planmoe_forward_int8_single: the one-launch kernel serves bf16 rows of 4096 values, up to 16 "
                "experts, top_k <= 4 and at most 64 tokens per compute unit; use planmoe_forward_int8");
     PM_LAUNCH_CHECK("planmoe_forward_int8_single");
     return rc;
+}
+
+extern "C" int planmoe_forward_int8_single_ceiling(const void *x, int samples, int model_dim, int experts, int top_k,
+                                                   int capacity, uint8_t *codes, void *bias, void *scale,
+                                                   int32_t *planes, void *workspace, size_t workspace_bytes,
+                                                   int mode, int spin_limit, int32_t *gave_up, void *stream)
+{
+    PM_REQUIRE(x && codes && bias && scale && planes && workspace, "planmoe_forward_int8_single_ceiling: NULL argument");
+    PM_REQUIRE(model_dim == 4096 && experts == 8 && top_k == 2 && samples >= 64 && samples % 128 == 0,
+               "planmoe_forward_int8_single_ceiling: serves rows of 4096 bf16 values, 8 experts, top-2 and a multiple of "
+               "128 tokens");
+    const int groups = samples / 64;
+    PM_REQUIRE(groups <= FS_MAX_GROUPS && capacity >= groups * 16 && (int64_t)experts * capacity < (1ll << 31),
+               "planmoe_forward_int8_single_ceiling: needs a capacity of at least samples / 4");
+    PM_REQUIRE(aligned16(x) && aligned16(codes) && (reinterpret_cast<uintptr_t>(workspace) & 7u) == 0,
+               "planmoe_forward_int8_single_ceiling: bad alignment");
+    PM_REQUIRE(workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
+               "planmoe_forward_int8_single_ceiling: workspace too small");
+    PM_REQUIRE(mode >= 0 && mode <= 2, "planmoe_forward_int8_single_ceiling: mode is 0, 1 or 2");
+    hipStream_t st = (hipStream_t)stream;
+    int dev = 0, per_cu = 0, cus = 0;
+    PM_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < STATIC_SCRATCH_DEVICES_MAX,
+               "planmoe_forward_int8_single_ceiling: no current device");
+    // like the kernel it stands in for: every work-group must be resident at once
+    const void *fn = mode == 0 ? (const void *)forward_single_ceiling_kernel<0> : mode == 1 ? (const void *)forward_single_ceiling_kernel<1>
+                               : (const void *)forward_single_ceiling_kernel<2>;
+    PM_REQUIRE(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, FS_THREADS, 0) == hipSuccess &&
+               hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+               groups <= per_cu * cus, "planmoe_forward_int8_single_ceiling: more work-groups than fit on the GPU at once");
+    SingleOrder &order = g_single_order[dev];
+    const bool ordered = !stream_is_capturing(st);
+    std::unique_lock<std::mutex> hold(order.lock);
+    if (ordered) {
+        if (!order.done)
+            PM_REQUIRE(hipEventCreateWithFlags(&order.done, hipEventDisableTiming) == hipSuccess,
+                       "planmoe_forward_int8_single_ceiling: cannot create an event");
+        if (order.recorded && order.last != st)
+            PM_REQUIRE(hipStreamWaitEvent(st, order.done, 0) == hipSuccess,
+                       "planmoe_forward_int8_single_ceiling: cannot wait for the launch before this one");
+    }
+    const int spins = spin_limit > 0 ? spin_limit : (1 << 20);
+#define PM_CEIL(MODE_) forward_single_ceiling_kernel<MODE_><<<groups, FS_THREADS, 0, st>>>((const uint4 *)x, samples, capacity, \
+            codes, (uint16_t *)bias, (uint16_t *)scale, planes, workspace, process_salt(), spins, gave_up)
+    if (mode == 0) PM_CEIL(0); else if (mode == 1) PM_CEIL(1); else PM_CEIL(2);
+#undef PM_CEIL
+    if (ordered) {
+        PM_REQUIRE(hipEventRecord(order.done, st) == hipSuccess, "planmoe_forward_int8_single_ceiling: cannot record an event");
+        order.last = st;
+        order.recorded = true;
+    }
+    hold.unlock();
+    PM_LAUNCH_CHECK("planmoe_forward_int8_single_ceiling");
+    return 0;
 }
 
 #ifdef PM_FS_TRACE
@@ -1072,6 +1175,7 @@ extern "C" int planmoe_forward_int8_redispatch(const void *x, int dtype, int sam
     const int vec = dtype == PLANMOE_F32 ? 4 : 8;
     PM_REQUIRE(model_dim % vec == 0 && aligned16(x) && (uintptr_t)codes % 8 == 0,
                "planmoe_forward_int8_redispatch: bad alignment");
+    workspace = fwd_tables(workspace);
     FwdPlan plan;
     fwd_plan(plan, workspace, samples, experts, top_k);
     if (run_dispatch_routed(x, dtype, samples, model_dim, experts, capacity, indices, locations,

@@ -57,6 +57,8 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 constexpr size_t FS_COUNTER_OFFSET = 256;
 constexpr size_t FS_PUB_OFFSET = FS_COUNTER_OFFSET + (size_t)(FS_MAX_GROUPS / FS_SHARE) * FS_COUNTER_STRIDE;
 __host__ __device__ inline size_t fs_pub_bytes(int groups) { return FS_PUB_OFFSET + (size_t)groups * (16 + 16) * 8; }
+static_assert(FS_PUB_OFFSET + (size_t)FS_MAX_GROUPS * (16 + 16) * 8 <= FWD_TABLES_OFFSET,
+              "the one-launch kernel's region ends where the tables of the other entry points begin");
 
 template <int NMMA> struct FsGeom {
     static constexpr int M = 256 * NMMA;          // model_dim: every wave owns M / 8 elements of a row
@@ -368,8 +370,15 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
     }
     FS_STAMP(7);
     if (!all) {
-        // not every group showed up in time: none of this group's rows is written
+        // not every group showed up in time: none of this group's rows is written.  So that a partial
+        // result cannot pass for a whole one, the group's tokens are marked dropped (location =
+        // capacity) and the loss becomes NaN; the flag is what the caller goes by
         if (tid == 0 && gave_up) __hip_atomic_store(gave_up, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int i = tid; i < k * TOK; i += FS_THREADS) {
+            const int j = i / TOK, t = t0 + i % TOK;
+            if (t < samples) locations[(int64_t)j * stride + t] = capacity;
+        }
+        if (tid == 0 && l_aux) *l_aux = __uint_as_float(0x7fc00000u);
         if (tid == 0 && grp == groups - 1) __hip_atomic_store(launches, launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return;
     }
@@ -568,7 +577,9 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
                     for (int i = 0; i < MG; ++i) me += s_mepart[i][ee];
                     a += me * ((float)s_full[0][ee] * ((float)experts / (float)samples));
                 }
-                *l_aux = a / (float)samples;
+                // (a group that gave up has made the loss NaN: it stays NaN)
+                const bool whole = !gave_up || __hip_atomic_load(gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0;
+                *l_aux = whole ? a / (float)samples : __uint_as_float(0x7fc00000u);
             }
         }
     }

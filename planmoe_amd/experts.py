@@ -46,18 +46,27 @@ class FusedExpertsNetwork(torch.nn.Module):
         y = torch.add(torch.matmul(y, self.batched_fc2_w), self.batched_fc2_bias.unsqueeze(1))
         return y
 
-    def forward_from_codes(self, codes, bias, scale, exact=False):
+    def forward_from_codes(self, codes, bias, scale, exact=True):
         """The same forward with the int8 codes of the receive buffer as input (inference: no autograd
         through the first GEMM): the GEMM reads the codes, so the decompressed [E, C, model_dim]
-        tensor is never written.  exact=False: planmoe_ffn_fc1_int8_affine (scale / bias in the
-        epilogue, about an ulp from decompress + GEMM); exact=True: planmoe_ffn_fc1_int8 (multiplies
-        the decompressor's very values).  bf16; model_dim % 64 == 0, hidden % 128 == 0."""
+        tensor is never written.  exact=True (the default): planmoe_ffn_fc1_int8 multiplies the
+        decompressor's very values, so the result is that of decompress + GEMM up to the GEMM's
+        summation order.  exact=False: planmoe_ffn_fc1_int8_affine puts the codes themselves on the
+        matrix cores and applies scale / bias in the epilogue; it skips the decompressor's three
+        roundings per element, which is about an ulp of the result for rows whose range is
+        comparable to their offset and more than that where |bias| >> scale or the weights'
+        column sum cancels -- an approximation to opt into, 1.4 x faster.
+        bf16; model_dim % 64 == 0, hidden % 128 == 0."""
         from . import ops
         w = self.batched_fc1_w
         cached = self._fc1_k_major
-        if cached is None or cached[0] != w._version or cached[1].device != w.device or cached[1].dtype != w.dtype:
+        key = (w._version, w.data_ptr(), w.device, w.dtype)     # (.data swaps change the pointer, not the version)
+        if cached is None or cached[0] != key:
             wk = w.detach().transpose(1, 2).contiguous()                        # [E, hidden, model_dim]
-            cached = (w._version, wk, ops.ffn_weight_colsum(wk))
+            cached = (key, wk, None if exact else ops.ffn_weight_colsum(wk))
+            self._fc1_k_major = cached
+        if not exact and cached[2] is None:
+            cached = (key, cached[1], ops.ffn_weight_colsum(cached[1]))
             self._fc1_k_major = cached
         if exact:
             y = ops.ffn_fc1_int8(codes, bias, scale, cached[1], self.batched_fc1_bias.detach())

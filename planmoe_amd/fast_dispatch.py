@@ -4,7 +4,7 @@ Same names, arguments, defaults and return structure; the work is done by libpla
 (one launch for all k choices instead of one JIT kernel launch per choice)."""
 import torch
 
-from . import losses, ops
+from . import host_route, losses, ops
 from ._lib import PlanMoEError
 from .gating import fast_cumsum_sub_one  # noqa: F401  (re-exported like the reference)
 
@@ -18,6 +18,8 @@ class GatingEncoder(torch.autograd.Function):
         ctx.reshaped_input = reshaped_input
         ctx.config = config
         ctx.gates = list(gates_) if gates_ else None
+        if not reshaped_input.is_cuda:          # host tensors: the reference's CPU entry points, by name
+            return host_route.scatter(config, reshaped_input, ctx.gates)
         return ops.dispatch_fwd(reshaped_input, config.indices_, config.locations_, ctx.gates,
                                 config.num_global_experts, config.capacity)
 
@@ -25,6 +27,9 @@ class GatingEncoder(torch.autograd.Function):
     def backward(ctx, dispatched_input):
         cfg = ctx.config
         dispatched_input = dispatched_input.contiguous()
+        if not dispatched_input.is_cuda:
+            grad_gates = host_route.gate_gradients(cfg, ctx.reshaped_input, dispatched_input) if ctx.gates is not None else []
+            return (None, host_route.gather(cfg, dispatched_input, ctx.gates), *grad_gates)
         grad_data = ops.combine_fwd(dispatched_input, cfg.indices_, cfg.locations_, ctx.gates,
                                     cfg.sample_size, cfg.capacity)
         grad_gates = []
@@ -44,6 +49,8 @@ class GatingDecoder(torch.autograd.Function):
         ctx.expert_output = expert_output
         ctx.config = config
         ctx.gates = list(gates_) if gates_ else None
+        if not expert_output.is_cuda:
+            return host_route.gather(config, expert_output, ctx.gates)
         return ops.combine_fwd(expert_output, config.indices_, config.locations_, ctx.gates,
                                config.sample_size, config.capacity)
 
@@ -51,6 +58,9 @@ class GatingDecoder(torch.autograd.Function):
     def backward(ctx, combined_output):
         cfg = ctx.config
         combined_output = combined_output.contiguous()
+        if not combined_output.is_cuda:
+            grad_gates = host_route.gate_gradients(cfg, combined_output, ctx.expert_output) if ctx.gates is not None else []
+            return (None, host_route.scatter(cfg, combined_output, ctx.gates), *grad_gates)
         grad_expert_output = ops.dispatch_fwd(combined_output, cfg.indices_, cfg.locations_, ctx.gates,
                                               cfg.num_global_experts, cfg.capacity)
         grad_gates = []
@@ -82,18 +92,30 @@ class TutelMoeFastDispatcher:
         self.gates_ = [x.to(self.dtype) for x in gates_]
         self.is_postscore = is_postscore
         self.sample_size, self.capacity = int(self.indices_[0].size(0)), int(capacity) or self.capacity
-        if not self.indices_[0].is_cuda:
-            raise PlanMoEError("fast_dispatcher: routing tensors must live on the GPU "
-                               "(this build has no CPU kernels)")
-        self.is_cuda = True
+        self.is_cuda = self.indices_[0].is_cuda
+
+    def _host(self, data):
+        # fast_dispatch.py:105-113: host routing tensors select the CPU kernels; they take fp32 / fp64
+        # rows (jit_compiler.py:40-49), so other dtypes pass through the dispatcher's compute dtype
+        if data.is_cuda:
+            raise PlanMoEError("fast_dispatcher: routing tensors on the host, data on the GPU")
+        return data.to(self.original_dtype if self.original_dtype is torch.float64 else self.dtype).contiguous()
 
     def encode(self, data):
+        if not self.is_cuda:
+            host = self._host(data)
+            out = GatingEncoder.apply(self, host) if self.is_postscore else GatingEncoder.apply(self, host, *self.gates_)
+            return out.to(self.original_dtype)
         data = data.to(self.original_dtype).contiguous()
         if self.is_postscore:
             return GatingEncoder.apply(self, data)
         return GatingEncoder.apply(self, data, *self.gates_)
 
     def decode(self, data):
+        if not self.is_cuda:
+            host = self._host(data)
+            out = GatingDecoder.apply(self, host, *self.gates_) if self.is_postscore else GatingDecoder.apply(self, host)
+            return out.to(self.original_dtype)
         data = data.to(self.original_dtype).contiguous()
         if self.is_postscore:
             return GatingDecoder.apply(self, data, *self.gates_)
@@ -145,7 +167,9 @@ def extract_critical(scores, top_k, loss_fn=losses.gshard_loss, capacity_factor=
     the order of their largest score, highest first.  The reference sorts with an unstable
     argsort; here tokens with equal importance keep their token order."""
     if not scores.is_cuda:
-        raise PlanMoEError("extract_critical: scores must live on the GPU (no CPU path in this build)")
+        # host scores: the reference's torch ops (an explicit branch; GPU scores never take it)
+        return host_route.extract_critical(scores, top_k, loss_fn, capacity_factor, batch_prioritized_routing,
+                                           normalize_gate, alignment)
     num_global_experts = int(scores.size(1))
     top_k = min(top_k, num_global_experts)
     want_kernel_loss = loss_fn is losses.gshard_loss

@@ -7,7 +7,10 @@ CAP_FACTOR), error texts and dtype flow of moe_layer.py:44-311.
 
 forward() picks, per call, the most fused send / receive side whose conditions the call meets
 (`_SendPlan`); every choice gives the routing and the bits of the step-by-step pipeline, which is
-the last choice and the reference's own structure."""
+the last choice and the reference's own structure.  Two exceptions, both in the experts and both
+tolerance-level as any GEMM is: under no_grad the built-in FFN's first GEMM reads the int8 codes
+(the decompressor's very values, summed in this kernel's order, overlap.FFN_FROM_CODES), and
+overlap.FFN_FROM_CODES_AFFINE opts into a faster form that skips the decompressor's roundings."""
 import logging
 import os
 import re

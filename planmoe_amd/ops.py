@@ -465,6 +465,33 @@ def forward_int8_single(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None
     return out
 
 
+class ForwardCeiling:
+    """planmoe_forward_int8_single_ceiling with its buffers allocated once: the grid, loads, exchange
+    and stores of the one-launch chain without its arithmetic (mode 0), without the wait at the
+    exchange (mode 1), or with the two-half dealing (mode 2).  A measuring stick; the outputs mean
+    nothing.  16384 x 4096 bf16, 8 experts, top-2."""
+
+    def __init__(self, x, experts, top_k, capacity_):
+        _need_gpu(x, "forward_ceiling")
+        self.x = _contig(x, "forward_ceiling")
+        T, M = x.shape
+        dev = x.device
+        self.shape = (T, M, int(experts), int(top_k), int(capacity_))
+        R = experts * capacity_
+        self.codes = torch.empty((R, M), dtype=torch.uint8, device=dev)
+        self.bias = torch.empty((R,), dtype=torch.bfloat16, device=dev)
+        self.scale = torch.empty((R,), dtype=torch.bfloat16, device=dev)
+        self.planes = torch.empty((3 * top_k * T,), dtype=torch.int32, device=dev)
+        self.gave_up = torch.zeros((), dtype=torch.int32, device=dev)
+        self.ws = torch.empty((lib.planmoe_forward_workspace_bytes(T, experts, top_k),), dtype=torch.uint8, device=dev)
+
+    def run(self, mode=0):
+        T, M, E, k, C = self.shape
+        check(lib.planmoe_forward_int8_single_ceiling(_ptr(self.x), T, M, E, k, C, _ptr(self.codes), _ptr(self.bias),
+                                                      _ptr(self.scale), _ptr(self.planes), _ptr(self.ws), self.ws.numel(),
+                                                      int(mode), 0, _ptr(self.gave_up), _stream(self.x)))
+
+
 def forward_int8_static(x, wg, top_k, capacity_, out, fp32_gate=True, logit_bias=None, normalize_gate=True):
     """forward_int8 through the entry point that allocates nothing: the workspace is the library's
     built-in device buffer and every output is the caller's (`out`: the dict of tensors a

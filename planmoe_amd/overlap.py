@@ -1,7 +1,8 @@
 """Compress -> comm -> decompress pipeline -- mirror of the reference's impls/overlap.py.
 
-One GPU: the comm step is the identity copy and the chunks run back to back on the current
-stream (no comm streams to overlap with)."""
+One GPU: the comm step is a copy on the device's comm stream between two events
+(compressor.comm_operation), so with a2a_ffn_overlap_degree > 1 a chunk's copy runs beside the
+next chunk's compress; the fused int8 / zfp paths below collapse the steps either side of it."""
 import torch
 
 from . import compressor as _ck
@@ -110,15 +111,20 @@ FUSE_INT8 = True
 # one step further: the gate GEMM and the routing join the send side (planmoe_forward_int8)
 FUSE_GATE = True
 # and with this the send side is the one-launch kernel that reads the tokens once
-# (planmoe_forward_int8_single) wherever it serves the shape.  Off by default: two such launches
-# running at the same time on one GPU (two layers on two streams) can keep each other's
-# work-groups from becoming resident until their bounded wait runs out; the backward pass of the
-# layer then raises.  Safe, and 5 us faster at 16384 x 4096, when one stream runs the layers.
-FORWARD_SINGLE_LAUNCH = False
+# (planmoe_forward_int8_single) wherever it serves the shape.  The library keeps such launches on
+# one device apart (each waits for the one before it, whatever their streams), and the layer
+# reads the kernel's give-up flag before it uses any output: a launch whose work-groups did not
+# all become resident in time (another long kernel holding compute units) is run again through the
+# two launches of planmoe_forward_int8.  That read is one host synchronisation per forward pass;
+# under a graph capture, where the host cannot read, the layer takes the two launches.
+FORWARD_SINGLE_LAUNCH = True
 # inference (no autograd) with the built-in expert FFN in bf16: the receive side hands the int8
-# codes straight to the experts' first GEMM (planmoe_ffn_fc1_int8_affine) instead of decompressing
-# them into a tensor first
+# codes straight to the experts' first GEMM (planmoe_ffn_fc1_int8, which multiplies the values the
+# decompressor would have written) instead of decompressing them into a tensor first
 FFN_FROM_CODES = True
+# the faster affine form of that GEMM (codes on the matrix cores, scale / bias in the epilogue):
+# not bit-equal to decompress + GEMM, so it is something to opt into
+FFN_FROM_CODES_AFFINE = False
 
 
 def ffn_from_codes_fn(module, x, degree, reserve_dims):
@@ -130,7 +136,20 @@ def ffn_from_codes_fn(module, x, degree, reserve_dims):
             module.hidden_size_per_expert % 128 == 0 and module.batched_fc1_w.dtype == torch.bfloat16 and
             module.output_dim in (None, x.shape[-1])):
         return None
+    if FFN_FROM_CODES_AFFINE:
+        return lambda codes, bias, scale: module.forward_from_codes(codes, bias, scale, exact=False)
     return module.forward_from_codes
+
+
+def forward_int8_send_side(x, w, top_k, capacity, fp32_gate, normalize_gate, **want):
+    """ops.forward_int8_single where it serves the shape, checked: if a work-group gave up, the
+    chain runs again in two launches.  Never returns a partial result."""
+    if (FORWARD_SINGLE_LAUNCH and ops.forward_int8_single_serves(x, w, top_k) and
+            not torch.cuda.is_current_stream_capturing()):
+        out = ops.forward_int8_single(x, w, top_k, capacity, fp32_gate=fp32_gate, normalize_gate=normalize_gate, **want)
+        if int(out.pop("gave_up")) == 0:
+            return out
+    return ops.forward_int8(x, w, top_k, capacity, fp32_gate=fp32_gate, normalize_gate=normalize_gate, **want)
 
 
 class _EncodeInt8(torch.autograd.Function):
@@ -175,22 +194,16 @@ class _DecodeInt8(torch.autograd.Function):
 
 
 class _GateRouteEncodeInt8(torch.autograd.Function):
-    """Gate GEMM + softmax / top-k / capacity slots + fast_encode + Compress in the two launches
-    of planmoe_forward_int8, then Decompress.  Outputs: the [E*C, M] tensor the experts see, the
+    """Gate GEMM + softmax / top-k / capacity slots + fast_encode + Compress in the one launch of
+    planmoe_forward_int8_single (the two of planmoe_forward_int8 where that does not serve the
+    shape), then Decompress.  Outputs: the [E*C, M] tensor the experts see, the
     gates [k, T] and l_aux (all three differentiable), indices and locations [k, T].
     Backward: the dispatch gradient as in _EncodeInt8; gates and l_aux go back through
     planmoe_route_bwd to the logits and from there into x and the gate weight (library GEMMs)."""
 
     @staticmethod
     def forward(ctx, x, w, top_k, capacity, fp32_gate, normalize_gate):
-        if FORWARD_SINGLE_LAUNCH and ops.forward_int8_single_serves(x, w, top_k):
-            out = ops.forward_int8_single(x, w, top_k, capacity, fp32_gate=fp32_gate, normalize_gate=normalize_gate,
-                                          want_scores=True, want_counts=True)
-            ctx.gave_up = out["gave_up"]
-        else:
-            out = ops.forward_int8(x, w, top_k, capacity, fp32_gate=fp32_gate, normalize_gate=normalize_gate,
-                                   want_scores=True, want_counts=True)
-            ctx.gave_up = None
+        out = forward_int8_send_side(x, w, top_k, capacity, fp32_gate, normalize_gate, want_scores=True, want_counts=True)
         ctx.save_for_backward(x, w, out["scores"], out["indices"], out["locations"], out["counts"])
         ctx.capacity, ctx.normalize_gate = capacity, normalize_gate
         ctx.mark_non_differentiable(out["indices"], out["locations"])
@@ -200,10 +213,6 @@ class _GateRouteEncodeInt8(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_y, grad_gates, grad_l_aux, *unused):
         x, w, scores, indices, locations, counts = ctx.saved_tensors
-        if ctx.gave_up is not None and int(ctx.gave_up) != 0:
-            raise RuntimeError("planmoe_forward_int8_single: a work-group gave up waiting for the others in the forward "
-                               "pass of this layer (two such launches at once on one GPU?); its outputs are incomplete. "
-                               "Set planmoe_amd.overlap.FORWARD_SINGLE_LAUNCH = False.")
         dx = None
         if grad_y is not None:
             codes, bias, scale = ops.int8_compress(grad_y.contiguous())
@@ -316,9 +325,7 @@ def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn, degr
     experts = w.shape[0]
     x = x.contiguous()
     if codes_fn is not None and not torch.is_grad_enabled():
-        single = FORWARD_SINGLE_LAUNCH and ops.forward_int8_single_serves(x, w, top_k)
-        out = (ops.forward_int8_single if single else ops.forward_int8)(
-            x, w.contiguous(), top_k, capacity, fp32_gate=bool(gate.fp32_gate), normalize_gate=bool(normalize_gate))
+        out = forward_int8_send_side(x, w.contiguous(), top_k, capacity, bool(gate.fp32_gate), bool(normalize_gate))
         M = x.shape[-1]
         y = codes_fn(out["codes"].view(experts, capacity, M), out["bias"].view(experts, capacity, 1),
                      out["scale"].view(experts, capacity, 1))

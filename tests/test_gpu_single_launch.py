@@ -38,22 +38,117 @@ def test_single_launch_forward(T, E, k, cf, fp32_gate):
     assert torch.allclose(out["logits"].float(), ref["logits"].float(), rtol=1e-2 if not fp32_gate else 1e-5, atol=1e-5)
     want = oracle.gshard_loss(out["scores"].float().cpu().numpy(), idx[0])
     assert abs(float(out["l_aux"]) - want) <= 1e-5 * abs(want)
-    c2, b2, s2 = ops.dispatch_int8(x, list(out["indices"]), list(out["locations"]), None, E, C)
-    assert torch.equal(out["codes"].view(-1), c2.view(-1))
-    assert np.array_equal(raw(out["bias"]).reshape(-1), raw(b2).reshape(-1))
-    assert np.array_equal(raw(out["scale"]).reshape(-1), raw(s2).reshape(-1))
+    # codes, bias and scale against the oracle itself: its dispatch of the rows to the slots it
+    # worked out, then its restatement of Int8Compressor::compress on the bf16 rows
+    from helpers import bf16_bits
+    d = torch.from_numpy(oracle.encode(x.float().cpu().numpy(), list(idx), list(loc), None, E, C)).bfloat16()
+    rc, rb, rs = oracle.int8_compress(bf16_bits(d))
+    del d
+    assert np.array_equal(out["codes"].cpu().numpy().reshape(-1), rc.reshape(-1))
+    assert np.array_equal(bf16_bits(out["bias"]).reshape(-1), rb.reshape(-1))
+    assert np.array_equal(bf16_bits(out["scale"]).reshape(-1), rs.reshape(-1))
 
 
 def test_single_launch_gives_up_cleanly_when_told_to():
     """spin_limit = 1 with more than one group: some group finds the others not in yet, gives up,
-    writes none of its rows and raises the flag; every work-group still exits."""
+    writes none of its rows and raises the flag; every work-group still exits.  What the groups that
+    finished wrote is the whole result's; the tokens of the groups that gave up are marked dropped and
+    the loss is NaN, so a partial result cannot pass for a whole one."""
     from planmoe_amd import ops
-    T, M, E, k = 16384, 4096, 8, 2
-    x = torch.randn(T, M, device=DEV).bfloat16()
-    wg = (torch.randn(E, M, device=DEV) * M ** -0.5).bfloat16()
-    out = ops.forward_int8_single(x, wg, k, 5120, spin_limit=1)
+    T, M, E, k, C = 16384, 4096, 8, 2, 5120
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(T, M, generator=g).bfloat16().to(DEV)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
+    whole = ops.forward_int8_single(x, wg, k, C, want_scores=True)
+    torch.cuda.synchronize()
+    assert int(whole["gave_up"]) == 0
+    out = ops.forward_int8_single(x, wg, k, C, spin_limit=1)
     torch.cuda.synchronize()
     assert int(out["gave_up"]) in (0, 1)
+    assert torch.equal(out["indices"], whole["indices"])          # routing is every group's own work
+    assert np.array_equal(raw(out["gates"]), raw(whole["gates"]))
+    if int(out["gave_up"]) == 0:
+        assert torch.equal(out["locations"], whole["locations"]) and torch.equal(out["codes"], whole["codes"])
+        return
+    assert bool(torch.isnan(out["l_aux"]))
+    loc, ref = out["locations"], whole["locations"]
+    done = (loc == ref).all(0)                                    # tokens whose group went through
+    # a token of a group that gave up is dropped in every plane ...
+    assert bool((loc[:, ~done] == C).all())
+    # ... and work-groups give up as a whole: runs of 64 tokens
+    assert bool((done.view(-1, 64).all(1) | (~done).view(-1, 64).all(1)).all())
+    # the rows of the groups that went through are where the whole result has them, with its codes
+    idx = out["indices"].long()
+    for j in range(k):
+        keep = done & (loc[j] < C)
+        rows = (idx[j] * C + loc[j].long())[keep]
+        assert torch.equal(out["codes"][rows], whole["codes"][rows])
+        assert np.array_equal(raw(out["scale"][rows]), raw(whole["scale"][rows]))
+
+
+def test_send_side_runs_the_two_launches_when_the_one_launch_gave_up(monkeypatch):
+    """overlap.forward_int8_send_side never hands out a partial result: with a launch that gives up
+    (forced through spin_limit) it returns what planmoe_forward_int8 returns."""
+    from planmoe_amd import ops, overlap
+    T, M, E, k, C = 16384, 4096, 8, 2, 5120
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(T, M, generator=g).bfloat16().to(DEV)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
+    real = ops.forward_int8_single
+    seen = []
+
+    def hurried(*a, **kw):
+        out = real(*a, spin_limit=1, **kw)
+        seen.append(int(out["gave_up"]))
+        return out
+
+    monkeypatch.setattr(ops, "forward_int8_single", hurried)
+    monkeypatch.setattr(overlap, "FORWARD_SINGLE_LAUNCH", True)
+    got = overlap.forward_int8_send_side(x, wg, k, C, True, True, want_counts=True)
+    ref = ops.forward_int8(x, wg, k, C, want_counts=True)
+    torch.cuda.synchronize()
+    assert seen and "gave_up" not in got
+    if seen[0]:
+        for key in ("indices", "locations", "codes", "counts"):
+            assert torch.equal(got[key], ref[key]), key
+    assert not bool(torch.isnan(got["l_aux"]))
+    assert int(got["counts"][0].sum()) == T
+
+
+def test_single_launch_and_two_launch_calls_take_turns_on_one_workspace():
+    """The one-launch kernel's tags are its workspace's launch counter: no other entry point may
+    write that region.  One workspace, one-launch calls at 16384 tokens between two-launch calls at
+    512 tokens and routing-only calls, fresh inputs every time, everything against the oracle."""
+    from helpers import bf16_bits
+    from planmoe_amd import ops
+    M, E, k = 4096, 8, 2
+    g = torch.Generator().manual_seed(21)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
+    for it in range(6):
+        T = 16384
+        x = torch.randn(T, M, generator=g).bfloat16().to(DEV)
+        C = ops.capacity(T, E, k, 1.25, 4)
+        out = ops.forward_int8_single(x, wg, k, C, want_scores=True)
+        torch.cuda.synchronize()
+        assert int(out["gave_up"]) == 0
+        idx, loc, gates, counts = oracle.route_topk(out["scores"].float().cpu().numpy(), k)
+        assert np.array_equal(out["indices"].cpu().numpy(), idx), it
+        assert np.array_equal(out["locations"].cpu().numpy(), loc), it
+        if it in (0, 5):
+            d = torch.from_numpy(oracle.encode(x.float().cpu().numpy(), list(idx), list(loc), None, E, C)).bfloat16()
+            rc, rb, rs = oracle.int8_compress(bf16_bits(d))
+            assert np.array_equal(out["codes"].cpu().numpy().reshape(-1), rc.reshape(-1)), it
+        else:
+            c2, _, _ = ops.dispatch_int8(x, list(out["indices"]), list(out["locations"]), None, E, C)
+            assert torch.equal(out["codes"], c2), it
+        # the same workspace (ops keeps one per device and stream) through the other entry points
+        for Ts in (512, 448 + 64 * it):
+            xs = torch.randn(Ts, M, generator=g).bfloat16().to(DEV)
+            Cs = ops.capacity(Ts, E, k, 1.25, 4)
+            small = ops.forward_int8(xs, wg, k, Cs, want_scores=True)
+            si, sl, _, _ = oracle.route_topk(small["scores"].float().cpu().numpy(), k)
+            assert np.array_equal(small["indices"].cpu().numpy(), si) and np.array_equal(small["locations"].cpu().numpy(), sl)
+            ops.gate_route(xs, wg, k)
 
 
 def test_single_launch_in_a_graph_replayed_with_fresh_inputs():
@@ -124,7 +219,7 @@ def test_moe_layer_with_the_single_launch_send_side():
             torch.cuda.synchronize()
             results.append((y.detach().float(), x.grad.float(), float(y.l_aux.detach()), layer.gates[0].wg.weight.grad.float()))
         finally:
-            overlap.FORWARD_SINGLE_LAUNCH = False
+            overlap.FORWARD_SINGLE_LAUNCH = True
     (y0, g0, l0, w0), (y1, g1, l1, w1) = results
     same_rows = (y0 == y1).all(dim=1).float().mean().item()
     assert same_rows > 0.999
@@ -155,13 +250,55 @@ def test_single_launch_options_against_the_two_launch_entry_point(T, E, k, cap, 
     assert int(got["gave_up"]) == 0
     same = (got["indices"] == ref["indices"]).all(0)
     assert float(same.float().mean()) > 0.98
-    if not bool(same.all()):
-        pytest.skip("a token within an ulp of a tie went elsewhere: slots differ from there on")
-    for key in ("locations", "counts"):
-        assert torch.equal(got[key], ref[key]), key
     assert torch.allclose(got["scores"].float(), ref["scores"].float(), rtol=1e-2 if not fp32_gate else 1e-5, atol=1e-6)
-    assert torch.allclose(got["gates"].float(), ref["gates"].float(), rtol=1e-2 if not fp32_gate else 1e-5, atol=1e-6)
-    assert torch.allclose(got["l_aux"].float(), ref["l_aux"].float(), rtol=1e-4)
+    assert torch.allclose(got["l_aux"].float(), ref["l_aux"].float(), rtol=1e-3)
+    # the routing, against the oracle on the scores this launch reports (the two entry points' gate
+    # GEMMs sum in another order, so a token within an ulp of a tie may go elsewhere in one of them)
+    from helpers import bf16_bits
+    sc = got["scores"].float().cpu().numpy() if fp32_gate else bf16_bits(got["scores"])
+    idx, loc, gates, counts = oracle.route_topk(sc, k, normalize_gate=normalize)
+    assert np.array_equal(got["indices"].cpu().numpy(), idx)
+    assert np.array_equal(got["locations"].cpu().numpy(), loc)
+    assert np.array_equal(raw(got["gates"]), np_raw(gates))
+    assert np.array_equal(got["counts"].cpu().numpy(), counts)
     if cap > 0:
-        assert torch.equal(got["codes"], ref["codes"])
-        assert np.array_equal(raw(got["bias"]), raw(ref["bias"])) and np.array_equal(raw(got["scale"]), raw(ref["scale"]))
+        # the codes, against the oracle's dispatch + compress of the rows to those slots
+        d = torch.from_numpy(oracle.encode(x.float().cpu().numpy(), list(idx), list(loc), None, E, cap)).bfloat16()
+        rc, rb, rs = oracle.int8_compress(bf16_bits(d))
+        assert np.array_equal(got["codes"].cpu().numpy().reshape(-1), rc.reshape(-1))
+        assert np.array_equal(bf16_bits(got["bias"]).reshape(-1), rb.reshape(-1))
+        assert np.array_equal(bf16_bits(got["scale"]).reshape(-1), rs.reshape(-1))
+    if bool(same.all()):
+        for key in ("locations", "counts", "codes"):
+            assert torch.equal(got[key], ref[key]), key
+
+
+def test_ceiling_entry_point_runs_and_leaves_the_chain_alone():
+    """planmoe_forward_int8_single_ceiling (the measuring stick of the one-launch kernel) writes every
+    row of its code buffer in all three modes, shares the workspace's launch counter with the real
+    kernel without disturbing it, and refuses the shapes it does not stand for."""
+    from planmoe_amd import ops
+    from planmoe_amd._lib import PlanMoEError
+    T, M, E, k, C = 16384, 4096, 8, 2, 5120
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(T, M, generator=g).bfloat16().to(DEV)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
+    ref = ops.forward_int8_single(x, wg, k, C)
+    ceil = ops.ForwardCeiling(x, E, k, C)
+    ceil.ws = ops._forward_workspace(T, E, k, x.device)           # the very workspace the real kernel uses
+    for mode in (0, 1, 2, 0):
+        ceil.codes.fill_(0xAA)
+        ceil.run(mode)
+        torch.cuda.synchronize()
+        assert int(ceil.gave_up) == 0
+        rows = ceil.codes.view(E, C, M)
+        assert bool((rows[:, 4096:, :] == 0).all())               # the empty slots
+        assert not bool((rows[:, :4096, :] == 0xAA).all(dim=2).any())   # every used slot was written
+        again = ops.forward_int8_single(x, wg, k, C)
+        torch.cuda.synchronize()
+        assert int(again["gave_up"]) == 0
+        assert torch.equal(again["codes"], ref["codes"]) and torch.equal(again["locations"], ref["locations"])
+    with pytest.raises(PlanMoEError):
+        ops.ForwardCeiling(x[:, :2048].contiguous(), E, k, C).run(0)
+    with pytest.raises(PlanMoEError):
+        ops.ForwardCeiling(x, 16, k, C).run(0)

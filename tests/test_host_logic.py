@@ -20,18 +20,64 @@ def test_fast_cumsum_sub_one_rejects_unsupported_calls():
         planmoe_amd.fast_cumsum_sub_one(torch.zeros(4, 4, dtype=torch.int32), dim=1)
     with pytest.raises(Exception, match="Unimplemented fast_cumsum_sub_one"):
         planmoe_amd.fast_cumsum_sub_one(torch.zeros(4, dtype=torch.int32))
-    with pytest.raises(PlanMoEError):           # no CPU fall-back
-        planmoe_amd.fast_cumsum_sub_one(torch.zeros(4, 4, dtype=torch.int32))
+    # host tensors: torch.cumsum - 1, as jit_kernels/gating.py:13-15 of the reference
+    m = torch.tensor([[1, 0], [0, 1], [1, 1]], dtype=torch.int32)
+    assert planmoe_amd.fast_cumsum_sub_one(m).tolist() == [[0, -1], [0, 0], [1, 1]]
 
 
-def test_cpu_tensors_fail_loudly():
-    with pytest.raises(PlanMoEError):
-        planmoe_amd.extract_critical(torch.rand(4, 2), 1)
+def test_cpu_tensors_fail_loudly_in_the_gpu_entry_points():
+    """The kernels' wrappers take GPU tensors only; host tensors have a route of their own (next
+    test) that is entered by an explicit branch, never as a fall-back."""
     with pytest.raises(PlanMoEError):
         ops.int8_compress(torch.rand(4, 8))
-    d = planmoe_amd.fast_dispatcher(2, 4, 8, torch.float32)
     with pytest.raises(PlanMoEError):
-        d.update([torch.zeros(4, dtype=torch.int32)], [torch.zeros(4, dtype=torch.int32)], [torch.ones(4)], 4)
+        ops.route_topk(torch.rand(4, 2), 1)
+    with pytest.raises(PlanMoEError):
+        ops.dispatch_fwd(torch.rand(4, 8), [torch.zeros(4, dtype=torch.int32)], [torch.zeros(4, dtype=torch.int32)], None, 2, 4)
+
+
+@pytest.mark.parametrize("dtype,k,cf,bpr,postscore", [(torch.float32, 2, 1.0, False, True), (torch.float32, 2, 0.5, False, False),
+                                                      (torch.float64, 1, 1.0, False, True), (torch.float32, 3, 2.0, True, True),
+                                                      (torch.float32, 2, 0.0, False, True), (torch.float32, 2, -0.5, False, False)])
+def test_host_tensors_take_the_reference_cpu_route(dtype, k, cf, bpr, postscore):
+    """fast_dispatch.py:105-113: host tensors go to invoke_cpu_fp32 / fp64 and torch's routing ops.
+    Checked against the oracle (routing, dispatch, combine) and autograd identities."""
+    import numpy as np
+    import oracle
+    from helpers import tie_free_scores
+    T, E, M = 96, 4, 24
+    scores = tie_free_scores(T, E, k, seed=3).to(dtype).requires_grad_(True)
+    x = torch.randn(T, M, generator=torch.Generator().manual_seed(1)).to(dtype).requires_grad_(True)
+    crit, l_loss = planmoe_amd.extract_critical(scores, k, capacity_factor=cf, batch_prioritized_routing=bpr)
+    experts, idx_s, loc_s, gates_s, cap = crit
+    sc = scores.detach().float().numpy()
+    idx, loc, gates, _ = oracle.route_topk(sc, k)
+    assert np.array_equal(torch.stack(idx_s).numpy(), idx)
+    if not bpr:
+        assert np.array_equal(torch.stack(loc_s).numpy(), loc)
+        if cf > 0:
+            assert cap == oracle.capacity(T, E, k, cf, 1)
+    else:
+        order = np.argsort(-sc.max(axis=1), kind="stable").astype(np.int32)
+        want, _ = oracle.route_locations(idx, E, order)
+        assert np.array_equal(torch.stack(loc_s).numpy(), want)
+    assert torch.allclose(torch.stack(gates_s).detach().float(), torch.from_numpy(gates.astype(np.float32)), rtol=1e-5)
+    assert abs(float(l_loss) - oracle.gshard_loss(sc, idx[0])) < 1e-5
+    y = planmoe_amd.fast_encode(x, crit, is_postscore=postscore)
+    assert y.shape == (E, cap, M) and y.dtype == dtype and not y.is_cuda
+    g_in = None if postscore else [g.detach().float().numpy() for g in gates_s]
+    locs_np = [l.numpy() for l in loc_s]
+    want = oracle.encode(x.detach().float().numpy(), list(idx), locs_np, g_in, E, cap)
+    assert torch.allclose(y.detach().float().reshape(-1, M), torch.from_numpy(want), rtol=1e-6, atol=1e-6)
+    out = planmoe_amd.fast_decode(y, crit, is_postscore=postscore)
+    g_out = [g.detach().float().numpy() for g in gates_s] if postscore else None
+    want_out = oracle.decode(want, list(idx), locs_np, g_out, T, cap)
+    assert torch.allclose(out.detach().float(), torch.from_numpy(want_out), rtol=1e-5, atol=1e-6)
+    (out.square().sum() + l_loss).backward()
+    assert x.grad is not None and scores.grad is not None and bool(torch.isfinite(x.grad).all())
+    # dropped tokens get no gradient through the data path
+    dropped = torch.stack([l >= cap for l in loc_s]).all(0)
+    assert bool((x.grad[dropped] == 0).all())
 
 
 def test_plane_packing_detects_views():
