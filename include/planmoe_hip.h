@@ -363,6 +363,31 @@ int planmoe_ffn_fc1_int8_affine(const uint8_t *codes, const void *bias, const vo
                                 const void *fc_bias, int experts, int rows, int model_dim, int hidden,
                                 void *out, void *stream);
 
+/* ---------------------------------------------------------------- expert FFN: batched bf16 GEMM
+ * The batched matrix products of FusedExpertsNetwork (experts/ffn.py:63-82: x @ batched_fc1_w,
+ * activation, @ batched_fc2_w, each followed by torch.add of the bias) and of their backward pass,
+ * on the matrix cores, in the one form a matrix-core operand wants: both operands with the
+ * reduction index running fastest,
+ *   c[e][i][j] = act( bf16( bf16( sum_k a[e][i][k] * b[e][j][k] ) + bias[e][j] ) )
+ * a [batches, m, k] with rows lda elements apart, b [batches, n, k] (ldb), c [batches, m, n] (ldc),
+ * all bf16, batches batch_stride_* elements apart; bias [batches, n] bf16 or NULL (then the sum is
+ * rounded once); activation 0 = none, 1 = relu (the reference's default activation_fn).  The sum is
+ * kept in fp32.  k, n and the pitches must be multiples of 8, one batch of an operand under 4 GiB.
+ *   forward   y  = x @ W (+ bias):  a = x,  b = W transposed to [out, in] (planmoe_transpose_bf16)
+ *   backward  dx = dy @ W^T:        a = dy, b = W as stored [in, out]
+ *             dW = x^T @ dy:        a = x^T [in, rows], b = dy^T [out, rows] (transposed copies whose
+ *                                   k dimension planmoe_transpose_bf16 pads with zeros) */
+int planmoe_gemm_nt_bf16(const void *a, const void *b, const void *bias, int activation, int batches,
+                         int m, int n, int k, int lda, int ldb, int ldc, int64_t batch_stride_a,
+                         int64_t batch_stride_b, int64_t batch_stride_c, void *c, void *stream);
+
+/* out[e][j][i] = in[e][i][j] for bf16 matrices [batches, rows, cols] -> [batches, cols, rows_out];
+ * rows_out >= rows, the columns rows .. rows_out - 1 of out are zero (padding of a reduction index).
+ * cols and rows_out multiples of 8.  Stands for the .transpose(...).contiguous() the GEMM form
+ * above needs for the weights of experts/ffn.py:33-56 and for the operands of their gradients. */
+int planmoe_transpose_bf16(const void *in, int batches, int rows, int cols, int rows_out, void *out,
+                           void *stream);
+
 /* ---------------------------------------------------------------- zfp fixed-rate codec
  * Replaces ZfpCompressor::compress / ::decompress (custom/compressor/zfpc.cpp:23-86), i.e.
  * zfp_compress / zfp_decompress of the third-party zfp library in fixed-rate mode on fp32.

@@ -611,6 +611,49 @@ def ffn_fc1_int8_affine(codes, bias, scale, weight_k_major, weight_colsum=None, 
     return out
 
 
+def transpose_bf16(x, pad_to=1):
+    """[B, R, C] bf16 -> [B, C, R'] with R' = R rounded up to a multiple of pad_to (at least 8), the
+    added columns zero (planmoe_transpose_bf16)."""
+    _need_gpu(x, "transpose_bf16")
+    x = _contig(x, "transpose_bf16")
+    if x.dtype != torch.bfloat16 or x.dim() != 3:
+        raise PlanMoEError("transpose_bf16: a bf16 [batches, rows, cols] tensor")
+    B, R, C = x.shape
+    if C % 8:
+        raise PlanMoEError("transpose_bf16: cols must be a multiple of 8")
+    step = max(8, int(pad_to))
+    Ro = (R + step - 1) // step * step
+    out = torch.empty((B, C, Ro), dtype=torch.bfloat16, device=x.device)
+    check(lib.planmoe_transpose_bf16(_ptr(x), B, R, C, Ro, _ptr(out), _stream(x)))
+    return out
+
+
+def gemm_nt_bf16(a, b, bias=None, relu=False, out=None):
+    """c[e] = act(bf16(bf16(a[e] @ b[e]^T) + bias[e])): a [B, m, k], b [B, n, k] (a [1, n, k] tensor is
+    shared by all batches), bias [B, n] or None, all bf16 -> [B, m, n] bf16 (planmoe_gemm_nt_bf16)."""
+    _need_gpu(a, "gemm_nt_bf16")
+    a, b = _contig(a, "gemm_nt_bf16"), _contig(b, "gemm_nt_bf16")
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or a.dim() != 3 or b.dim() != 3:
+        raise PlanMoEError("gemm_nt_bf16: bf16 [batches, rows, k] operands")
+    B, m, k = a.shape
+    n = b.shape[1]
+    if b.shape[2] != k or b.shape[0] not in (1, B):
+        raise PlanMoEError("gemm_nt_bf16: operands disagree: a %s, b %s" % (tuple(a.shape), tuple(b.shape)))
+    if k % 8 or n % 8:
+        raise PlanMoEError("gemm_nt_bf16: k and n must be multiples of 8 (got k = %d, n = %d)" % (k, n))
+    if bias is not None:
+        bias = _contig(bias.to(torch.bfloat16), "gemm_nt_bf16")
+        if tuple(bias.shape) != (B, n):
+            raise PlanMoEError("gemm_nt_bf16: bias must be [batches, n]")
+    if out is None:
+        out = torch.empty((B, m, n), dtype=torch.bfloat16, device=a.device)
+    elif tuple(out.shape) != (B, m, n) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise PlanMoEError("gemm_nt_bf16: out must be a contiguous bf16 [batches, m, n] tensor")
+    check(lib.planmoe_gemm_nt_bf16(_ptr(a), _ptr(b), _ptr(bias), int(bool(relu)), B, m, n, k, k, k, n, m * k,
+                                   n * k if b.shape[0] == B else 0, m * n, _ptr(out), _stream(a)))
+    return out
+
+
 # ------------------------------------------------------------------------------ zfp codec
 def zfp_stream_bytes(dims, nx, ny, rate=8.0):
     return int(lib.planmoe_zfp_stream_bytes(dims, nx, ny, float(rate)))

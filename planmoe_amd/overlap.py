@@ -120,8 +120,11 @@ FUSE_GATE = True
 FORWARD_SINGLE_LAUNCH = True
 # inference (no autograd) with the built-in expert FFN in bf16: the receive side hands the int8
 # codes straight to the experts' first GEMM (planmoe_ffn_fc1_int8, which multiplies the values the
-# decompressor would have written) instead of decompressing them into a tensor first
-FFN_FROM_CODES = True
+# decompressor would have written) instead of decompressing them into a tensor first.  Off by
+# default since the experts' GEMMs are planmoe_gemm_nt_bf16: at 8 x 5120 x 4096 x 4096 the decode in
+# the first GEMM's prologue makes that GEMM 1.9 ms, against 0.07 ms of planmoe_int8_decompress
+# plus 1.35 ms of the plain GEMM; worth it only where the decompressed tensor's memory is what counts.
+FFN_FROM_CODES = False
 # the faster affine form of that GEMM (codes on the matrix cores, scale / bias in the epilogue):
 # not bit-equal to decompress + GEMM, so it is something to opt into
 FFN_FROM_CODES_AFFINE = False
