@@ -207,7 +207,13 @@ def kernel_table(only=None):
     add("ffn_fc1_int8_affine (GEMM on codes)", "2", R * M + R * 4 + E * Hf * M * 2 + R * Hf * 2,
         lambda: ops.ffn_fc1_int8_affine(codes.view(E, C, M), b.view(E, C, 1), s_.view(E, C, 1), wk, wcs, fb, out=fout), iters=5)
     ffn_flops = 2.0 * R * M * Hf
-    del d, dc, codes, plan, plan1, wk, fout
+    # the experts' GEMMs proper (planmoe_gemm_nt_bf16): the first one with bias + relu on the decompressed
+    # rows, and the transpose that brings an operand into the kernel's form
+    xin = torch.randn(E, C, M, generator=g).bfloat16().to(dev)
+    add("ffn_gemm_nt_bf16 (x @ W + b, relu)", "2", R * M * 2 + E * Hf * M * 2 + R * Hf * 2,
+        lambda: ops.gemm_nt_bf16(xin, wk, fb, relu=True, out=fout), iters=5)
+    add("ffn_transpose_bf16 [8, 5120, 4096]", "2", 2 * R * M * 2, lambda: ops.transpose_bf16(xin, 64), iters=5)
+    del d, dc, codes, plan, plan1, wk, fout, xin
 
     # config 1: 8192 x 2048 fp32, 2 experts, top-2
     T1, M1, E1 = 8192, 2048, 2
@@ -284,7 +290,7 @@ def kernel_table(only=None):
         gbs = nbytes / avg / 1e3
         print("%-36s %-4s %10.1f %9.1f %9.1f %8.0f %6.2f %10.1f %10.1f" % (name, cfg, nbytes / 1e6, avg, best, gbs,
                                                                          gbs / HBM_PEAK_GBS, cold_r, cold_w))
-        if name.startswith("ffn_fc1_int8"):
+        if name.startswith("ffn_fc1_int8") or name.startswith("ffn_gemm"):
             print("%-36s %-4s %10s %9s %9s %8.0f TFLOP/s = %.3f of the %.0f TFLOP/s dense bf16 MFMA peak" % (
                 "  ^ as a GEMM", cfg, "", "", "", ffn_flops / avg / 1e6, ffn_flops / avg / 1e6 / 2500.0, 2500.0))
 

@@ -144,13 +144,43 @@ def ffn_from_codes_fn(module, x, degree, reserve_dims):
     return module.forward_from_codes
 
 
-def forward_int8_send_side(x, w, top_k, capacity, fp32_gate, normalize_gate, **want):
-    """ops.forward_int8_single where it serves the shape, checked: if a work-group gave up, the
-    chain runs again in two launches.  Never returns a partial result."""
-    if (FORWARD_SINGLE_LAUNCH and ops.forward_int8_single_serves(x, w, top_k) and
+class _GaveUp:
+    """The give-up flag of a one-launch forward on its way to the host without stalling the stream:
+    an asynchronous copy into pinned memory and an event behind it.  Asked at the end of the
+    layer's forward pass, when the launch is long done, the answer costs no wait and the host has
+    been free to enqueue everything behind the launch in the meantime."""
+    _slots = {}
+
+    def __init__(self, flag):
+        dev = flag.device.index
+        ring = _GaveUp._slots.get(dev)
+        if ring is None:
+            ring = _GaveUp._slots[dev] = [torch.zeros(64, dtype=torch.int32).pin_memory(), 0]
+        ring[1] = (ring[1] + 1) % 64
+        self.host = ring[0][ring[1]:ring[1] + 1]
+        self.host.copy_(flag.reshape(1), non_blocking=True)
+        self.event = torch.cuda.Event()
+        self.event.record()
+
+    def __bool__(self):
+        self.event.synchronize()
+        return int(self.host) != 0
+
+
+def forward_int8_send_side(x, w, top_k, capacity, fp32_gate, normalize_gate, single=True, checks=None, **want):
+    """ops.forward_int8_single where it serves the shape, else ops.forward_int8.  A one-launch result
+    is valid only if no work-group gave up: with `checks` (a list) the flag's _GaveUp is appended for
+    the caller to ask later (and to run the pass again with single=False if it is set); without, the
+    flag is read here and the two launches run in its place if need be.  Never hands out a partial
+    result unchecked."""
+    if (single and FORWARD_SINGLE_LAUNCH and ops.forward_int8_single_serves(x, w, top_k) and
             not torch.cuda.is_current_stream_capturing()):
         out = ops.forward_int8_single(x, w, top_k, capacity, fp32_gate=fp32_gate, normalize_gate=normalize_gate, **want)
-        if int(out.pop("gave_up")) == 0:
+        flag = out.pop("gave_up")
+        if checks is not None:
+            checks.append(_GaveUp(flag))
+            return out
+        if int(flag) == 0:
             return out
     return ops.forward_int8(x, w, top_k, capacity, fp32_gate=fp32_gate, normalize_gate=normalize_gate, **want)
 
@@ -205,8 +235,9 @@ class _GateRouteEncodeInt8(torch.autograd.Function):
     planmoe_route_bwd to the logits and from there into x and the gate weight (library GEMMs)."""
 
     @staticmethod
-    def forward(ctx, x, w, top_k, capacity, fp32_gate, normalize_gate):
-        out = forward_int8_send_side(x, w, top_k, capacity, fp32_gate, normalize_gate, want_scores=True, want_counts=True)
+    def forward(ctx, x, w, top_k, capacity, fp32_gate, normalize_gate, single=True, checks=None):
+        out = forward_int8_send_side(x, w, top_k, capacity, fp32_gate, normalize_gate, single=single, checks=checks,
+                                     want_scores=True, want_counts=True)
         ctx.save_for_backward(x, w, out["scores"], out["indices"], out["locations"], out["counts"])
         ctx.capacity, ctx.normalize_gate = capacity, normalize_gate
         ctx.mark_non_differentiable(out["indices"], out["locations"])
@@ -221,7 +252,7 @@ class _GateRouteEncodeInt8(torch.autograd.Function):
             codes, bias, scale = ops.int8_compress(grad_y.contiguous())
             dx = ops.combine_int8(codes, bias, scale, list(indices), list(locations), None, x.shape[0], ctx.capacity)
         dx, dw = _gate_backward(x, w, scores, indices, counts, ctx.normalize_gate, dx, grad_gates, grad_l_aux)
-        return dx, dw, None, None, None, None
+        return dx, dw, None, None, None, None, None, None
 
 
 def _gate_backward(x, w, scores, indices, counts, normalize_gate, dx, grad_gates, grad_l_aux):
@@ -318,17 +349,20 @@ def fused_gate_eligible(x, gate, experts, compress_name, degree, is_postscore):
             experts <= 64 and x.shape[0] >= 1 and gate_weight_fits(gate, x))
 
 
-def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn, degree=1, codes_fn=None):
+def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn, degree=1, codes_fn=None, single=True):
     """moe_layer's forward from the gate to the combine for the int8 compressor, the GShard loss
     and plain routing.  Returns (output [T, M], l_aux).  codes_fn (inference only): the experts as a
-    function of the codes, see ffn_from_codes_fn."""
+    function of the codes, see ffn_from_codes_fn.  The one-launch send side is checked at the end
+    (by then its flag has long arrived): if a work-group gave up, the pass runs again in two launches."""
     w = gate.wg.weight
     if w.dtype != x.dtype:
         w = w.to(x.dtype)
     experts = w.shape[0]
     x = x.contiguous()
+    checks = []
     if codes_fn is not None and not torch.is_grad_enabled():
-        out = forward_int8_send_side(x, w.contiguous(), top_k, capacity, bool(gate.fp32_gate), bool(normalize_gate))
+        out = forward_int8_send_side(x, w.contiguous(), top_k, capacity, bool(gate.fp32_gate), bool(normalize_gate),
+                                     single=single, checks=checks)
         M = x.shape[-1]
         y = codes_fn(out["codes"].view(experts, capacity, M), out["bias"].view(experts, capacity, 1),
                      out["scale"].view(experts, capacity, 1))
@@ -336,14 +370,17 @@ def fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn, degr
         k = out["indices"].shape[0]
         res = ops.combine_int8(codes, bias, scale, list(out["indices"]), list(out["locations"]),
                                [out["gates"][j].float() for j in range(k)], x.shape[0], capacity)
-        return res, out["l_aux"]
-    y, gates, l_aux, indices, locations = _GateRouteEncodeInt8.apply(x, w.contiguous(), top_k, capacity,
-                                                                     bool(gate.fp32_gate), bool(normalize_gate))
-    y = _experts_in_chunks(expert_fn, y.view(experts, capacity, x.shape[-1]), degree)
-    y = y.reshape(experts * capacity, -1).to(x.dtype)
-    k = indices.shape[0]
-    out = _DecodeInt8.apply(y, indices, locations, experts, capacity, x.shape[0], *[gates[j].float() for j in range(k)])
-    return out, l_aux
+        l_aux = out["l_aux"]
+    else:
+        y, gates, l_aux, indices, locations = _GateRouteEncodeInt8.apply(x, w.contiguous(), top_k, capacity, bool(gate.fp32_gate),
+                                                                         bool(normalize_gate), single, checks)
+        y = _experts_in_chunks(expert_fn, y.view(experts, capacity, x.shape[-1]), degree)
+        y = y.reshape(experts * capacity, -1).to(x.dtype)
+        k = indices.shape[0]
+        res = _DecodeInt8.apply(y, indices, locations, experts, capacity, x.shape[0], *[gates[j].float() for j in range(k)])
+    if any(bool(c) for c in checks):
+        return fused_gate_forward(x, gate, top_k, capacity, normalize_gate, expert_fn, degree, codes_fn, single=False)
+    return res, l_aux
 
 
 # ------------------------------------------------------------------------------ fused zfp path

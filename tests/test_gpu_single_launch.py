@@ -113,6 +113,55 @@ def test_send_side_runs_the_two_launches_when_the_one_launch_gave_up(monkeypatch
             assert torch.equal(got[key], ref[key]), key
     assert not bool(torch.isnan(got["l_aux"]))
     assert int(got["counts"][0].sum()) == T
+    # the deferred form: the flag comes back as a check to ask later
+    checks = []
+    part = overlap.forward_int8_send_side(x, wg, k, C, True, True, checks=checks)
+    assert len(checks) == 1 and bool(checks[0]) == bool(seen[-1]) and "gave_up" not in part
+
+
+def test_layer_runs_again_in_two_launches_when_the_one_launch_gave_up(monkeypatch):
+    """moe_layer with a one-launch send side that is made to give up: the layer's output, loss and
+    gradients are those of the layer on the two-launch send side."""
+    import planmoe_amd
+    from planmoe_amd import ops, overlap
+
+    class Identity(torch.nn.Module):
+        def update(self, ctx):
+            self.dummy = torch.nn.Parameter(torch.zeros(1))
+
+        def forward(self, x, ctx):
+            return x
+
+    T, M, E = 16384, 4096, 8
+    layer = planmoe_amd.moe_layer({'type': 'top', 'k': 2, 'capacity_factor': 1.25, 'fp32_gate': True}, M,
+                                  experts={'type': 'custom', 'module': Identity(), 'count_per_node': E},
+                                  seeds=(1, 2, 3), compress_name='int8').to(DEV).to(torch.bfloat16)
+    x = torch.randn(T, M, generator=torch.Generator().manual_seed(0)).bfloat16().to(DEV)
+
+    def run():
+        xi = x.clone().requires_grad_(True)
+        y = layer(xi)
+        (y.float().square().mean() + y.l_aux.float()).backward()
+        torch.cuda.synchronize()
+        return y.detach(), float(y.l_aux.detach()), xi.grad
+
+    monkeypatch.setattr(overlap, "FORWARD_SINGLE_LAUNCH", False)
+    y0, l0, g0 = run()
+    monkeypatch.setattr(overlap, "FORWARD_SINGLE_LAUNCH", True)
+    real = ops.forward_int8_single
+    seen = []
+
+    def hurried(*a, **kw):
+        out = real(*a, spin_limit=1, **kw)
+        seen.append(int(out["gave_up"]))
+        return out
+
+    monkeypatch.setattr(ops, "forward_int8_single", hurried)
+    y1, l1, g1 = run()
+    assert seen
+    if seen[0]:
+        assert torch.equal(y0, y1) and l0 == l1 and torch.equal(g0, g1)
+    assert bool(torch.isfinite(y1.float()).all()) and l1 == l1
 
 
 def test_single_launch_and_two_launch_calls_take_turns_on_one_workspace():
