@@ -184,12 +184,15 @@ __global__ __launch_bounds__(256, 1) void gemm_nt_bf16_kernel(const GemmArgs p)
 
 // ---- the same product with the operands loaded straight into LDS (global_load_lds_dwordx4: the
 // memory pipeline writes LDS itself, 16 bytes per lane at consecutive addresses, no register and no
-// LDS-store instruction in between).  k-tiles of 32; LDS holds four of them for both operands and
-// the loads run three tiles ahead of the MFMAs, which is what hides the latency of the loads from
-// a kernel with one wave per SIMD.  A load instruction fills 1 KB = 16 rows of 64 bytes; which
-// 16-byte chunk of its row a lane fetches is chosen so that the chunk c of row r lies at unit
-// c ^ ((r >> 1) + (r >> 3)) & 3 of the row: the rows that one pass of a fragment read touches then
-// fall into different banks whether the LDS serves 32 or 64 banks per clock.  Needs k % 32 == 0.
+// LDS-store instruction in between).  k-tiles of 64; LDS holds two of them for both operands and
+// the loads of a tile are in flight during the MFMAs of the tile before it.  A load instruction
+// fills 1 KB = 8 rows of 128 bytes; which 16-byte chunk of its row a lane fetches is chosen so
+// that chunk c of row r lies at unit c ^ (r >> 1) & 7 of the row.  The LDS of this GPU serves 64
+// banks (256 bytes) per clock, a 16-byte read 16 lanes at a time: the 16 consecutive rows of such a
+// pass are 8 pairs of rows, the rows of a pair in different halves of the 256 bytes, the pairs at
+// 8 different units.  (Measured with SQ_LDS_BANK_CONFLICT: 1.3 M conflict cycles per launch at
+// 8 x 5120 x 4096 x 4096 against 85 M with c ^ r & 7, which would suit an LDS of 32 banks.)
+// Needs k % 64 == 0.
 constexpr int DMA_BK = 64, DMA_STAGES = 2;
 constexpr int DMA_ROW = DMA_BK * 2;                         // bytes of a row of a k-tile
 constexpr int DMA_OPERAND = 256 * DMA_ROW;                  // bytes of one operand's k-tile
@@ -203,7 +206,7 @@ __device__ __forceinline__ void gemm_dma16(const void *gbase, uint32_t voff, uin
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(lds_addr), "v"(voff), "s"(gbase) : "memory", "m0");
 }
 // where chunk c of row r lies in its row of 8 units
-__device__ __forceinline__ int dma_unit(int row, int chunk) { return chunk ^ ((row + (row >> 3)) & 7); }
+__device__ __forceinline__ int dma_unit(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
 
 template <int ACT>
 __global__ __launch_bounds__(256, 1) void gemm_nt_bf16_dma_kernel(const GemmArgs p)
