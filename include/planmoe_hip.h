@@ -274,8 +274,9 @@ int planmoe_forward_int8(const void *x, const void *wg, int dtype, int fp32_gate
  * caller reads that word before it uses any output and, if it is set, runs planmoe_forward_int8.
  * Two such launches that run at the same time on one GPU could keep each other's work-groups from
  * becoming resident, so the library puts them in a row: a launch on another stream than the one
- * before it on the same device first waits (on the device) for that launch's event.  Launches
- * recorded into a HIP graph are outside that order: keep replays of such graphs apart.
+ * before it on the same device first waits (on the device) for an event recorded at the tail of
+ * that earlier stream.  Launches recorded into a HIP graph are outside that order: keep replays
+ * of such graphs apart.
  * The first FWD region of the workspace (its launch counter and published words) is written by
  * this entry point alone; the other entry points that take a forward workspace keep their tables
  * behind it, so one workspace may serve all of them in turn, whatever the shapes.

@@ -840,16 +840,18 @@ static unsigned long long process_salt()
 
 // Two one-launch kernels that run at the same time on one GPU can keep each other's work-groups
 // from becoming resident, and then both wait until their bound.  So launches of the kernel on one
-// device are put in a row on the host: behind every launch an event is recorded, and a launch on
-// another stream first makes its stream wait for the event of the launch before it.  (Launches on
-// one stream follow each other anyway.  A stream that is being captured into a graph is left
-// alone: neither the wait nor the record belongs into the caller's graph; replays of such graphs
-// are the caller's to keep apart.)
+// device are put in a row on the host.  Launches on one stream follow each other anyway and cost
+// nothing extra; when a launch comes in on another stream than the one before it, an event is
+// recorded at the tail of that earlier stream (behind its launch, and behind whatever followed it
+// there) and the new stream waits for it on the device.  (An event behind every launch would put a
+// marker between back-to-back launches of one stream: 4 us each, measured.  A stream that is being
+// captured into a graph is left alone: neither the wait nor the record belongs into the caller's
+// graph; replays of such graphs are the caller's to keep apart.)
 struct SingleOrder {
     std::mutex lock;
     hipEvent_t done = nullptr;
     hipStream_t last = nullptr;
-    bool recorded = false;
+    bool has_last = false;
 };
 static SingleOrder g_single_order[STATIC_SCRATCH_DEVICES_MAX];
 
@@ -858,6 +860,25 @@ static bool stream_is_capturing(hipStream_t st)
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &status) != hipSuccess) { (void)hipGetLastError(); return false; }
     return status != hipStreamCaptureStatusNone;
+}
+
+// Call with order.lock held, before the launch on `st`.  0, or 1 with the error text set.
+static int single_order_before(SingleOrder &order, hipStream_t st, bool ordered, const char *who)
+{
+    if (!ordered || !order.has_last || order.last == st || stream_is_capturing(order.last)) return 0;
+    if (!order.done && hipEventCreateWithFlags(&order.done, hipEventDisableTiming) != hipSuccess)
+        return fail("%s: cannot create an event", who);
+    if (hipEventRecord(order.done, order.last) != hipSuccess) {
+        (void)hipGetLastError();              // the earlier stream is gone: so is its work
+        return 0;
+    }
+    if (hipStreamWaitEvent(st, order.done, 0) != hipSuccess)
+        return fail("%s: cannot wait for the launch before this one", who);
+    return 0;
+}
+static void single_order_after(SingleOrder &order, hipStream_t st, bool ordered)
+{
+    if (ordered) { order.last = st; order.has_last = true; }
 }
 
 // Whether the one-launch kernel serves the shape, and with how many rounds: model_dim 4096 bf16, up to
@@ -1021,23 +1042,12 @@ extern "C" int planmoe_forward_int8_single(const void *x, const void *wg, int dt
     SingleOrder &order = g_single_order[dev];
     const bool ordered = !stream_is_capturing(st);
     std::unique_lock<std::mutex> hold(order.lock);
-    if (ordered) {
-        if (!order.done)
-            PM_REQUIRE(hipEventCreateWithFlags(&order.done, hipEventDisableTiming) == hipSuccess,
-                       "planmoe_forward_int8_single: cannot create an event");
-        if (order.recorded && order.last != st)
-            PM_REQUIRE(hipStreamWaitEvent(st, order.done, 0) == hipSuccess,
-                       "planmoe_forward_int8_single: cannot wait for the launch before this one");
-    }
+    if (single_order_before(order, st, ordered, "planmoe_forward_int8_single")) return 1;
     const int rc = run_forward_single(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
                                       normalize_gate, capacity, indices, locations, gates, plane_stride, logits_out,
                                       scores_out, l_aux, expert_counts, codes, bias, scale, workspace,
                                       spin_limit > 0 ? spin_limit : (1 << 20), gave_up, st);
-    if (ordered && rc == 0) {
-        PM_REQUIRE(hipEventRecord(order.done, st) == hipSuccess, "planmoe_forward_int8_single: cannot record an event");
-        order.last = st;
-        order.recorded = true;
-    }
+    if (rc == 0) single_order_after(order, st, ordered);
     hold.unlock();
     PM_REQUIRE(rc != 2, "planmoe_forward_int8_single: the one-launch kernel serves bf16 rows of 4096 values, up to 16 "
                "experts, top_k <= 4 and at most 64 tokens per compute unit; use planmoe_forward_int8");
@@ -1075,24 +1085,13 @@ extern "C" int planmoe_forward_int8_single_ceiling(const void *x, int samples, i
     SingleOrder &order = g_single_order[dev];
     const bool ordered = !stream_is_capturing(st);
     std::unique_lock<std::mutex> hold(order.lock);
-    if (ordered) {
-        if (!order.done)
-            PM_REQUIRE(hipEventCreateWithFlags(&order.done, hipEventDisableTiming) == hipSuccess,
-                       "planmoe_forward_int8_single_ceiling: cannot create an event");
-        if (order.recorded && order.last != st)
-            PM_REQUIRE(hipStreamWaitEvent(st, order.done, 0) == hipSuccess,
-                       "planmoe_forward_int8_single_ceiling: cannot wait for the launch before this one");
-    }
+    if (single_order_before(order, st, ordered, "planmoe_forward_int8_single_ceiling")) return 1;
     const int spins = spin_limit > 0 ? spin_limit : (1 << 20);
 #define PM_CEIL(MODE_) forward_single_ceiling_kernel<MODE_><<<groups, FS_THREADS, 0, st>>>((const uint4 *)x, samples, capacity, \
             codes, (uint16_t *)bias, (uint16_t *)scale, planes, workspace, process_salt(), spins, gave_up)
     if (mode == 0) PM_CEIL(0); else if (mode == 1) PM_CEIL(1); else PM_CEIL(2);
 #undef PM_CEIL
-    if (ordered) {
-        PM_REQUIRE(hipEventRecord(order.done, st) == hipSuccess, "planmoe_forward_int8_single_ceiling: cannot record an event");
-        order.last = st;
-        order.recorded = true;
-    }
+    single_order_after(order, st, ordered);
     hold.unlock();
     PM_LAUNCH_CHECK("planmoe_forward_int8_single_ceiling");
     return 0;

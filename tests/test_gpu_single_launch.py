@@ -351,3 +351,30 @@ def test_ceiling_entry_point_runs_and_leaves_the_chain_alone():
         ops.ForwardCeiling(x[:, :2048].contiguous(), E, k, C).run(0)
     with pytest.raises(PlanMoEError):
         ops.ForwardCeiling(x, 16, k, C).run(0)
+
+
+def test_single_launch_on_two_streams_at_once():
+    """Two one-launch kernels at the same time on one GPU could keep each other's work-groups from
+    becoming resident; the library puts launches on one device in a row whatever their streams.
+    Two different full-size batches, enqueued alternately on two streams without waiting: nobody
+    gives up and every result is that of the same call made alone."""
+    from planmoe_amd import ops
+    T, M, E, k = 16384, 4096, 8, 2
+    C = ops.capacity(T, E, k, 1.25, 4)
+    g = torch.Generator().manual_seed(41)
+    xs = [torch.randn(T, M, generator=g).bfloat16().to(DEV) for _ in range(2)]
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
+    want = [ops.forward_int8_single(x, wg, k, C) for x in xs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [[], []]
+    for _ in range(6):
+        for i in (0, 1):
+            with torch.cuda.stream(streams[i]):
+                got[i].append(ops.forward_int8_single(xs[i], wg, k, C))
+    torch.cuda.synchronize()
+    for i in (0, 1):
+        for out in got[i]:
+            assert int(out["gave_up"]) == 0
+            for name in ("indices", "locations", "codes", "bias", "scale", "l_aux"):
+                assert torch.equal(out[name].reshape(-1).view(torch.uint8), want[i][name].reshape(-1).view(torch.uint8)), name
