@@ -467,6 +467,67 @@ def overlap_run(passes=6):
     print("outputs of degree 2 equal to degree 1:", bool(torch.equal(outs[0], outs[1])))
 
 
+def phase_table():
+    """Wall-clock stamps of the phases of the one-launch forward kernel and of its ceiling kernel
+    (modes 0 and 1), per work-group, from the measurement build of the library
+    (make -C planmoe_amd/csrc libplanmoe_hip_trace.so: forward.hip with -DPM_FS_TRACE).  Config 2."""
+    import ctypes
+    import subprocess
+    import numpy as np
+    import torch
+    from planmoe_amd import ops, _lib
+    csrc = os.path.join(os.path.dirname(os.path.abspath(__file__)), "planmoe_amd", "csrc")
+    path = os.path.join(csrc, "libplanmoe_hip_trace.so")
+    if not os.path.exists(path):
+        subprocess.check_call(["make", "-C", csrc, "libplanmoe_hip_trace.so"])
+    tl = ctypes.CDLL(path)
+    dev = "cuda:0"
+    T, M, E, k = 16384, 4096, 8, 2
+    C = ops.capacity(T, E, k, 1.25, 4)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(T, M, generator=g).bfloat16().to(dev)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(dev)
+    plan = ops.ForwardInt8Plan(x, wg, k, C, fp32_gate=True, single=True)
+    a = list(plan._args)
+    fn, cf = tl.planmoe_forward_int8_single, tl.planmoe_forward_int8_single_ceiling
+    fn.restype = cf.restype = ctypes.c_int
+    fn.argtypes = _lib.SIGNATURES["planmoe_forward_int8_single"][1]
+    cf.argtypes = _lib.SIGNATURES["planmoe_forward_int8_single_ceiling"][1]
+    gave = torch.zeros((), dtype=torch.int32, device=dev)
+    st = ops._stream(x)
+    ceil = ops.ForwardCeiling(x, E, k, C)
+
+    def trace(run):
+        for _ in range(5):
+            run()
+        torch.cuda.synchronize()
+        buf = np.zeros(1024 * 16, dtype=np.uint64)
+        tl.planmoe_debug_fs_trace(buf.ctypes.data_as(ctypes.c_void_p))
+        tr = buf.reshape(1024, 16)[:(T + 63) // 64, :16].astype(np.int64)
+        return (tr - tr[:, 0].min()) / 100.0            # the stamps count a 100 MHz clock
+
+    def real():
+        assert fn(*a, 0, ops._ptr(gave), st) == 0
+
+    res = {"forward_single": trace(real)}
+    for mode in (0, 1):
+        def run(mode=mode):
+            assert cf(ops._ptr(x), T, M, E, k, C, ops._ptr(ceil.codes), ops._ptr(ceil.bias), ops._ptr(ceil.scale),
+                      ops._ptr(ceil.planes), ops._ptr(ceil.ws), ceil.ws.numel(), mode, 0, ops._ptr(gave), st) == 0
+        res["ceiling mode %d" % mode] = trace(run)
+    names = {0: "first instruction", 1: "round 0 done", 2: "round 1 done", 3: "round 2 done", 4: "round 3 done + barrier",
+             5: "histogram published", 7: "all groups seen", 8: "slot bases known", 9: "parked rows flushed (wave 0)",
+             10: "register rounds in LDS", 11: "register rounds flushed", 12: "empty slots zeroed (end)"}
+    print("microseconds since the first work-group's first instruction; thread 0 of each of the %d work-groups; median / max" % ((T + 63) // 64))
+    print("%-30s" % "stamp" + "".join("%24s" % n for n in res))
+    for i, n in names.items():
+        print("%-30s" % n + "".join("%14.2f %9.2f" % (np.median(r[:, i]), r[:, i].max()) for r in res.values()))
+    for n, r in res.items():
+        print("%-16s published at (percentiles 0/10/50/90/100) %s | ended at %s" % (
+            n, " ".join("%.1f" % np.percentile(r[:, 5], p) for p in (0, 10, 50, 90, 100)),
+            " ".join("%.1f" % np.percentile(r[:, 12], p) for p in (0, 10, 50, 90, 100))))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -489,6 +550,9 @@ def main():
     ap.add_argument("--cpu-stages", action="store_true",
                     help="instead of the JSON line, time the CPU oracle (one thread) stage by stage on bounded "
                          "samples of the same workloads; needs no GPU")
+    ap.add_argument("--phases", action="store_true",
+                    help="instead of the JSON line, print the phase stamps of the one-launch forward kernel and of its "
+                         "ceiling kernel from the measurement build of the library")
     ap.add_argument("--only", default=None, help="with --kernels: only the lines whose 'name [config]' contains this, e.g. lz_ or [5]")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -499,10 +563,12 @@ def main():
         __graft_entry__.ensure_built()
         cpu_stage_table()
         return
-    if args.kernels or args.layer or args.overlap:
+    if args.kernels or args.layer or args.overlap or args.phases:
         import __graft_entry__
         __graft_entry__.ensure_built()
-        if args.kernels:
+        if args.phases:
+            phase_table()
+        elif args.kernels:
             kernel_table(args.only)
         elif args.layer:
             layer_table()

@@ -92,6 +92,7 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_ceiling_kernel(
         return __ballot(!ok) == 0;
     };
 
+    FS_STAMP(0);
     {
         const uint4 *p0 = row_ptr(0), *p1 = row_ptr(1);
 #pragma unroll
@@ -101,7 +102,9 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_ceiling_kernel(
     }
     bool early = false;
     round(std::integral_constant<int, 0>{}, buf0);
+    FS_STAMP(1);
     round(std::integral_constant<int, 1>{}, buf1);
+    FS_STAMP(2);
     if constexpr (MODE == 2) {
         lds_barrier();
         publish(1);
@@ -113,8 +116,10 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_ceiling_kernel(
             for (int tok = w; tok < 32; tok += FS_WAVES) flush_row(tok, tok, 1);
         }
     }
+    FS_STAMP(3);
     round(std::integral_constant<int, 3>{}, buf1);
     lds_barrier();
+    FS_STAMP(4);
     // the routing planes: 3 x [2][samples] words
     if (tid < TOK * K) {
         const int tok = tid % TOK, j = tid / TOK;
@@ -126,6 +131,7 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_ceiling_kernel(
         }
     }
     publish(0);
+    FS_STAMP(5);
 
     bool all = MODE == 1;
     for (int spin = 0; spin <= spin_limit && MODE != 1; ++spin) {
@@ -146,8 +152,11 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_ceiling_kernel(
         return;
     }
 
+    FS_STAMP(7);
+    FS_STAMP(8);
     // phase 2: the parked rows, then the register rounds through the same LDS rows, then the zero rows
     for (int tok = w; tok < 32; tok += FS_WAVES) flush_row(tok, tok, early ? 2 : 3);
+    FS_STAMP(9);
     lds_barrier();
 #pragma unroll
     for (int i = 0; i < NMMA; ++i) {
@@ -155,7 +164,9 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_ceiling_kernel(
         *reinterpret_cast<uint2 *>(my_park + 16 * G::RS + 32 * i) = make_uint2(buf1[i].x ^ buf1[i].y, buf1[i].z ^ buf1[i].w);
     }
     lds_barrier();
+    FS_STAMP(10);
     for (int i = w; i < 32; i += FS_WAVES) flush_row(i, 32 + i, 3);
+    FS_STAMP(11);
     {
         // empty slots: 32 per group, 4 per wave, behind the 4096 used slots of every expert
         const uint4 z[G::RV] = {};
@@ -171,6 +182,7 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_ceiling_kernel(
             }
         }
     }
+    FS_STAMP(12);
     if (grp == groups - 1 && tid == 0) __hip_atomic_store(launches, launch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
