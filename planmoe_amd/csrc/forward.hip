@@ -479,7 +479,11 @@ __global__ __launch_bounds__(256) void route_locations_merged_kernel(
 // itself (hist_t: one or two 16-byte loads per lane and column, k (k + 1) / 2 columns per token),
 // the zero-fill blocks sum the expert totals, and one more block at the end of the grid finishes
 // the GShard loss and the per-plane expert counts.  Used for top_k <= 4.
-template <int DT, int CACHE, bool MERGED>
+// SLOT_FIRST: a token's slots are worked out before its row is requested, and a token that keeps
+// none of its choices leaves without reading its row.  Pays when many tokens are dropped (a
+// capacity factor of 1 with skewed routing drops half of them); otherwise the row is requested
+// first so that it travels while the slots are being worked out.
+template <int DT, int CACHE, bool MERGED, bool SLOT_FIRST = false>
 __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     const void *__restrict__ x, const int32_t *__restrict__ indices, int32_t *__restrict__ locations,
     int64_t stride, int top_k, int samples, int model_dim, int experts, int capacity,
@@ -550,34 +554,47 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     if (t < 0) return;
     const uint4 *src = reinterpret_cast<const uint4 *>((const char *)x + (int64_t)t * model_dim * (int64_t)sizeof(typename E::store_t));
     uint4 cache[CACHE > 0 ? CACHE : 1];
-    if constexpr (CACHE > 0) {
+    auto request_row = [&]() {
+        if constexpr (CACHE > 0) {
 #pragma unroll
-        for (int c = 0; c < CACHE; ++c) {
-            const int u = c * WAVE + lane;
-            // (index clamped, not predicated: straight-line loads let the compiler wait for exactly these
-            // loads; the re-read last vector is harmless for min / max and is never stored)
-            cache[c] = src[min(u, units - 1)];
+            for (int c = 0; c < CACHE; ++c) {
+                const int u = c * WAVE + lane;
+                // (index clamped, not predicated: straight-line loads let the compiler wait for exactly these
+                // loads; the re-read last vector is harmless for min / max and is never stored)
+                cache[c] = src[min(u, units - 1)];
+            }
         }
-    }
-
+    };
     // lane j finalises choice j: slot = expert * capacity + rank in group + group offset
-    int slot = -1;
-    if constexpr (MERGED) {
-        int e_l;
-        const int l = merged_location(indices, rank, hist_t, stride, top_k, samples, experts, t, group_tokens, groups,
-                                      gstride, e_l);
-        if (lane < top_k) {
-            locations[(int64_t)lane * stride + t] = l;
-            if (l < capacity) slot = e_l * capacity + l;
+    auto find_slot = [&]() {
+        int slot = -1;
+        if constexpr (MERGED) {
+            int e_l;
+            const int l = merged_location(indices, rank, hist_t, stride, top_k, samples, experts, t, group_tokens, groups,
+                                          gstride, e_l);
+            if (lane < top_k) {
+                locations[(int64_t)lane * stride + t] = l;
+                if (l < capacity) slot = e_l * capacity + l;
+            }
+        } else if (lane < top_k) {
+            const int64_t o = (int64_t)lane * stride + t;
+            const int e = indices[o];
+            const int l = rank[(int64_t)lane * samples + t] + hist[((int64_t)(t / group_tokens) * top_k + lane) * experts + e];
+            locations[o] = l;
+            if (l < capacity) slot = e * capacity + l;
         }
-    } else if (lane < top_k) {
-        const int64_t o = (int64_t)lane * stride + t;
-        const int e = indices[o];
-        const int l = rank[(int64_t)lane * samples + t] + hist[((int64_t)(t / group_tokens) * top_k + lane) * experts + e];
-        locations[o] = l;
-        if (l < capacity) slot = e * capacity + l;
+        return slot;
+    };
+    int slot;
+    if constexpr (SLOT_FIRST) {
+        slot = find_slot();
+        if (__ballot(slot >= 0) == 0) return;
+        request_row();
+    } else {
+        request_row();
+        slot = find_slot();
+        if (__ballot(slot >= 0) == 0) return;
     }
-    if (__ballot(slot >= 0) == 0) return;
 
     float mn, mx;
     if (row_min) {                                      // the gate kernel already scanned the row
@@ -651,12 +668,15 @@ static void launch_dispatch_routed(int per_lane, unsigned grid, hipStream_t st, 
                                    const int32_t *hist_t, const float *me_t, int groups, int gstride,
                                    int fill_blocks, int32_t *counts, int fill_first)
 {
-#define PM_DR_(CACHE, MERGED)                                                                        \
-    dispatch_int8_routed_kernel<DT, CACHE, MERGED><<<grid, 256, 0, st>>>(x, indices, locations, stride, top_k, \
+    // a capacity factor of at most 1: every imbalance of the routing drops tokens
+    const bool slot_first = merged && (int64_t)experts * capacity <= (int64_t)top_k * samples;
+#define PM_DR_(CACHE, MERGED, FIRST)                                                                 \
+    dispatch_int8_routed_kernel<DT, CACHE, MERGED, FIRST><<<grid, 256, 0, st>>>(x, indices, locations, stride, top_k, \
         samples, model_dim, experts, capacity, codes, bias, scale, offs, totals, rank, group_tokens,  \
         token_blocks, loss_part, loss_parts, l_aux, row_min, row_max, hist_t, me_t, groups, gstride,  \
         fill_blocks, counts, fill_first)
-#define PM_DR(CACHE) do { if (merged) PM_DR_(CACHE, true); else PM_DR_(CACHE, false); } while (0)
+#define PM_DR(CACHE) do { if (slot_first) PM_DR_(CACHE, true, true); else if (merged) PM_DR_(CACHE, true, false); \
+                          else PM_DR_(CACHE, false, false); } while (0)
     if (per_lane <= 2) PM_DR(2);
     else if (per_lane <= 4) PM_DR(4);
     else if (per_lane <= 8) PM_DR(8);

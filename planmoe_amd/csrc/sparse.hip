@@ -63,6 +63,7 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
         const int np = min(top_k - j0, WAVE);
         int slot; float gate;
         fetch_planes(gates, indices, locations, stride, t, j0, np, experts, capacity, slot, gate);
+        if (__ballot(slot >= 0) == 0) continue;          // every choice of this pass dropped: the row is not read
         for (int u = lane; u < units; u += WAVE) {
             float v[IO::U];
             IO::load(src, u, v);
