@@ -168,12 +168,19 @@ def kernel_table(only=None):
     r = ops.gate_route(x, wg, k)
     idx, loc, gates = list(r["indices"]), list(r["locations"]), list(r["gates"])
     live = int(sum(((l >= 0) & (l < C)).sum() for l in loc))                 # token rows that reach a slot
+
+    def kept(locs, cap):
+        """Tokens with at least one slot: a dispatch has no use for the rows of the others."""
+        hit = torch.zeros_like(locs[0], dtype=torch.bool)
+        for l in locs:
+            hit |= (l >= 0) & (l < cap)
+        return int(hit.sum())
     xb, db, plane = T * M * 2, R * M * 2, T * k * 12
     add("gate_logits", "2", xb + E * M * 2 + T * E * 4, lambda: ops.gate_logits(x, wg, torch.float32))
     add("gate_route (gate + routing)", "2", xb + E * M * 2 + plane, lambda: ops.gate_route(x, wg, k))
     sc = torch.softmax(ops.gate_logits(x, wg, torch.float32), 1)
     add("route_topk (scores in)", "2", T * E * 4 + plane, lambda: ops.route_topk(sc, k))
-    add("dispatch_fwd", "2", xb + db + plane, lambda: ops.dispatch_fwd(x, idx, loc, None, E, C))
+    add("dispatch_fwd", "2", kept(loc, C) * M * 2 + db + plane, lambda: ops.dispatch_fwd(x, idx, loc, None, E, C))
     d = ops.dispatch_fwd(x, idx, loc, None, E, C)
     add("combine_fwd", "2", live * M * 2 + xb + plane, lambda: ops.combine_fwd(d, idx, loc, gates, T, C))
     add("bwd_gate", "2", live * M * 2 + xb + plane, lambda: ops.bwd_gate(x, d, idx, loc, C))
@@ -223,7 +230,7 @@ def kernel_table(only=None):
     r1 = ops.gate_route(x1, w1, 2)
     i1, l1, g1 = list(r1["indices"]), list(r1["locations"]), list(r1["gates"])
     add("gate_route (gate + routing)", "1", T1 * M1 * 4 + T1 * 24, lambda: ops.gate_route(x1, w1, 2))
-    add("dispatch_fwd", "1", T1 * M1 * 4 + E1 * C1 * M1 * 4, lambda: ops.dispatch_fwd(x1, i1, l1, None, E1, C1))
+    add("dispatch_fwd", "1", kept(l1, C1) * M1 * 4 + E1 * C1 * M1 * 4, lambda: ops.dispatch_fwd(x1, i1, l1, None, E1, C1))
     d1 = ops.dispatch_fwd(x1, i1, l1, None, E1, C1)
     add("combine_fwd", "1", 3 * T1 * M1 * 4, lambda: ops.combine_fwd(d1, i1, l1, g1, T1, C1))
     del d1
@@ -241,7 +248,7 @@ def kernel_table(only=None):
         lambda: ops.forward_int8(x3, w3, 1, C3, logit_bias=bias))
     r3 = ops.gate_route(x3, w3, 1, logit_bias=bias)
     i3, l3 = list(r3["indices"]), list(r3["locations"])
-    add("dispatch_fwd", "3", T3 * M3 * 2 + E3 * C3 * M3 * 2 + T3 * 12, lambda: ops.dispatch_fwd(x3, i3, l3, None, E3, C3))
+    add("dispatch_fwd", "3", kept(l3, C3) * M3 * 2 + E3 * C3 * M3 * 2 + T3 * 12, lambda: ops.dispatch_fwd(x3, i3, l3, None, E3, C3))
     lg = ops.gate_logits(x3, w3, torch.float32)
     add("route_topk (logits in)", "3", T3 * E3 * 4 + T3 * 12, lambda: ops.route_topk(lg, 1, is_logits=True, logit_bias=bias))
     mask = (torch.rand(T3, E3, device=dev) < 0.1).to(torch.int32)
@@ -265,7 +272,7 @@ def kernel_table(only=None):
     zs = ops.dispatch_zfp(x5, i5, l5, None, E5, C5)
     g5 = [t.float() for t in r5["gates"]]
     d5 = ops.zfp_decompress(zs, M5, E5 * C5, 2)
-    add("dispatch_fwd", "5", T5 * M5 * 4 + E5 * C5 * M5 * 4, lambda: ops.dispatch_fwd(x5, i5, l5, None, E5, C5), iters=5)
+    add("dispatch_fwd", "5", kept(l5, C5) * M5 * 4 + E5 * C5 * M5 * 4, lambda: ops.dispatch_fwd(x5, i5, l5, None, E5, C5), iters=5)
     add("combine_fwd", "5", 3 * T5 * M5 * 4, lambda: ops.combine_fwd(d5, i5, l5, g5, T5, C5), iters=5)
     add("combine_zfp (fused)", "5", E5 * C5 * M5 + T5 * M5 * 4,
         lambda: ops.combine_zfp(zs, i5, l5, g5, T5, E5, C5, M5), iters=5)

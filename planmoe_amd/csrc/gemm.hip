@@ -230,17 +230,21 @@ __global__ __launch_bounds__(256, 1) void gemm_nt_bf16_dma_kernel(const GemmArgs
         bo[i] = (uint32_t)min(n0 + row, p.N - 1) * (uint32_t)p.ldb * 2u + chunk * 16;
     }
     const int KT = p.K / DMA_BK;
-    auto load_stage = [&](int kt) {
+    // a quarter of the loads of tile kt (a tile's loads go out in four parts, one before each k-step
+    // of the tile before: 16 loads in a row hold the wave up at the address unit, and arrive in one burst)
+    auto load_part = [&](int kt, int part) {
         // past the end: the last tile once more, into a buffer nobody reads again (keeps the number
         // of loads in flight the same in every round, which the waits below count on)
         const int k = min(kt, KT - 1);
         const uint8_t *ga = A + (int64_t)k * (DMA_BK * 2), *gb = B + (int64_t)k * (DMA_BK * 2);
         const uint32_t sa = lds0 + (kt % DMA_STAGES) * DMA_STAGE + wave_u * (64 * DMA_ROW), sb = sa + DMA_OPERAND;
+        constexpr int PER = DMA_LOADS / 4;
 #pragma unroll
-        for (int i = 0; i < DMA_LOADS; ++i) gemm_dma16(ga, ao[i], sa + i * 1024);
+        for (int i = PER * part; i < PER * part + PER; ++i) gemm_dma16(ga, ao[i], sa + i * 1024);
 #pragma unroll
-        for (int i = 0; i < DMA_LOADS; ++i) gemm_dma16(gb, bo[i], sb + i * 1024);
+        for (int i = PER * part; i < PER * part + PER; ++i) gemm_dma16(gb, bo[i], sb + i * 1024);
     };
+    static_assert(DMA_LOADS % 4 == 0, "a tile's loads go out in four parts");
 
     f32x16 acc[4][4];
 #pragma unroll
@@ -269,24 +273,28 @@ __global__ __launch_bounds__(256, 1) void gemm_nt_bf16_dma_kernel(const GemmArgs
     };
 #undef PM_MMA
 
-    load_stage(0);
+#pragma unroll
+    for (int part = 0; part < 4; ++part) load_part(0, part);
     for (int kt = 0; kt < KT; ++kt) {
         // this wave's loads of tile kt are in; behind the barrier everybody's are, and everybody is
         // done reading tile kt - 1, whose buffer the loads of tile kt + 1 then fill during this tile's MFMAs
         asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-        load_stage(kt + 1);
         const uint8_t *st = lds + (kt % DMA_STAGES) * DMA_STAGE;
         Frags g0, g1;
         read_frags(g0, st, 0);
         read_frags(g1, st, 1);
+        load_part(kt + 1, 0);
         mma_step(g0);
         __builtin_amdgcn_sched_barrier(0);
         read_frags(g0, st, 2);
+        load_part(kt + 1, 1);
         mma_step(g1);
         __builtin_amdgcn_sched_barrier(0);
         read_frags(g1, st, 3);
+        load_part(kt + 1, 2);
         mma_step(g0);
         __builtin_amdgcn_sched_barrier(0);
+        load_part(kt + 1, 3);
         mma_step(g1);
     }
     // nothing may still be on its way into LDS when the quadrants overwrite it

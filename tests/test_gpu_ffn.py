@@ -114,6 +114,38 @@ def test_fc1_affine_against_the_oracle(E, C, M, H, with_bias):
     assert float((got[0, 0] - (fb[0].float() if with_bias else 0.0)).abs().max()) == 0.0     # the empty slot: bias only
 
 
+def test_fc1_affine_gap_where_offsets_dwarf_ranges_and_weight_columns_cancel():
+    """The case that separates the two forms: rows 100 + 2 N(0, 1) (bf16 spacing at 100 is 0.5, a code
+    step 16 / 255) times weight columns that sum to zero, so the offset cancels and only the variation is
+    left in the result.  The exact form stays at decompress + GEMM.  The affine form multiplies
+    code / 255 * scale + bias without the decompressor's three roundings, so it differs by up to their
+    share, 2^-8 of sum |w| |x| -- a bound in terms of the operands, not of the result: here more than a
+    fifth of the outputs differ by over rtol 1e-2 of the result itself, which is why the layer takes
+    the exact form unless told otherwise."""
+    from planmoe_amd import ops
+    E, C, M, H = 2, 128, 512, 128
+    g = torch.Generator().manual_seed(7)
+    x = (100.0 + 2.0 * torch.randn(E, C, M, generator=g)).bfloat16()
+    half = (torch.randn(E, H, M // 2, generator=g) * M ** -0.5).bfloat16()
+    w = torch.cat([half, -half], dim=2).contiguous()                   # every column of every expert sums to 0
+    codes, bias, scale = ops.int8_compress(x.to(DEV))
+    wd = w.to(DEV)
+    exact = ops.ffn_fc1_int8(codes, bias, scale, wd, None).float().cpu().double()
+    affine = ops.ffn_fc1_int8_affine(codes, bias, scale, wd, ops.ffn_weight_colsum(wd), None).float().cpu().double()
+    rc, rb, rs = oracle.int8_compress(bf16_bits(x))
+    assert np.array_equal(codes.cpu().numpy(), rc)
+    dec = from_bf16_bits(oracle.int8_decompress(rc, rb, rs)).double()
+    ref = torch.einsum("ecm,ehm->ech", dec, w.double())
+    mag = torch.einsum("ecm,ehm->ech", dec.abs(), w.double().abs())
+    # exact form: the decompressor's values, fp32 sums (512 terms: 2^-15 mag at worst) and one bf16 rounding
+    assert ((exact - ref).abs() <= 2.0 ** -8 * ref.abs() + 2.0 ** -14 * mag).all()
+    # affine form: within the skipped roundings of the exact one ...
+    gap = (affine - exact).abs()
+    assert (gap <= 1.05 * 2.0 ** -8 * mag + 2.0 ** -7 * ref.abs()).all()
+    # ... and that is not "an ulp of the result" here
+    assert float((gap > 1e-2 * ref.abs()).double().mean()) > 0.2
+
+
 def test_fc1_affine_config2_shape():
     from planmoe_amd import ops
     E, C, M, H = 8, 5120, 4096, 4096
