@@ -45,6 +45,7 @@ struct GemmArgs {
     int M, N, K;                  // rows of A, rows of B, reduction length
     int lda, ldb, ldc;            // elements between rows
     int64_t sA, sB, sC, sBias;    // elements between batches
+    int batches;
 };
 
 template <int ACT>
@@ -214,7 +215,21 @@ __global__ __launch_bounds__(256, 1) void gemm_nt_bf16_dma_kernel(const GemmArgs
     extern __shared__ __align__(16) uint8_t lds[];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int wm = wave >> 1, wn = wave & 1;
-    const int e = blockIdx.z, m0 = blockIdx.y * GEMM_BM, n0 = blockIdx.x * GEMM_BN;
+    // Work-groups go to the 8 XCDs in turn, each XCD with an L2 of its own: XCD j (work-groups j, j + 8,
+    // ...) takes the j-th eighth of the tiles, in the order batch, panel of 8 tile columns, tile row,
+    // column of the panel, so that the 32 tiles it works on at a time are a 4 x 8 block of one batch
+    // (12 operand tiles for 32 products; measured at 8 x 5120 x 4096 x 4096: L2 hits 69 -> 80 %, HBM reads
+    // 3.3 -> 2.0 GB per launch).  The grid is one-dimensional, a multiple of 8; the surplus returns.
+    const int tiles_m = (p.M + GEMM_BM - 1) / GEMM_BM, tiles_n = (p.N + GEMM_BN - 1) / GEMM_BN;
+    const int64_t tiles = (int64_t)tiles_m * tiles_n * p.batches, per_xcd = (tiles + 7) / 8;
+    const int64_t tile = (int64_t)(blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile >= tiles) return;
+    const int e = (int)(tile / (tiles_m * tiles_n));
+    int in_batch = (int)(tile - (int64_t)e * tiles_m * tiles_n);
+    const int panel = in_batch / (tiles_m * 8);
+    in_batch -= panel * tiles_m * 8;
+    const int panel_width = min(8, tiles_n - panel * 8);
+    const int m0 = (in_batch / panel_width) * GEMM_BM, n0 = (panel * 8 + in_batch % panel_width) * GEMM_BN;
     const uint8_t *A = reinterpret_cast<const uint8_t *>(p.A + (int64_t)e * p.sA);
     const uint8_t *B = reinterpret_cast<const uint8_t *>(p.B + (int64_t)e * p.sB);
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds;
@@ -380,7 +395,7 @@ extern "C" int planmoe_gemm_nt_bf16(const void *a, const void *b, const void *bi
     PM_REQUIRE((int64_t)m * lda * 2 < ((int64_t)1 << 32) && (int64_t)n * ldb * 2 < ((int64_t)1 << 32),
                "planmoe_gemm_nt_bf16: an operand of one batch must stay under 4 GiB");
     GemmArgs p{(const uint16_t *)a, (const uint16_t *)b, (const uint16_t *)bias, (uint16_t *)c, m, n, k, lda, ldb, ldc,
-               batch_stride_a, batch_stride_b, batch_stride_c, (int64_t)n};
+               batch_stride_a, batch_stride_b, batch_stride_c, (int64_t)n, batches};
     const void *fn = activation == 0 ? (const void *)gemm_nt_bf16_kernel<0> : (const void *)gemm_nt_bf16_kernel<1>;
     PM_REQUIRE(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS) == hipSuccess,
                "planmoe_gemm_nt_bf16: the kernel needs %d bytes of LDS", GEMM_LDS);
@@ -390,8 +405,11 @@ extern "C" int planmoe_gemm_nt_bf16(const void *a, const void *b, const void *bi
         const void *fd = activation == 0 ? (const void *)gemm_nt_bf16_dma_kernel<0> : (const void *)gemm_nt_bf16_dma_kernel<1>;
         PM_REQUIRE(hipFuncSetAttribute(fd, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS) == hipSuccess,
                    "planmoe_gemm_nt_bf16: the kernel needs %d bytes of LDS", GEMM_LDS);
-        if (activation == 0) gemm_nt_bf16_dma_kernel<0><<<grid, 256, GEMM_LDS, (hipStream_t)stream>>>(p);
-        else gemm_nt_bf16_dma_kernel<1><<<grid, 256, GEMM_LDS, (hipStream_t)stream>>>(p);
+        const int64_t per_xcd = (tm * tn * batches + 7) / 8;
+        PM_REQUIRE(per_xcd * 8 < ((int64_t)1 << 31), "planmoe_gemm_nt_bf16: too many tiles");
+        const dim3 tiles((unsigned)(per_xcd * 8));
+        if (activation == 0) gemm_nt_bf16_dma_kernel<0><<<tiles, 256, GEMM_LDS, (hipStream_t)stream>>>(p);
+        else gemm_nt_bf16_dma_kernel<1><<<tiles, 256, GEMM_LDS, (hipStream_t)stream>>>(p);
         PM_LAUNCH_CHECK("planmoe_gemm_nt_bf16");
         return 0;
     }
