@@ -242,6 +242,7 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
         constexpr int LPT = CAP, TPP = WAVE / LPT;
         const int el = lane % LPT, tk = lane / LPT;
         auto token_reduce = [&](auto v, auto op) { return row_allreduce<LPT>(v, op); };
+        const float lbias = (logit_bias && el < experts) ? logit_bias[el] : 0.f;    // (one round trip, not one per pass)
 #pragma unroll
         for (int p = 0; p < RPASSES; ++p) {
             const int tok = min((p * FS_WAVES + w) * TPP + tk, TOK - 1), t = t0 + tok;
@@ -250,7 +251,7 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
             if (el < experts) {
                 v = S::round(s_logit[tok][el]);
                 if (logits_out && valid) S::store(logits_out, (int64_t)t * experts + el, v);
-                if (logit_bias) v = S::round(v + logit_bias[el]);
+                if (logit_bias) v = S::round(v + lbias);
             }
             const float mxl = token_reduce(v, [](float a, float c) { return fmaxf(a, c); });
             float sc = el < experts ? expf(v - mxl) : 0.f;

@@ -91,6 +91,17 @@ def test_many_blocks_and_scan_chunks():
     check(x)
 
 
+def test_one_workspace_call_after_call():
+    """What a call leaves in the workspace (class bytes, chunk totals) must not reach into the next:
+    a long input, then shorter and different ones, on one workspace."""
+    rng = np.random.default_rng(9)
+    big = rng.integers(0, 3, size=5000 * 512).astype(np.float32)
+    ws = torch.empty((int(_lib.lib.planmoe_lz_workspace_bytes(big.nbytes)),), dtype=torch.uint8, device=DEV)
+    for x in (big, rng.standard_normal(700 * 512).astype(np.float32), np.zeros(2000 * 512, np.float32), big[::-1].copy()):
+        got = ops.lz_compress(torch.from_numpy(x).to(DEV), workspace=ws)
+        same_streams(got, oracle.lz_compress(x))
+
+
 def test_config5_full_size():
     """The [16, 8192, 1024] fp32 buffer of config 5 (512 MiB, 262 144 blocks): a quarter of the
     capacity slots empty, some rows thinned out like an activation after a ReLU, the rest dense.
