@@ -626,8 +626,25 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
     tokens_per_s = T / (wall / args.steps)
+    note = None
     if int(plan.gave_up) != 0:
-        sys.exit("bench.py: a work-group of the one-launch kernel gave up waiting for the others")
+        # what the layer does then: the pass again through the two launches (measured as the step, and said so)
+        note = "a work-group of the one-launch kernel gave up waiting for the others: the step is planmoe_forward_int8 (two launches)"
+        print("bench.py: " + note, file=sys.stderr)
+        plan = plan2
+        for _ in range(args.warmup):
+            chain()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            chain()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        ms_per_step = wall / args.steps * 1e3
+        tokens_per_s = T / (wall / args.steps)
+
+    # algorithmic bytes: every input read once, every output written once
+    chain_bytes = T * M * 2 + R * M + R * 2 * 2 + T * k * 12 + E * M * 2
 
     # device times (HIP events on the stream the kernels are launched on): the one-launch chain, the
     # two-launch chain and its two launches on their own
@@ -642,11 +659,19 @@ def main():
     # the measuring stick: the chain's grid, loads, exchange and stores without its arithmetic (the
     # floor under this kernel's structure), and the same with nobody waiting at the exchange (the
     # floor under any arrangement of these loads and stores: what the dependency costs is the difference)
-    ceiling = ops.ForwardCeiling(xd, E, k, C)
-    ceil_ev = {mode: event_time_us(lambda mode=mode: ceiling.run(mode), 30, 5) for mode in (0, 1, 2)}
+    # (a side measurement: whatever goes wrong with it leaves its fields empty, not the line unprinted)
+    ceil_ev = {0: (None,), 1: (None,), 2: (None,)}
+    try:
+        ceiling = ops.ForwardCeiling(xd, E, k, C)
+        got = {mode: event_time_us(lambda mode=mode: ceiling.run(mode), 30, 5) for mode in (0, 1, 2)}
+        if int(ceiling.gave_up) == 0:
+            ceil_ev = got
+        else:
+            print("bench.py: a work-group of the ceiling kernel gave up waiting for the others", file=sys.stderr)
+    except Exception as ex:                                          # noqa: BLE001
+        print("bench.py: the ceiling kernel was not measured: %s" % ex, file=sys.stderr)
     chain_ev_again = event_time_us(chain, 30, 5)
-    if int(ceiling.gave_up) != 0:
-        sys.exit("bench.py: a work-group of the ceiling kernel gave up waiting for the others")
+    frac_of_peak = lambda us: None if us is None else chain_bytes / us / 1e3 / HBM_PEAK_GBS
 
     # the chains with none of their operands in the L2s or the 256 MB memory-side cache: a reduction
     # over 1 GiB of other data before every call, one event pair per call, median of 9
@@ -666,8 +691,6 @@ def main():
     cold_us, cold2_us = cold(chain), cold(plan2.run)
     del scrub
 
-    # algorithmic bytes: every input read once, every output written once
-    chain_bytes = T * M * 2 + R * M + R * 2 * 2 + T * k * 12 + E * M * 2
     achieved = chain_bytes / chain_ev[0] / 1e3                     # GB/s, hot (back-to-back calls)
     traffic = profile_traffic_bytes()
 
@@ -683,16 +706,17 @@ def main():
         # same buffers, cold = after a pass over 1 GiB of other data
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "forward_single_kernel (the whole chain: planmoe_forward_int8_single, one launch)",
+                     "kernel": "forward_single_kernel (the whole chain: planmoe_forward_int8_single, one launch)"
+                               if note is None else "gate_route_kernel + dispatch_int8_routed_kernel (planmoe_forward_int8)",
                      "algorithmic_bytes": chain_bytes, "avg_us": chain_ev[0], "min_us": chain_ev[2],
                      "cold_us": cold_us, "cold_achieved": chain_bytes / cold_us / 1e3,
                      "cold_frac": chain_bytes / cold_us / 1e3 / HBM_PEAK_GBS,
                      "target_frac": 0.70, "target_met": achieved / HBM_PEAK_GBS >= 0.70,
                      # planmoe_forward_int8_single_ceiling in the same run: same grid, loads, exchange and
                      # stores, no arithmetic
-                     "ceiling_us": ceil_ev[0][0], "ceiling_frac": chain_bytes / ceil_ev[0][0] / 1e3 / HBM_PEAK_GBS,
+                     "ceiling_us": ceil_ev[0][0], "ceiling_frac": frac_of_peak(ceil_ev[0][0]),
                      "ceiling_no_exchange_us": ceil_ev[1][0],
-                     "ceiling_no_exchange_frac": chain_bytes / ceil_ev[1][0] / 1e3 / HBM_PEAK_GBS,
+                     "ceiling_no_exchange_frac": frac_of_peak(ceil_ev[1][0]),
                      "ceiling_two_halves_us": ceil_ev[2][0],
                      "avg_us_after_ceilings": chain_ev_again[0]},
         "two_launch_chain": {"entry_point": "planmoe_forward_int8 (x read by both launches)",
@@ -702,6 +726,8 @@ def main():
                              "device_us_cold_caches": cold2_us,
                              "stage_us_avg": {n: v[0] for n, v in stages.items()}},
     }
+    if note is not None:
+        out["note"] = note
     if args.cpu_sample > 0:
         n = min(args.cpu_sample, T)
         v, dt, reps = cpu_baseline(n, M, E, k, cf, x, wg, args.cpu_seconds)
