@@ -27,7 +27,10 @@ def _check(got, a, b, bias, relu):
 @pytest.mark.parametrize("B,m,n,k,with_bias,relu,shared_b", [
     (2, 200, 136, 72, True, False, False), (3, 300, 264, 128, False, False, False), (1, 1, 8, 8, True, True, False),
     (2, 513, 520, 200, True, True, False), (1, 256, 256, 64, False, False, False), (4, 130, 24, 1032, True, False, True),
-    (2, 700, 512, 640, False, True, False)])
+    (2, 700, 512, 640, False, True, False),
+    # more than 8 tile columns, not a multiple of 8, tile count not a multiple of 8: panels of 8 + 2 and 8 + 1
+    # columns, an XCD's stretch of the tiles crossing batches, surplus work-groups
+    (3, 700, 2312, 64, True, True, False), (5, 520, 2056, 128, False, False, True)])
 def test_gemm_against_an_fp64_product(B, m, n, k, with_bias, relu, shared_b):
     from planmoe_amd import ops
     print("case", B, m, n, k, with_bias, relu, shared_b, flush=True)
