@@ -214,11 +214,20 @@ def kernel_table(only=None):
     add("ffn_fc1_int8_affine (GEMM on codes)", "2", R * M + R * 4 + E * Hf * M * 2 + R * Hf * 2,
         lambda: ops.ffn_fc1_int8_affine(codes.view(E, C, M), b.view(E, C, 1), s_.view(E, C, 1), wk, wcs, fb, out=fout), iters=5)
     ffn_flops = 2.0 * R * M * Hf
-    # the experts' GEMMs proper (planmoe_gemm_nt_bf16): the first one with bias + relu on the decompressed
-    # rows, and the transpose that brings an operand into the kernel's form
+    # the experts' GEMMs proper: the first one with bias + relu on the decompressed rows (planmoe_gemm_nt_bf16,
+    # second operand k-major), and the transpose that brings an operand into that form
     xin = torch.randn(E, C, M, generator=g).bfloat16().to(dev)
     add("ffn_gemm_nt_bf16 (x @ W + b, relu)", "2", R * M * 2 + E * Hf * M * 2 + R * Hf * 2,
         lambda: ops.gemm_nt_bf16(xin, wk, fb, relu=True, out=fout), iters=5)
+    # the same product with the weight as the experts store it ([E, in, out]: no transposed copy), and the
+    # weight gradient x^T dy with both operands as they lie (Hf == M here, so the flops are the same)
+    wst = wk.transpose(1, 2).contiguous()
+    add("ffn_gemm_nn_bf16 (x @ W + b, relu)", "2", R * M * 2 + E * Hf * M * 2 + R * Hf * 2,
+        lambda: ops.gemm_nn_bf16(xin, wst, fb, relu=True, out=fout), iters=5)
+    dwout = torch.empty(E, M, Hf, dtype=torch.bfloat16, device=dev)
+    add("ffn_gemm_tn_bf16 (dW = x^T @ dy)", "2", R * M * 2 + R * Hf * 2 + E * M * Hf * 2,
+        lambda: ops.gemm_tn_bf16(xin, fout, out=dwout), iters=5)
+    del wst, dwout
     add("ffn_transpose_bf16 [8, 5120, 4096]", "2", 2 * R * M * 2, lambda: ops.transpose_bf16(xin, 64), iters=5)
     del d, dc, codes, plan, plan1, wk, fout, xin
 

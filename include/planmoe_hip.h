@@ -382,6 +382,24 @@ int planmoe_gemm_nt_bf16(const void *a, const void *b, const void *bias, int act
                          int m, int n, int k, int lda, int ldb, int ldc, int64_t batch_stride_a,
                          int64_t batch_stride_b, int64_t batch_stride_c, void *c, void *stream);
 
+/* c[e] = act(bf16(bf16(a[e] b[e]) + bias[e])) for bf16 a [batches, m, k] and b [batches, k, n] with n the
+ * fast index -- a weight as experts/ffn.py:33-56 stores it, [E, in, out]: the matmul + add of
+ * ffn.py:77-79 with no transposed copy of the weight.  k a multiple of 64; n and the pitches multiples
+ * of 8; bias, activation, roundings and the order of the sums as planmoe_gemm_nt_bf16. */
+int planmoe_gemm_nn_bf16(const void *a, const void *b, const void *bias, int activation, int batches,
+                         int m, int n, int k, int lda, int ldb, int ldc, int64_t batch_stride_a,
+                         int64_t batch_stride_b, int64_t batch_stride_c, void *c, void *stream);
+
+/* c[e] = a[e]^T b[e] for bf16 a [batches, k, m], b [batches, k, n] (row pitches lda >= m, ldb >= n,
+ * the reduction index the slow one) -> c [batches, m, n] bf16, fp32 sums, one rounding: the weight
+ * gradient matmul(x.transpose(1, 2), dy) of the autograd of experts/ffn.py:77-79 with both operands
+ * as they lie in memory (no transposed copies; the fragments are transposed on their way out of
+ * LDS).  k a multiple of 64; m, n and the pitches multiples of 8; sums in the order of
+ * planmoe_gemm_nt_bf16 on transposed copies. */
+int planmoe_gemm_tn_bf16(const void *a, const void *b, int batches, int m, int n, int k, int lda, int ldb,
+                         int ldc, int64_t batch_stride_a, int64_t batch_stride_b, int64_t batch_stride_c,
+                         void *c, void *stream);
+
 /* out[e][j][i] = in[e][i][j] for bf16 matrices [batches, rows, cols] -> [batches, cols, rows_out];
  * rows_out >= rows, the columns rows .. rows_out - 1 of out are zero (padding of a reduction index).
  * cols and rows_out multiples of 8.  Stands for the .transpose(...).contiguous() the GEMM form

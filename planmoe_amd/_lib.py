@@ -71,6 +71,10 @@ SIGNATURES = {
                                                     c_void_p, c_void_p, c_size_t, c_int, c_int, c_void_p, c_void_p]),
     "planmoe_gemm_nt_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_int64, c_int64, c_int64, c_void_p, c_void_p]),
+    "planmoe_gemm_nn_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                     c_int64, c_int64, c_int64, c_void_p, c_void_p]),
+    "planmoe_gemm_tn_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
+                                     c_int64, c_int64, c_void_p, c_void_p]),
     "planmoe_transpose_bf16": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "planmoe_forward_int8_static": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_int,
                                             c_int, c_int, c_void_p, c_void_p, c_void_p, c_int64, c_void_p,

@@ -1,16 +1,19 @@
 // Batched bf16 GEMM of the expert FFN, written for gfx950's matrix cores, and the transpose that
-// brings an operand into the form it wants.
+// brings an operand into k-major form where the direct forms do not apply.
 //
 //   C[e][m][n] = act( bf16( bf16( sum_k A[e][m][k] * B[e][n][k] ) + bias[e][n] ) )
 //
-// Both operands are taken with k running fastest ("NT"): a matrix-core operand is eight
-// consecutive k per lane.  The reference's experts (experts/ffn.py:63-82) compute
-// x @ fc1_w -> activation -> @ fc2_w with weights stored [experts, in, out]; the four GEMM shapes
-// of its forward and backward pass map onto this one kernel as
-//   forward   y  = x  @ W          A = x  [rows, in],   B = W^T  [out, in]    (transposed copy of W)
-//   backward  dx = dy @ W^T        A = dy [rows, out],  B = W    [in, out]    (W as stored)
-//             dW = x^T @ dy        A = x^T [in, rows],  B = dy^T [out, rows]  (transposed copies, k padded)
-// so the only extra passes are transposes, which run at the speed of the memory.
+// A matrix-core operand is eight consecutive k per lane.  An operand stored with k running fastest
+// ("N" for A, "T" for B) gives that as one 16-byte read of LDS; an operand stored the other way round
+// is read through LDS reads that transpose (ds_read_b64_tr_b16), so the direct-to-LDS kernel below
+// takes either operand either way.  The reference's experts (experts/ffn.py:63-82) compute
+// x @ fc1_w -> activation -> @ fc2_w with weights stored [experts, in, out]; the GEMM shapes of its
+// forward and backward pass are
+//   forward   y  = x  @ W          A = x  [rows, in],   B = W  [in, out]      planmoe_gemm_nn_bf16
+//   backward  dx = dy @ W^T        A = dy [rows, out],  B = W  [in, out]      planmoe_gemm_nt_bf16
+//             dW = x^T @ dy        A = x  [rows, in],   B = dy [rows, out]    planmoe_gemm_tn_bf16
+// all with the operands as they lie in memory when the reduction length is a multiple of 64; for other
+// lengths planmoe_gemm_nt_bf16 serves on transposed copies (the register-staged kernel, any k % 8 == 0).
 //
 // Tile 256 x 256 x 64 per work-group of four waves; a wave owns 128 x 128 as 4 x 4 tiles of
 // v_mfma_f32_32x32x16_bf16 (256 accumulator registers, so one wave per SIMD: latency is covered by
@@ -209,7 +212,27 @@ __device__ __forceinline__ void gemm_dma16(const void *gbase, uint32_t voff, uin
 // where chunk c of row r lies in its row of 8 units
 __device__ __forceinline__ int dma_unit(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
 
-template <int ACT>
+// TA / TB = true: the operand is stored the other way round, a[e][k][m] / b[e][k][n] (both: c = a^T b, the
+// weight gradient x^T dy; only b: c = a b with a weight as experts/ffn.py stores it; no transposed copies
+// either way): a k-tile of such an operand is 64 rows of 512 bytes,
+// a load instruction fills two of them, chunk c of row k lies at unit c ^ (k & 3) << 2, and a fragment
+// comes out of LDS through ds_read_b64_tr_b16, which hands lane i of every 16 lanes element i % 4 of
+// the 8 bytes that lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12 point at: with lane s pointing at row
+// s / 4, columns 4 (s % 4) .. + 3 of a 4 x 16 patch, lane i receives 4 consecutive k of column i --
+// the matrix cores' operand layout.  Two such reads make the 8 k of a step; the 4 rows of a patch lie
+// in different quarters of the 256 bytes the LDS serves per clock.  Needs k % 64 == 0.
+typedef short gemm_s16x4 __attribute__((ext_vector_type(4)));
+typedef short gemm_s16x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ gemm_bf16x8 gemm_read_tr(const uint8_t *lo, const uint8_t *hi)
+{
+    typedef gemm_s16x4 __attribute__((address_space(3))) *lds_s16x4;
+    const gemm_s16x4 x = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)lo);
+    const gemm_s16x4 y = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4)hi);
+    const gemm_s16x8 v = __builtin_shufflevector(x, y, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(gemm_bf16x8, v);
+}
+
+template <int ACT, bool TA = false, bool TB = false>
 __global__ __launch_bounds__(256, 1) void gemm_nt_bf16_dma_kernel(const GemmArgs p)
 {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -240,9 +263,14 @@ __global__ __launch_bounds__(256, 1) void gemm_nt_bf16_dma_kernel(const GemmArgs
     uint32_t ao[DMA_LOADS], bo[DMA_LOADS];
 #pragma unroll
     for (int i = 0; i < DMA_LOADS; ++i) {
+        // an operand with the reduction index slow: wave w brings in rows (k) 16 w .. 16 w + 15 of its
+        // tile, 8 loads of 2 rows of 512 bytes
+        const int trow = 16 * wave + 2 * i + (lane >> 5), tchunk = (lane & 31) ^ ((trow & 3) << 2);
         const int row = 64 * wave + 8 * i + (lane >> 3), chunk = dma_unit(row, lane & 7);
-        ao[i] = (uint32_t)min(m0 + row, p.M - 1) * (uint32_t)p.lda * 2u + chunk * 16;
-        bo[i] = (uint32_t)min(n0 + row, p.N - 1) * (uint32_t)p.ldb * 2u + chunk * 16;
+        ao[i] = TA ? (uint32_t)trow * (uint32_t)p.lda * 2u + (uint32_t)min(m0 + tchunk * 8, p.M - 8) * 2u
+                   : (uint32_t)min(m0 + row, p.M - 1) * (uint32_t)p.lda * 2u + chunk * 16;
+        bo[i] = TB ? (uint32_t)trow * (uint32_t)p.ldb * 2u + (uint32_t)min(n0 + tchunk * 8, p.N - 8) * 2u
+                   : (uint32_t)min(n0 + row, p.N - 1) * (uint32_t)p.ldb * 2u + chunk * 16;
     }
     const int KT = p.K / DMA_BK;
     // a quarter of the loads of tile kt (a tile's loads go out in four parts, one before each k-step
@@ -251,8 +279,9 @@ __global__ __launch_bounds__(256, 1) void gemm_nt_bf16_dma_kernel(const GemmArgs
         // past the end: the last tile once more, into a buffer nobody reads again (keeps the number
         // of loads in flight the same in every round, which the waits below count on)
         const int k = min(kt, KT - 1);
-        const uint8_t *ga = A + (int64_t)k * (DMA_BK * 2), *gb = B + (int64_t)k * (DMA_BK * 2);
-        const uint32_t sa = lds0 + (kt % DMA_STAGES) * DMA_STAGE + wave_u * (64 * DMA_ROW), sb = sa + DMA_OPERAND;
+        const uint8_t *ga = A + (TA ? (int64_t)k * DMA_BK * p.lda * 2 : (int64_t)k * (DMA_BK * 2));
+        const uint8_t *gb = B + (TB ? (int64_t)k * DMA_BK * p.ldb * 2 : (int64_t)k * (DMA_BK * 2));
+        const uint32_t sa = lds0 + (kt % DMA_STAGES) * DMA_STAGE + wave_u * (64 * DMA_ROW), sb = sa + DMA_OPERAND;   // (a wave's share is 8 KB either way)
         constexpr int PER = DMA_LOADS / 4;
 #pragma unroll
         for (int i = PER * part; i < PER * part + PER; ++i) gemm_dma16(ga, ao[i], sa + i * 1024);
@@ -272,12 +301,32 @@ __global__ __launch_bounds__(256, 1) void gemm_nt_bf16_dma_kernel(const GemmArgs
     // fragment of a step: lane l holds row l % 32, chunk 2 ks + l / 32 of its rows
     const int fr = lane & 31, fc = lane >> 5;
     struct Frags { gemm_bf16x8 a0, a1, a2, a3, b0, b1, b2, b3; };
+    // an operand with the reduction index slow: lane = (group g of 16 lanes, s): row 8 (g / 2) + s / 4 of the step's 16, bytes 8 (s % 4) of the
+    // 32 that columns 16 (g % 2) .. + 15 of the fragment take; unit of the row swizzled by s / 4 = row & 3
+    const int tg = lane >> 4, ts = lane & 15;
+    const int t_row = (8 * (tg >> 1) + (ts >> 2)) * 512;
+    int t_col[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t_col[i] = (4 * (i ^ (ts >> 2)) + 2 * (tg & 1) + ((ts & 3) >> 1)) * 16 + 8 * (ts & 1);
     auto read_frags = [&](Frags &f, const uint8_t *st, int ks) {
-        const uint8_t *sa = st + (wm * 128 + fr) * DMA_ROW, *sb = st + DMA_OPERAND + (wn * 128 + fr) * DMA_ROW;
+#define PM_FT(base, i) gemm_read_tr(base + t_col[i], base + t_col[i] + 4 * 512)
 #define PM_FR(base, i) *reinterpret_cast<const gemm_bf16x8 *>(base + (i) * 32 * DMA_ROW + dma_unit(32 * (i) + fr, 2 * ks + fc) * 16)
-        f.a0 = PM_FR(sa, 0); f.a1 = PM_FR(sa, 1); f.a2 = PM_FR(sa, 2); f.a3 = PM_FR(sa, 3);
-        f.b0 = PM_FR(sb, 0); f.b1 = PM_FR(sb, 1); f.b2 = PM_FR(sb, 2); f.b3 = PM_FR(sb, 3);
+        if constexpr (TA) {
+            const uint8_t *sa = st + t_row + ks * (16 * 512) + wm * 256;
+            f.a0 = PM_FT(sa, 0); f.a1 = PM_FT(sa, 1); f.a2 = PM_FT(sa, 2); f.a3 = PM_FT(sa, 3);
+        } else {
+            const uint8_t *sa = st + (wm * 128 + fr) * DMA_ROW;
+            f.a0 = PM_FR(sa, 0); f.a1 = PM_FR(sa, 1); f.a2 = PM_FR(sa, 2); f.a3 = PM_FR(sa, 3);
+        }
+        if constexpr (TB) {
+            const uint8_t *sb = st + DMA_OPERAND + t_row + ks * (16 * 512) + wn * 256;
+            f.b0 = PM_FT(sb, 0); f.b1 = PM_FT(sb, 1); f.b2 = PM_FT(sb, 2); f.b3 = PM_FT(sb, 3);
+        } else {
+            const uint8_t *sb = st + DMA_OPERAND + (wn * 128 + fr) * DMA_ROW;
+            f.b0 = PM_FR(sb, 0); f.b1 = PM_FR(sb, 1); f.b2 = PM_FR(sb, 2); f.b3 = PM_FR(sb, 3);
+        }
 #undef PM_FR
+#undef PM_FT
     };
 #define PM_MMA(i, j, x, y) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x, y, acc[i][j], 0, 0, 0)
     auto mma_step = [&](const Frags &f) {
@@ -416,6 +465,64 @@ extern "C" int planmoe_gemm_nt_bf16(const void *a, const void *b, const void *bi
     if (activation == 0) gemm_nt_bf16_kernel<0><<<grid, 256, GEMM_LDS, (hipStream_t)stream>>>(p);
     else gemm_nt_bf16_kernel<1><<<grid, 256, GEMM_LDS, (hipStream_t)stream>>>(p);
     PM_LAUNCH_CHECK("planmoe_gemm_nt_bf16");
+    return 0;
+}
+
+extern "C" int planmoe_gemm_nn_bf16(const void *a, const void *b, const void *bias, int activation, int batches,
+                                    int m, int n, int k, int lda, int ldb, int ldc, int64_t batch_stride_a,
+                                    int64_t batch_stride_b, int64_t batch_stride_c, void *c, void *stream)
+{
+    PM_REQUIRE(batches >= 0 && m >= 0 && n >= 0 && k >= 64, "planmoe_gemm_nn_bf16: bad shape");
+    if (batches == 0 || m == 0 || n == 0) return 0;
+    PM_REQUIRE(a && b && c, "planmoe_gemm_nn_bf16: NULL argument");
+    PM_REQUIRE(activation == 0 || activation == 1, "planmoe_gemm_nn_bf16: activation is 0 (none) or 1 (relu)");
+    PM_REQUIRE(k % DMA_BK == 0, "planmoe_gemm_nn_bf16: k must be a multiple of %d", DMA_BK);
+    PM_REQUIRE(n % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && ldc % 8 == 0 && lda >= k && ldb >= n && ldc >= n,
+               "planmoe_gemm_nn_bf16: n and the row pitches must be multiples of 8 (16-byte pieces); pitches cover their rows");
+    PM_REQUIRE(batch_stride_a % 8 == 0 && batch_stride_b % 8 == 0 && batch_stride_c % 8 == 0 && aligned16(a) && aligned16(b) && aligned16(c),
+               "planmoe_gemm_nn_bf16: operands must be 16-byte aligned");
+    PM_REQUIRE((int64_t)m * lda * 2 < ((int64_t)1 << 32) && (int64_t)DMA_BK * ldb * 2 < ((int64_t)1 << 31),
+               "planmoe_gemm_nn_bf16: the first operand of one batch must stay under 4 GiB, 64 rows of the second under 2 GiB");
+    const int64_t tm = ((int64_t)m + GEMM_BM - 1) / GEMM_BM, tn = ((int64_t)n + GEMM_BN - 1) / GEMM_BN;
+    const int64_t per_xcd = (tm * tn * batches + 7) / 8;
+    PM_REQUIRE(per_xcd * 8 < ((int64_t)1 << 31), "planmoe_gemm_nn_bf16: too many tiles");
+    GemmArgs p{(const uint16_t *)a, (const uint16_t *)b, (const uint16_t *)bias, (uint16_t *)c, m, n, k, lda, ldb, ldc,
+               batch_stride_a, batch_stride_b, batch_stride_c, (int64_t)n, batches};
+    const void *fd = activation == 0 ? (const void *)gemm_nt_bf16_dma_kernel<0, false, true>
+                                     : (const void *)gemm_nt_bf16_dma_kernel<1, false, true>;
+    PM_REQUIRE(hipFuncSetAttribute(fd, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS) == hipSuccess,
+               "planmoe_gemm_nn_bf16: the kernel needs %d bytes of LDS", GEMM_LDS);
+    const dim3 tiles((unsigned)(per_xcd * 8));
+    if (activation == 0) gemm_nt_bf16_dma_kernel<0, false, true><<<tiles, 256, GEMM_LDS, (hipStream_t)stream>>>(p);
+    else gemm_nt_bf16_dma_kernel<1, false, true><<<tiles, 256, GEMM_LDS, (hipStream_t)stream>>>(p);
+    PM_LAUNCH_CHECK("planmoe_gemm_nn_bf16");
+    return 0;
+}
+
+extern "C" int planmoe_gemm_tn_bf16(const void *a, const void *b, int batches, int m, int n, int k, int lda, int ldb,
+                                    int ldc, int64_t batch_stride_a, int64_t batch_stride_b, int64_t batch_stride_c,
+                                    void *c, void *stream)
+{
+    PM_REQUIRE(batches >= 0 && m >= 0 && n >= 0 && k >= 64, "planmoe_gemm_tn_bf16: bad shape");
+    if (batches == 0 || m == 0 || n == 0) return 0;
+    PM_REQUIRE(a && b && c, "planmoe_gemm_tn_bf16: NULL argument");
+    PM_REQUIRE(k % DMA_BK == 0, "planmoe_gemm_tn_bf16: k must be a multiple of %d", DMA_BK);
+    PM_REQUIRE(m % 8 == 0 && n % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && ldc % 8 == 0 && lda >= m && ldb >= n && ldc >= n,
+               "planmoe_gemm_tn_bf16: m, n and the row pitches must be multiples of 8 (16-byte pieces); pitches cover their rows");
+    PM_REQUIRE(batch_stride_a % 8 == 0 && batch_stride_b % 8 == 0 && batch_stride_c % 8 == 0 && aligned16(a) && aligned16(b) && aligned16(c),
+               "planmoe_gemm_tn_bf16: operands must be 16-byte aligned");
+    PM_REQUIRE((int64_t)DMA_BK * lda * 2 < ((int64_t)1 << 31) && (int64_t)DMA_BK * ldb * 2 < ((int64_t)1 << 31),
+               "planmoe_gemm_tn_bf16: 64 rows of an operand must stay under 2 GiB");
+    const int64_t tm = ((int64_t)m + GEMM_BM - 1) / GEMM_BM, tn = ((int64_t)n + GEMM_BN - 1) / GEMM_BN;
+    const int64_t per_xcd = (tm * tn * batches + 7) / 8;
+    PM_REQUIRE(per_xcd * 8 < ((int64_t)1 << 31), "planmoe_gemm_tn_bf16: too many tiles");
+    GemmArgs p{(const uint16_t *)a, (const uint16_t *)b, nullptr, (uint16_t *)c, m, n, k, lda, ldb, ldc,
+               batch_stride_a, batch_stride_b, batch_stride_c, 0, batches};
+    const void *fd = (const void *)gemm_nt_bf16_dma_kernel<0, true, true>;
+    PM_REQUIRE(hipFuncSetAttribute(fd, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS) == hipSuccess,
+               "planmoe_gemm_tn_bf16: the kernel needs %d bytes of LDS", GEMM_LDS);
+    gemm_nt_bf16_dma_kernel<0, true, true><<<dim3((unsigned)(per_xcd * 8)), 256, GEMM_LDS, (hipStream_t)stream>>>(p);
+    PM_LAUNCH_CHECK("planmoe_gemm_tn_bf16");
     return 0;
 }
 

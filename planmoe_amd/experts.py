@@ -1,7 +1,7 @@
 """Fused expert FFN -- mirror of the reference's experts/ffn.py (two batched GEMMs with bias and
 activation between dispatch and combine).  On the GPU in bf16 both GEMMs, and the four of their
-backward pass, are planmoe_gemm_nt_bf16 (hand-written for the matrix cores; no library GEMM is
-called at the layer's sizes); forward_from_codes() takes the int8 codes of the receive buffer
+backward pass, are planmoe_gemm_nt_bf16 / _nn_ / _tn_ (one hand-written kernel for the matrix cores
+that reads either operand either way round; no library GEMM is called at the layer's sizes); forward_from_codes() takes the int8 codes of the receive buffer
 straight into the first GEMM."""
 import torch
 
@@ -32,15 +32,21 @@ class _WeightForms:
 class _BatchedLinear(torch.autograd.Function):
     """y = act(x @ w + bias) over experts: x [E, R, in], w [E, in, out] (as the reference stores it),
     bias [E, out], act = relu or nothing; torch.add(torch.matmul(x, w), bias.unsqueeze(1)) of
-    experts/ffn.py:77-79 with its two bf16 roundings.  Backward: dx = dy @ w^T reads w as stored;
-    dw = x^T @ dy takes transposed copies of x and dy whose row index (the reduction) is padded with
-    zeros to the kernel's k-tile; dbias sums in fp32."""
+    experts/ffn.py:77-79 with its two bf16 roundings.  All three products read their operands as they
+    lie in memory when the reduction length is a multiple of 64 (planmoe_gemm_nn_bf16 for y,
+    planmoe_gemm_nt_bf16 for dx = dy @ w^T, planmoe_gemm_tn_bf16 for dw = x^T @ dy); otherwise y takes a
+    transposed copy of w (kept per weight version) and dw transposed copies of x and dy whose row index
+    (the reduction) is padded with zeros to the kernel's k-tile.  dbias sums in fp32."""
 
     @staticmethod
     def forward(ctx, x, w, bias, relu, forms):
         from . import ops
         x = x.contiguous()
-        y = ops.gemm_nt_bf16(x, forms.k_major(w), bias.detach() if bias is not None else None, relu=relu)
+        b = bias.detach() if bias is not None else None
+        if x.shape[2] % 64 == 0:
+            y = ops.gemm_nn_bf16(x, w.detach().contiguous(), b, relu=relu)          # the weight as it is stored
+        else:
+            y = ops.gemm_nt_bf16(x, forms.k_major(w), b, relu=relu)
         ctx.save_for_backward(x, w, y if relu else None)
         ctx.relu, ctx.has_bias = relu, bias is not None
         return y
@@ -56,7 +62,10 @@ class _BatchedLinear(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             dx = ops.gemm_nt_bf16(gy, w.detach().contiguous())                    # [E, R, out] x [E, in, out]^T
         if ctx.needs_input_grad[1]:
-            dw = ops.gemm_nt_bf16(ops.transpose_bf16(x, 64), ops.transpose_bf16(gy, 64))      # [E, in, R'] x [E, out, R']^T
+            if x.shape[1] % 64 == 0:
+                dw = ops.gemm_tn_bf16(x, gy)                                          # x^T dy, both as they lie
+            else:
+                dw = ops.gemm_nt_bf16(ops.transpose_bf16(x, 64), ops.transpose_bf16(gy, 64))      # [E, in, R'] x [E, out, R']^T
         if ctx.has_bias and ctx.needs_input_grad[2]:
             db = gy.sum(dim=1, dtype=torch.float32).to(gy.dtype)
         return dx, dw, db, None, None

@@ -654,6 +654,53 @@ def gemm_nt_bf16(a, b, bias=None, relu=False, out=None):
     return out
 
 
+def gemm_nn_bf16(a, b, bias=None, relu=False, out=None):
+    """c[e] = act(bf16(bf16(a[e] @ b[e]) + bias[e])): a [B, m, k], b [B, k, n] (a weight as the experts store
+    it), bias [B, n] or None, bf16 -> [B, m, n] bf16 (planmoe_gemm_nn_bf16; k a multiple of 64, n of 8)."""
+    _need_gpu(a, "gemm_nn_bf16")
+    a, b = _contig(a, "gemm_nn_bf16"), _contig(b, "gemm_nn_bf16")
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or a.dim() != 3 or b.dim() != 3:
+        raise PlanMoEError("gemm_nn_bf16: bf16 [batches, m, k] x [batches, k, n] operands")
+    B, m, k = a.shape
+    n = b.shape[2]
+    if b.shape[0] != B or b.shape[1] != k:
+        raise PlanMoEError("gemm_nn_bf16: operands disagree: a %s, b %s" % (tuple(a.shape), tuple(b.shape)))
+    if k % 64 or n % 8:
+        raise PlanMoEError("gemm_nn_bf16: k must be a multiple of 64, n of 8 (got k = %d, n = %d)" % (k, n))
+    if bias is not None:
+        bias = _contig(bias.to(torch.bfloat16), "gemm_nn_bf16")
+        if tuple(bias.shape) != (B, n):
+            raise PlanMoEError("gemm_nn_bf16: bias must be [batches, n]")
+    if out is None:
+        out = torch.empty((B, m, n), dtype=torch.bfloat16, device=a.device)
+    elif tuple(out.shape) != (B, m, n) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise PlanMoEError("gemm_nn_bf16: out must be a contiguous bf16 [batches, m, n] tensor")
+    check(lib.planmoe_gemm_nn_bf16(_ptr(a), _ptr(b), _ptr(bias), int(bool(relu)), B, m, n, k, k, n, n, m * k, k * n,
+                                   m * n, _ptr(out), _stream(a)))
+    return out
+
+
+def gemm_tn_bf16(a, b, out=None):
+    """c[e] = a[e]^T @ b[e]: a [B, k, m], b [B, k, n] bf16 -> [B, m, n] bf16 (planmoe_gemm_tn_bf16; k a
+    multiple of 64, m and n multiples of 8)."""
+    _need_gpu(a, "gemm_tn_bf16")
+    a, b = _contig(a, "gemm_tn_bf16"), _contig(b, "gemm_tn_bf16")
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or a.dim() != 3 or b.dim() != 3:
+        raise PlanMoEError("gemm_tn_bf16: bf16 [batches, k, cols] operands")
+    B, k, m = a.shape
+    n = b.shape[2]
+    if b.shape[0] != B or b.shape[1] != k:
+        raise PlanMoEError("gemm_tn_bf16: operands disagree: a %s, b %s" % (tuple(a.shape), tuple(b.shape)))
+    if k % 64 or m % 8 or n % 8:
+        raise PlanMoEError("gemm_tn_bf16: k must be a multiple of 64, m and n of 8 (got k = %d, m = %d, n = %d)" % (k, m, n))
+    if out is None:
+        out = torch.empty((B, m, n), dtype=torch.bfloat16, device=a.device)
+    elif tuple(out.shape) != (B, m, n) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise PlanMoEError("gemm_tn_bf16: out must be a contiguous bf16 [batches, m, n] tensor")
+    check(lib.planmoe_gemm_tn_bf16(_ptr(a), _ptr(b), B, m, n, k, m, n, n, k * m, k * n, m * n, _ptr(out), _stream(a)))
+    return out
+
+
 # ------------------------------------------------------------------------------ zfp codec
 def zfp_stream_bytes(dims, nx, ny, rate=8.0):
     return int(lib.planmoe_zfp_stream_bytes(dims, nx, ny, float(rate)))

@@ -84,3 +84,39 @@ def test_gemm_config2_ffn_shape():
     rows = torch.tensor([0, 1, 31, 32, 127, 128, 255, 256, 257, 2559, 2560, 4000, 5118, 5119])
     _check(got[:, rows].float().cpu(), a[:, rows], w, bias, True)
     assert bool(torch.isfinite(got.float()).all())
+
+
+@pytest.mark.parametrize("B,k,m,n", [(1, 64, 8, 8), (2, 128, 256, 256), (3, 192, 264, 520), (2, 640, 1000, 136),
+                                     (3, 64, 696, 2312), (1, 4096, 72, 200)])
+def test_gemm_tn_equals_the_nt_form_on_transposed_copies(B, k, m, n):
+    """c = a^T b with the operands as they lie (reduction index slow) against planmoe_gemm_nt_bf16 on
+    transposed copies: same products, same order of the fp32 sums, hence the same bits; and against fp64."""
+    from planmoe_amd import ops
+    print("case", B, k, m, n, flush=True)
+    g = torch.Generator().manual_seed(B + k + m + n)
+    a = torch.randn(B, k, m, generator=g).bfloat16()
+    b = (torch.randn(B, k, n, generator=g) * k ** -0.5).bfloat16()
+    got = ops.gemm_tn_bf16(a.to(DEV), b.to(DEV))
+    want = ops.gemm_nt_bf16(ops.transpose_bf16(a.to(DEV), 64), ops.transpose_bf16(b.to(DEV), 64))
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    ref = torch.einsum("bkm,bkn->bmn", a.double(), b.double())
+    mag = torch.einsum("bkm,bkn->bmn", a.double().abs(), b.double().abs())
+    assert ((got.double().cpu() - ref).abs() <= 2.0 ** -8 * ref.abs() + 2.0 ** -14 * mag + 1e-30).all()
+
+
+@pytest.mark.parametrize("B,m,k,n,with_bias,relu", [(1, 8, 64, 8, True, False), (2, 300, 128, 264, False, True),
+                                                    (3, 513, 192, 2312, True, True), (2, 1, 4096, 136, True, False)])
+def test_gemm_nn_equals_the_nt_form_on_a_transposed_weight(B, m, k, n, with_bias, relu):
+    """c = act(a w + bias) with the weight as the experts store it, [k, n], against planmoe_gemm_nt_bf16 on its
+    transposed copy: the same bits."""
+    from planmoe_amd import ops
+    print("case", B, m, k, n, with_bias, relu, flush=True)
+    g = torch.Generator().manual_seed(B + m + k + n)
+    a = torch.randn(B, m, k, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(B, k, n, generator=g) * k ** -0.5).bfloat16().to(DEV)
+    bias = torch.randn(B, n, generator=g).bfloat16().to(DEV) if with_bias else None
+    got = ops.gemm_nn_bf16(a, w, bias, relu=relu)
+    want = ops.gemm_nt_bf16(a, ops.transpose_bf16(w), bias, relu=relu)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
