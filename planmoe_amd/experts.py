@@ -57,7 +57,7 @@ class _BatchedLinear(torch.autograd.Function):
         x, w, y = ctx.saved_tensors
         gy = gy.contiguous()
         if ctx.relu:
-            gy = gy * (y > 0)
+            gy = torch.ops.aten.threshold_backward(gy, y, 0.0)      # relu's own backward: one pass over dy and y
         dx = dw = db = None
         if ctx.needs_input_grad[0]:
             dx = ops.gemm_nt_bf16(gy, w.detach().contiguous())                    # [E, R, out] x [E, in, out]^T
