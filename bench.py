@@ -244,6 +244,13 @@ def kernel_table(only=None):
     add("combine_fwd", "1", 3 * T1 * M1 * 4, lambda: ops.combine_fwd(d1, i1, l1, g1, T1, C1))
     del d1
 
+    def chain1():
+        r = ops.forward_plain(x1, w1, 2, C1)
+        return ops.combine_fwd(r["dispatched"], list(r["indices"]), list(r["locations"]), list(r["gates"]), T1, C1)
+    add("forward_plain (gate, routing, dispatch)", "1", T1 * M1 * 4 + E1 * C1 * M1 * 4 + T1 * 24, lambda: ops.forward_plain(x1, w1, 2, C1))
+    # the config's whole chain: x read, the dispatched buffer written and read, y written
+    add("chain: forward_plain, combine", "1", T1 * M1 * 4 + E1 * C1 * M1 * 4 + 2 * T1 * M1 * 4 + T1 * M1 * 4 + T1 * 24, chain1)
+
     # config 3: 32768 x 2048 bf16, 64 experts, top-1, skewed logits
     T3, M3, E3 = 32768, 2048, 64
     x3 = torch.randn(T3, M3, generator=g).bfloat16().to(dev)
@@ -258,6 +265,10 @@ def kernel_table(only=None):
     r3 = ops.gate_route(x3, w3, 1, logit_bias=bias)
     i3, l3 = list(r3["indices"]), list(r3["locations"])
     add("dispatch_fwd", "3", kept(l3, C3) * M3 * 2 + E3 * C3 * M3 * 2 + T3 * 12, lambda: ops.dispatch_fwd(x3, i3, l3, None, E3, C3))
+
+    # the config's chain as stated (no codec): x read by the gate, kept rows read again, the buffer written
+    add("forward_plain (gate, routing, dispatch)", "3", T3 * M3 * 2 + E3 * C3 * M3 * 2 + T3 * 12,
+        lambda: ops.forward_plain(x3, w3, 1, C3, logit_bias=bias))
     lg = ops.gate_logits(x3, w3, torch.float32)
     add("route_topk (logits in)", "3", T3 * E3 * 4 + T3 * 12, lambda: ops.route_topk(lg, 1, is_logits=True, logit_bias=bias))
     mask = (torch.rand(T3, E3, device=dev) < 0.1).to(torch.int32)

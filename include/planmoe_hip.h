@@ -251,6 +251,17 @@ int planmoe_gate_route(const void *x, const void *wg, int dtype, int fp32_gate,
                        int64_t plane_stride, void *logits_out, void *scores_out, float *l_aux,
                        int32_t *expert_counts, void *workspace, size_t workspace_bytes, void *stream);
 
+/* gate GEMM + routing + dispatch without a codec (LinearTopKGate + extract_critical + fast_encode with
+ * no gates, moe_layer.py:230-266 when no compressor is set): additionally `dispatched`
+ * [experts*capacity, model_dim] in `dtype`, equal to what planmoe_dispatch_fwd produces from the same
+ * routing (kept rows as 0 + x, empty slots zero).  Two launches; the second works out the slots from
+ * the first one's group histograms, so planmoe_gate_route's launch that finishes them is not needed. */
+int planmoe_forward_plain(const void *x, const void *wg, int dtype, int fp32_gate,
+                          const float *logit_bias, int samples, int model_dim, int experts, int top_k,
+                          int normalize_gate, int capacity, int32_t *indices, int32_t *locations,
+                          void *gates, int64_t plane_stride, void *logits_out, void *scores_out,
+                          float *l_aux, int32_t *expert_counts, void *dispatched,
+                          void *workspace, size_t workspace_bytes, void *stream);
 /* gate GEMM + routing + dispatch + int8 compress: additionally codes [experts*capacity,
  * model_dim] uint8 and bias / scale [experts*capacity] in `dtype`, equal to what
  * planmoe_dispatch_int8 produces from the same routing. */

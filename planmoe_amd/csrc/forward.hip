@@ -492,7 +492,9 @@ __global__ __launch_bounds__(256) void route_locations_merged_kernel(
 // none of its choices leaves without reading its row.  Pays when many tokens are dropped (a
 // capacity factor of 1 with skewed routing drops half of them); otherwise the row is requested
 // first so that it travels while the slots are being worked out.
-template <int DT, int CACHE, bool MERGED, bool SLOT_FIRST = false>
+// PLAIN: no codec -- `codes` is the dispatched buffer in x's dtype and a kept row arrives there as
+// 0 + x (what fast_encode's accumulation into zeros leaves: -0 becomes +0), an empty slot as zeros.
+template <int DT, int CACHE, bool MERGED, bool SLOT_FIRST = false, bool PLAIN = false>
 __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
     const void *__restrict__ x, const int32_t *__restrict__ indices, int32_t *__restrict__ locations,
     int64_t stride, int top_k, int samples, int model_dim, int experts, int capacity,
@@ -547,6 +549,11 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
             const int e = s / capacity;
             const int filled = MERGED ? s_tot[e] : totals[e];
             if (s - e * capacity < filled) continue;             // slot holds a token
+            if constexpr (PLAIN) {
+                uint4 *row = reinterpret_cast<uint4 *>(codes + (int64_t)s * units * 16);
+                for (int u = lane; u < units; u += WAVE) stream_store(row + u, make_uint4(0u, 0u, 0u, 0u));
+                continue;
+            }
             uint8_t *row = codes + (int64_t)s * model_dim;
             for (int u = lane; u < units; u += WAVE) {
                 if constexpr (V == 8) stream_store(reinterpret_cast<uint2 *>(row) + u, make_uint2(0u, 0u));
@@ -603,6 +610,27 @@ __global__ __launch_bounds__(256) void dispatch_int8_routed_kernel(
         request_row();
         slot = find_slot();
         if (__ballot(slot >= 0) == 0) return;
+    }
+
+    if constexpr (PLAIN) {
+        auto copy = [&](int u, const uint4 &raw) {
+            float f[V];
+            E::unpack(raw, f);
+#pragma unroll
+            for (int i = 0; i < V; ++i) f[i] = 0.f + f[i];
+            const uint4 v = E::pack(f);
+            for (int j = 0; j < top_k; ++j) {
+                const int sl = rl_i(slot, j);
+                if (sl >= 0) stream_store(reinterpret_cast<uint4 *>(codes + (int64_t)sl * units * 16) + u, v);
+            }
+        };
+        if constexpr (CACHE > 0) {
+#pragma unroll
+            for (int c = 0; c < CACHE; ++c) if (c * WAVE + lane < units) copy(c * WAVE + lane, cache[c]);
+        } else {
+            for (int u = lane; u < units; u += WAVE) copy(u, src[u]);
+        }
+        return;
     }
 
     float mn, mx;
@@ -675,17 +703,19 @@ static void launch_dispatch_routed(int per_lane, unsigned grid, hipStream_t st, 
                                    const float *loss_part, int loss_parts, float *l_aux,
                                    const float *row_min, const float *row_max, bool merged,
                                    const int32_t *hist_t, const float *me_t, int groups, int gstride,
-                                   int fill_blocks, int32_t *counts, int fill_first)
+                                   int fill_blocks, int32_t *counts, int fill_first, bool plain = false)
 {
     // a capacity factor of at most 1: every imbalance of the routing drops tokens
     const bool slot_first = merged && (int64_t)experts * capacity <= (int64_t)top_k * samples;
-#define PM_DR_(CACHE, MERGED, FIRST)                                                                 \
-    dispatch_int8_routed_kernel<DT, CACHE, MERGED, FIRST><<<grid, 256, 0, st>>>(x, indices, locations, stride, top_k, \
+#define PM_DR_(CACHE, MERGED, FIRST, PLAIN)                                                          \
+    dispatch_int8_routed_kernel<DT, CACHE, MERGED, FIRST, PLAIN><<<grid, 256, 0, st>>>(x, indices, locations, stride, top_k, \
         samples, model_dim, experts, capacity, codes, bias, scale, offs, totals, rank, group_tokens,  \
         token_blocks, loss_part, loss_parts, l_aux, row_min, row_max, hist_t, me_t, groups, gstride,  \
         fill_blocks, counts, fill_first)
-#define PM_DR(CACHE) do { if (slot_first) PM_DR_(CACHE, true, true); else if (merged) PM_DR_(CACHE, true, false); \
-                          else PM_DR_(CACHE, false, false); } while (0)
+#define PM_DR(CACHE) do { if (plain) { if (slot_first) PM_DR_(CACHE, true, true, true); else if (merged) PM_DR_(CACHE, true, false, true); \
+                                       else PM_DR_(CACHE, false, false, true); }                      \
+                          else if (slot_first) PM_DR_(CACHE, true, true, false); else if (merged) PM_DR_(CACHE, true, false, false); \
+                          else PM_DR_(CACHE, false, false, false); } while (0)
     if (per_lane <= 2) PM_DR(2);
     else if (per_lane <= 4) PM_DR(4);
     else if (per_lane <= 8) PM_DR(8);
@@ -823,7 +853,7 @@ static int run_gate_route(const void *x, const void *wg, int dtype, int fp32_gat
 static int run_dispatch_routed(const void *x, int dtype, int samples, int model_dim, int experts,
                                int capacity, const int32_t *indices, int32_t *locations, int64_t stride,
                                float *l_aux, int32_t *counts, uint8_t *codes, void *bias, void *scale,
-                               const FwdPlan &plan, hipStream_t st)
+                               const FwdPlan &plan, hipStream_t st, bool plain = false)
 {
     const int slots = experts * capacity;
     const int token_blocks = (samples + 3) / 4;
@@ -844,7 +874,7 @@ static int run_dispatch_routed(const void *x, int dtype, int samples, int model_
                                    dtype == PLANMOE_BF16 ? plan.ws.row_min : nullptr,
                                    dtype == PLANMOE_BF16 ? plan.ws.row_max : nullptr, plan.merged,
                                    plan.ws.hist_t, plan.ws.me_t, plan.groups, plan.ws.gstride, fill_blocks, counts,
-                                   plan.merged && plan.k * experts > 32));
+                                   plan.merged && plan.k * experts > 32, plain));
     return 0;
 }
 
@@ -1044,6 +1074,35 @@ extern "C" int planmoe_forward_int8(const void *x, const void *wg, int dtype, in
     if (run_dispatch_routed(x, dtype, samples, model_dim, experts, capacity, indices, locations,
                             plane_stride, l_aux, expert_counts, codes, bias, scale, plan, st)) return 1;
     PM_LAUNCH_CHECK("planmoe_forward_int8");
+    return 0;
+}
+
+extern "C" int planmoe_forward_plain(const void *x, const void *wg, int dtype, int fp32_gate,
+                                     const float *logit_bias, int samples, int model_dim, int experts,
+                                     int top_k, int normalize_gate, int capacity, int32_t *indices,
+                                     int32_t *locations, void *gates, int64_t plane_stride,
+                                     void *logits_out, void *scores_out, float *l_aux,
+                                     int32_t *expert_counts, void *dispatched, void *workspace,
+                                     size_t workspace_bytes, void *stream)
+{
+    PM_REQUIRE(capacity >= 0 && (int64_t)experts * capacity < (1ll << 31), "planmoe_forward_plain: bad capacity");
+    if (fused_check("planmoe_forward_plain", x, wg, dtype, samples, model_dim, experts, top_k, plane_stride)) return 1;
+    PM_REQUIRE(indices && locations && gates, "planmoe_forward_plain: NULL routing output");
+    PM_REQUIRE(dispatched || capacity == 0, "planmoe_forward_plain: NULL output");
+    PM_REQUIRE(aligned16(dispatched), "planmoe_forward_plain: the dispatched buffer must be 16-byte aligned");
+    PM_REQUIRE(workspace && workspace_bytes >= planmoe_forward_workspace_bytes(samples, experts, top_k),
+               "planmoe_forward_plain: workspace too small");
+    workspace = fwd_tables(workspace);
+    hipStream_t st = (hipStream_t)stream;
+    FwdPlan plan;
+    fwd_plan(plan, workspace, samples, experts, top_k);
+    if (run_gate_route(x, wg, dtype, fp32_gate, logit_bias, samples, model_dim, experts, top_k,
+                       normalize_gate, indices, locations, gates, plane_stride, logits_out, scores_out,
+                       l_aux, expert_counts, workspace, st, plan, !plan.merged)) return 1;
+    if (run_dispatch_routed(x, dtype, samples, model_dim, experts, capacity, indices, locations,
+                            plane_stride, l_aux, expert_counts, (uint8_t *)dispatched, nullptr, nullptr, plan, st,
+                            true)) return 1;
+    PM_LAUNCH_CHECK("planmoe_forward_plain");
     return 0;
 }
 

@@ -434,6 +434,23 @@ def forward_int8(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, norma
     return out
 
 
+def forward_plain(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
+                  want_logits=False, want_scores=False, want_l_aux=True, want_counts=False):
+    """Gate GEMM + routing + dispatch (no codec) in two launches: gate_route's outputs plus
+    `dispatched` [E*capacity, M] in x's dtype, what fast_encode without gates makes of x (the second
+    launch works out the slots itself, so the stand-alone routing's launch that finishes them and a
+    pass over the routing planes are saved)."""
+    x, wg, T, M, E, k, bias, out, ws = _forward_common(x, wg, top_k, fp32_gate, logit_bias, want_logits,
+                                                       want_scores, want_l_aux, want_counts)
+    out["dispatched"] = torch.empty((E * capacity_, M), dtype=x.dtype, device=x.device)
+    check(lib.planmoe_forward_plain(_ptr(x), _ptr(wg), _dt(x, "forward_plain"), int(bool(fp32_gate)), _ptr(bias),
+                                    T, M, E, k, int(bool(normalize_gate)), capacity_, _ptr(out["indices"]),
+                                    _ptr(out["locations"]), _ptr(out["gates"]), max(T, 1), _ptr(out["logits"]),
+                                    _ptr(out["scores"]), _ptr(out["l_aux"]), _ptr(out["counts"]),
+                                    _ptr(out["dispatched"]), _ptr(ws), ws.numel(), _stream(x)))
+    return out
+
+
 def forward_int8_single_serves(x, wg, top_k):
     """The shapes planmoe_forward_int8_single takes: bf16 rows of 4096 values, up to 16 experts,
     top_k <= 4, at most 64 tokens per compute unit."""

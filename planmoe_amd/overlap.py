@@ -281,14 +281,20 @@ class _GateRouteEncode(torch.autograd.Function):
     """Gate GEMM, routing and fast_encode as one node of the graph for the compressors without an
     int8 send side: x has one consumer, so its two gradients (through the dispatched rows and
     through the gate) meet in the epilogue of one GEMM instead of a pass of their own.
-    codec 'plain': x -> the [E * C, M] buffer (planmoe_gate_route + planmoe_dispatch_fwd);
+    codec 'plain': x -> the [E * C, M] buffer (planmoe_forward_plain: gate + routing, then a dispatch
+                   launch that works out the slots itself);
     codec 'zfp':   x -> Decompress(Comm(Compress(buffer))) (planmoe_dispatch_zfp, as _EncodeZfp).
     Outputs as _GateRouteEncodeInt8."""
 
     @staticmethod
     def forward(ctx, x, w, top_k, experts, capacity, fp32_gate, normalize_gate, codec):
-        out = ops.gate_route(x, w, top_k, fp32_gate=fp32_gate, normalize_gate=normalize_gate,
-                             want_scores=True, want_counts=True)
+        if codec == 'zfp':
+            out = ops.gate_route(x, w, top_k, fp32_gate=fp32_gate, normalize_gate=normalize_gate,
+                                 want_scores=True, want_counts=True)
+        else:
+            # planmoe_forward_plain: the dispatch launch works out the slots itself (one launch less)
+            out = ops.forward_plain(x, w, top_k, capacity, fp32_gate=fp32_gate, normalize_gate=normalize_gate,
+                                    want_scores=True, want_counts=True)
         indices, locations = out["indices"], out["locations"]
         ctx.save_for_backward(x, w, out["scores"], indices, locations, out["counts"])
         ctx.experts, ctx.capacity, ctx.normalize_gate, ctx.codec = experts, capacity, normalize_gate, codec
@@ -297,7 +303,7 @@ class _GateRouteEncode(torch.autograd.Function):
             stream = ops.dispatch_zfp(x, list(indices), list(locations), None, experts, capacity)
             y = ops.zfp_decompress(stream, x.shape[1], experts * capacity, 2)
         else:
-            y = ops.dispatch_fwd(x, list(indices), list(locations), None, experts, capacity)
+            y = out["dispatched"]
         return y, out["gates"], out["l_aux"], indices, locations
 
     @staticmethod

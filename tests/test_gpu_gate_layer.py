@@ -223,6 +223,39 @@ def test_fused_forward_matches_unfused_and_oracle(T, M, E, k, cf, dtype, fp32_ga
         assert abs(float(r2["l_aux"]) - float(out["l_aux"])) <= 1e-6 * abs(float(out["l_aux"]))
 
 
+@pytest.mark.parametrize("T,M,E,k,cf,dtype,fp32_gate,use_bias", [
+    (1000, 512, 8, 2, 1.25, torch.bfloat16, True, False), (33, 256, 4, 2, 1.0, torch.bfloat16, True, False),
+    (4096, 1024, 64, 1, 1.0, torch.bfloat16, True, True), (500, 2048, 2, 2, 1.0, torch.float32, True, False),
+    (700, 264, 16, 3, 0.5, torch.bfloat16, False, False), (257, 128, 33, 4, 1.0, torch.float16, True, False),
+    (31, 64, 5, 5, 2.0, torch.float32, False, True), (900, 260, 24, 20, 1.0, torch.float32, True, False),
+    (640, 512, 64, 17, 1.0, torch.bfloat16, False, False), (8192, 2048, 2, 2, 1.0, torch.float32, True, False)])
+def test_forward_plain_matches_routing_plus_dispatch_and_the_oracle(T, M, E, k, cf, dtype, fp32_gate, use_bias):
+    """planmoe_forward_plain (gate + routing + dispatch without a codec, two launches) against
+    planmoe_gate_route + planmoe_dispatch_fwd bit for bit, and its buffer against the oracle's encode of
+    the same routing (the last case is config 1 at full size)."""
+    from planmoe_amd import ops
+    g = torch.Generator().manual_seed(T + E)
+    x = torch.randn(T, M, generator=g).to(dtype)
+    x[min(3, T - 1), :8] = -0.0                              # 0 + (-0) = +0 in the reference's accumulation
+    x = x.to(DEV)
+    wg = (torch.randn(E, M, generator=g) * M ** -0.5).to(dtype).to(DEV)
+    bias = zipf_bias(E) if use_bias else None
+    C = ops.capacity(T, E, k, cf, 4)
+    for rep in range(2):
+        out = ops.forward_plain(x, wg, k, C, fp32_gate=fp32_gate, logit_bias=bias, want_scores=True, want_counts=True)
+        r2 = ops.gate_route(x, wg, k, fp32_gate=fp32_gate, logit_bias=bias, want_scores=True, want_counts=True)
+        for name in ("indices", "locations", "counts"):
+            assert torch.equal(r2[name], out[name]), name
+        assert np.array_equal(raw(r2["gates"]), raw(out["gates"])) and np.array_equal(raw(r2["scores"]), raw(out["scores"]))
+        assert abs(float(r2["l_aux"]) - float(out["l_aux"])) <= 1e-6 * abs(float(out["l_aux"]))
+        d2 = ops.dispatch_fwd(x, list(out["indices"]), list(out["locations"]), None, E, C)
+        assert np.array_equal(raw(out["dispatched"]), raw(d2))
+    if dtype != torch.float16:
+        idx, loc = out["indices"].cpu().numpy(), out["locations"].cpu().numpy()
+        want = oracle.encode(x.float().cpu().numpy(), list(idx), list(loc), None, E, C)
+        assert np.array_equal(out["dispatched"].float().cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
 @pytest.mark.parametrize("T,M,E,k", [(300, 776, 24, 2), (200, 264, 8, 2), (130, 1032, 64, 1)])
 def test_fused_forward_rows_of_one_sign(T, M, E, k):
     """Row min / max come out of the gate kernel's scan of the rows it streams: rows that do not
