@@ -51,6 +51,29 @@ def test_forward_chain_replays():
                                                o["scale"], o["counts"], o["l_aux"].reshape(1)])
 
 
+def test_forward_plain_and_the_expert_gemms_replay():
+    T, M, E, k, H = 1024, 256, 4, 2, 128
+    C = ops.capacity(T, E, k, 1.0, 4)                  # 512: a multiple of 64, so dW takes the direct form
+
+    def make(seed):
+        g = torch.Generator().manual_seed(20 + seed)
+        return [torch.randn(T, M, generator=g).bfloat16().to(DEV),
+                (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV),
+                (torch.randn(E, M, H, generator=g) * M ** -0.5).bfloat16().to(DEV),
+                torch.randn(E, H, generator=g).bfloat16().to(DEV)]
+
+    def run(inp):
+        out = ops.forward_plain(inp[0], inp[1], k, C, want_counts=True)
+        d = out["dispatched"].view(E, C, M)
+        h = ops.gemm_nn_bf16(d, inp[2], inp[3], relu=True)                       # [E, C, H]
+        dw = ops.gemm_tn_bf16(d, h)                                              # [E, M, H]
+        dx = ops.gemm_nt_bf16(h, inp[2])                                         # [E, C, M]
+        return out, h, dw, dx
+
+    replay_against_eager(make, run, lambda r: [r[0]["indices"], r[0]["locations"], r[0]["gates"], r[0]["dispatched"],
+                                               r[0]["counts"], r[0]["l_aux"].reshape(1), r[1], r[2], r[3]])
+
+
 def test_routing_and_sparse_kernels_replay():
     T, M, E, k = 1500, 256, 16, 2
     C = ops.capacity(T, E, k, 1.0, 4)
