@@ -940,7 +940,7 @@ static void single_order_after(SingleOrder &order, hipStream_t st, bool ordered)
     if (ordered) { order.last = st; order.has_last = true; }
 }
 
-// Whether the one-launch kernel serves the shape, and with how many rounds: model_dim 4096 bf16, up to
+// Whether the one-launch kernel serves the shape, and with how many rounds: bf16 rows of 1024 .. 4096 values, up to
 // 16 experts, top_k <= 4, and so few tokens that every work-group is resident at once.
 template <int SDT, int CAP, int NMMA, int ROUNDS>
 static bool single_fits(int groups)
@@ -992,7 +992,7 @@ static int run_forward_single(const void *x, const void *wg, int dtype, int fp32
                               void *scale, void *workspace, int spin_limit, int32_t *gave_up, hipStream_t st)
 {
     const int k = top_k < experts ? top_k : experts;
-    if (dtype != PLANMOE_BF16 || model_dim != 4096 || experts > 16 || k > 4 || samples < 1) return 2;
+    if (dtype != PLANMOE_BF16 || model_dim % 1024 != 0 || model_dim > 4096 || experts > 16 || k > 4 || samples < 1) return 2;
     if (!aligned16(codes) && capacity > 0) return 2;
     int cus = 0, dev = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -1005,9 +1005,19 @@ static int run_forward_single(const void *x, const void *wg, int dtype, int fp32
 #define PM_FS_ARGS rounds, groups, st, x, wg, logit_bias, samples, experts, k, normalize_gate, capacity, indices, \
                    locations, gates, stride, logits_out, scores_out, l_aux, counts, codes, bias, scale, workspace,   \
                    spin_limit, gave_up
-    if (fp32_gate) return experts <= 8 ? launch_single<PLANMOE_F32, 8, 16>(PM_FS_ARGS)
-                                       : launch_single<PLANMOE_F32, 16, 16>(PM_FS_ARGS);
-    return experts <= 8 ? launch_single<PLANMOE_BF16, 8, 16>(PM_FS_ARGS) : launch_single<PLANMOE_BF16, 16, 16>(PM_FS_ARGS);
+#define PM_FS_M(NMMA)                                                                                               \
+    do {                                                                                                           \
+        if (fp32_gate) return experts <= 8 ? launch_single<PLANMOE_F32, 8, NMMA>(PM_FS_ARGS)                         \
+                                           : launch_single<PLANMOE_F32, 16, NMMA>(PM_FS_ARGS);                       \
+        return experts <= 8 ? launch_single<PLANMOE_BF16, 8, NMMA>(PM_FS_ARGS) : launch_single<PLANMOE_BF16, 16, NMMA>(PM_FS_ARGS); \
+    } while (0)
+    switch (model_dim) {                        // rows of 256 NMMA values: every wave owns an eighth of a row
+    case 1024: PM_FS_M(4);
+    case 2048: PM_FS_M(8);
+    case 3072: PM_FS_M(12);
+    default: PM_FS_M(16);
+    }
+#undef PM_FS_M
 #undef PM_FS_ARGS
 }
 
@@ -1137,7 +1147,7 @@ extern "C" int planmoe_forward_int8_single(const void *x, const void *wg, int dt
                                       spin_limit > 0 ? spin_limit : (1 << 20), gave_up, st);
     if (rc == 0) single_order_after(order, st, ordered);
     hold.unlock();
-    PM_REQUIRE(rc != 2, "planmoe_forward_int8_single: the one-launch kernel serves bf16 rows of 4096 values, up to 16 "
+    PM_REQUIRE(rc != 2, "planmoe_forward_int8_single: the one-launch kernel serves bf16 rows of 1024, 2048, 3072 or 4096 values, up to 16 "
                "experts, top_k <= 4 and at most 64 tokens per compute unit; use planmoe_forward_int8");
     PM_LAUNCH_CHECK("planmoe_forward_int8_single");
     return rc;

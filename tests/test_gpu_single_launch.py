@@ -13,10 +13,9 @@ DEV = "cuda:0"
 @pytest.mark.parametrize("T,E,k,cf,fp32_gate", [(16384, 8, 2, 1.25, True), (16384, 8, 2, 1.25, False), (16000, 8, 2, 1.25, True),
                                                 (4096, 8, 2, 1.0, True), (100, 4, 2, 1.0, True), (9000, 16, 3, 0.5, True),
                                                 (12288, 8, 1, 1.0, True), (5000, 12, 4, 2.0, False), (1, 3, 2, 1.0, True)])
-def test_single_launch_forward(T, E, k, cf, fp32_gate):
+def test_single_launch_forward(T, E, k, cf, fp32_gate, M=4096):
     from planmoe_amd import ops
-    M = 4096
-    print("case", T, E, k, cf, fp32_gate, flush=True)
+    print("case", T, E, k, cf, fp32_gate, M, flush=True)
     g = torch.Generator().manual_seed(T + E)
     x = torch.randn(T, M, generator=g).bfloat16().to(DEV)
     wg = (torch.randn(E, M, generator=g) * M ** -0.5).bfloat16().to(DEV)
@@ -47,6 +46,15 @@ def test_single_launch_forward(T, E, k, cf, fp32_gate):
     assert np.array_equal(out["codes"].cpu().numpy().reshape(-1), rc.reshape(-1))
     assert np.array_equal(bf16_bits(out["bias"]).reshape(-1), rb.reshape(-1))
     assert np.array_equal(bf16_bits(out["scale"]).reshape(-1), rs.reshape(-1))
+
+
+@pytest.mark.parametrize("T,M,E,k,cf,fp32_gate", [(16384, 2048, 8, 2, 1.25, True), (9000, 2048, 16, 3, 0.5, False),
+                                                  (16384, 1024, 8, 2, 1.25, True), (5000, 1024, 4, 1, 1.0, True),
+                                                  (12000, 3072, 8, 2, 1.25, True), (100, 3072, 12, 4, 2.0, False),
+                                                  (1, 2048, 3, 2, 1.0, True)])
+def test_single_launch_forward_other_row_lengths(T, M, E, k, cf, fp32_gate):
+    """The one-launch kernel at rows of 1024, 2048 and 3072 values: the same checks against the oracle."""
+    test_single_launch_forward(T, E, k, cf, fp32_gate, M)
 
 
 def test_single_launch_gives_up_cleanly_when_told_to():
