@@ -69,6 +69,16 @@ def test_argument_errors_are_reported_without_a_gpu():
     rc = lib.planmoe_forward_int8(p16, p16, 1, 1, None, 64, 512, 65, 2, 1, 16, p16, p16, p16, 64, None, None, None,
                                   None, p16, p16, p16, p16, 1 << 40, None)
     assert rc != 0 and b"64 experts" in lib.planmoe_last_error()
+    # the GEMM forms that read an operand along its slow index take the reduction in steps of 64
+    rc = lib.planmoe_gemm_nn_bf16(p16, p16, None, 0, 1, 64, 64, 96, 96, 64, 64, 0, 0, 0, p16, None)
+    assert rc != 0 and b"multiple of 64" in lib.planmoe_last_error()
+    rc = lib.planmoe_gemm_tn_bf16(p16, p16, 1, 64, 64, 96, 64, 64, 64, 0, 0, 0, p16, None)
+    assert rc != 0 and b"multiple of 64" in lib.planmoe_last_error()
+    rc = lib.planmoe_gemm_tn_bf16(p16, p16, 1, 60, 64, 64, 64, 64, 64, 0, 0, 0, p16, None)
+    assert rc != 0 and b"multiples of 8" in lib.planmoe_last_error()
+    rc = lib.planmoe_gemm_nn_bf16(p16, p16, None, 2, 1, 64, 64, 64, 64, 64, 64, 0, 0, 0, p16, None)
+    assert rc != 0 and b"activation" in lib.planmoe_last_error()
+    assert lib.planmoe_gemm_tn_bf16(None, None, 0, 64, 64, 64, 64, 64, 64, 0, 0, 0, None, None) == 0
     # empty inputs are a successful no-op
     assert lib.planmoe_int8_compress(None, 0, 0, 8, None, None, None, None) == 0
     assert lib.planmoe_lz_blocks(0) == 0 and lib.planmoe_lz_blocks(2049) == 2
