@@ -20,17 +20,12 @@
 // totals[E], loss_part[64], hist[groups][k][E], offs[groups][k][E], me[groups][E] (fp32),
 // rank[k][samples] (rank of a token inside its group), row_min[samples], row_max[samples]
 // (fp32; bf16 inputs only: the gate kernel scans the rows it streams anyway).
-#include "gate_core.hpp"
-#include "rows.hpp"
-#include "int8_core.hpp"
-#include "offsets.hpp"
+#include "forward_shared.hpp"
 #include <mutex>
 #include <atomic>
 #include <random>
 
 namespace pm {
-
-constexpr int STATIC_SCRATCH_DEVICES_MAX = 64;
 
 // tokens per work-group of the gate kernel = tokens per routing group (one lane each in the
 // routing epilogue): 64, or 32 on the split-K path (up to 16 experts) when 64 would leave
@@ -42,11 +37,6 @@ inline int fwd_group_tokens(int experts, int samples)
     return (experts <= 16 && samples < 64 * 256) ? 32 : 64;
 }
 constexpr int FWD_LOSS_PARTS = 64;
-// The first bytes of a forward workspace belong to the one-launch kernel alone (its launch counter,
-// ticket counters and published words, forward_single.hpp): its tags are unique only while that
-// counter grows by one per launch, so no other entry point may write there.  The tables of the
-// two-launch chain and of the stand-alone routing start behind it, whatever the shape.
-constexpr size_t FWD_TABLES_OFFSET = 139520;
 inline void *fwd_tables(void *workspace) { return (char *)workspace + FWD_TABLES_OFFSET; }
 
 // hist_t / me_t are the transposes of hist / me with the group index running fastest (rows of
@@ -104,8 +94,6 @@ __device__ __forceinline__ void wave_sum_n(T (&v)[N])
 #pragma unroll
     for (int i = 0; i < N; ++i) v[i] = wave_allreduce(v[i], [](T a, T b) { return a + b; });
 }
-
-__device__ __forceinline__ uint64_t lanes_below() { return ((uint64_t)1 << lane_id()) - 1; }
 
 // SDT: dtype of logits / scores / gates (F32 when fp32_gate, else the input dtype)
 // CAP: compile-time bound of the expert count held in registers by the routing epilogue
@@ -880,7 +868,7 @@ static int run_dispatch_routed(const void *x, int dtype, int samples, int model_
 
 } // namespace pm
 
-#include "forward_single.hpp"
+#include "forward_single_launch.hpp"
 #include "forward_ceiling.hpp"
 
 namespace pm {
@@ -940,49 +928,14 @@ static void single_order_after(SingleOrder &order, hipStream_t st, bool ordered)
     if (ordered) { order.last = st; order.has_last = true; }
 }
 
-// Whether the one-launch kernel serves the shape, and with how many rounds: bf16 rows of 1024 .. 4096 values, up to
-// 16 experts, top_k <= 4, and so few tokens that every work-group is resident at once.
-template <int SDT, int CAP, int NMMA, int ROUNDS>
-static bool single_fits(int groups)
-{
-    static int resident[STATIC_SCRATCH_DEVICES_MAX] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_SCRATCH_DEVICES_MAX) return false;
-    if (resident[dev] == 0) {
-        int per_cu = 0, cus = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, forward_single_kernel<SDT, CAP, NMMA, ROUNDS>,
-                                                         FS_THREADS, 0) != hipSuccess) per_cu = 0;
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 0;
-        resident[dev] = per_cu * cus > 0 ? per_cu * cus : -1;
-    }
-    return groups <= resident[dev];
-}
-
-template <int SDT, int CAP, int NMMA>
-static int launch_single(int rounds, int groups, hipStream_t st, const void *x, const void *wg, const float *bias,
-                         int samples, int experts, int k, int normalize, int capacity, int32_t *indices,
-                         int32_t *locations, void *gates, int64_t stride, void *logits_out, void *scores_out,
-                         float *l_aux, int32_t *counts, uint8_t *codes, void *bias_out, void *scale_out, void *ws,
-                         int spin_limit, int32_t *gave_up)
-{
-    const unsigned long long salt = process_salt();
-#define PM_FS(ROUNDS)                                                                                     \
-    do {                                                                                                  \
-        if (!single_fits<SDT, CAP, NMMA, ROUNDS>(groups)) return 2;                                       \
-        forward_single_kernel<SDT, CAP, NMMA, ROUNDS><<<groups, FS_THREADS, 0, st>>>(                     \
-            (const uint4 *)x, (const uint4 *)wg, bias, samples, experts, k, normalize, capacity, indices, \
-            locations, gates, stride, logits_out, scores_out, l_aux, counts, codes, bias_out, scale_out,  \
-            ws, salt, spin_limit, gave_up);                                                               \
-    } while (0)
-    switch (rounds) {
-    case 1: PM_FS(1); break;
-    case 2: PM_FS(2); break;
-    case 3: PM_FS(3); break;
-    default: PM_FS(4); break;
-    }
-#undef PM_FS
-    return 0;
-}
+#ifdef PM_FS_TRACE
+// measurement build: the one-launch kernel's four translation units folded into this one, so that its
+// stamps and the ceiling kernels' land in one array
+PM_FS_DEFINE(4)
+PM_FS_DEFINE(8)
+PM_FS_DEFINE(12)
+PM_FS_DEFINE(16)
+#endif
 
 // 0: launched; 2: the shape is not served by the one-launch kernel (nothing was enqueued)
 static int run_forward_single(const void *x, const void *wg, int dtype, int fp32_gate, const float *logit_bias,
@@ -1002,23 +955,15 @@ static int run_forward_single(const void *x, const void *wg, int dtype, int fp32
     if (rounds > 4) return 2;
     const int groups = (samples + 16 * rounds - 1) / (16 * rounds);
     if (groups > FS_MAX_GROUPS) return 2;
-#define PM_FS_ARGS rounds, groups, st, x, wg, logit_bias, samples, experts, k, normalize_gate, capacity, indices, \
-                   locations, gates, stride, logits_out, scores_out, l_aux, counts, codes, bias, scale, workspace,   \
-                   spin_limit, gave_up
-#define PM_FS_M(NMMA)                                                                                               \
-    do {                                                                                                           \
-        if (fp32_gate) return experts <= 8 ? launch_single<PLANMOE_F32, 8, NMMA>(PM_FS_ARGS)                         \
-                                           : launch_single<PLANMOE_F32, 16, NMMA>(PM_FS_ARGS);                       \
-        return experts <= 8 ? launch_single<PLANMOE_BF16, 8, NMMA>(PM_FS_ARGS) : launch_single<PLANMOE_BF16, 16, NMMA>(PM_FS_ARGS); \
-    } while (0)
+    const FsLaunch a{rounds, groups, st, x, wg, logit_bias, samples, experts, k, normalize_gate, capacity, indices,
+                     locations, gates, stride, logits_out, scores_out, l_aux, counts, codes, bias, scale, workspace,
+                     process_salt(), spin_limit, gave_up, fp32_gate};
     switch (model_dim) {                        // rows of 256 NMMA values: every wave owns an eighth of a row
-    case 1024: PM_FS_M(4);
-    case 2048: PM_FS_M(8);
-    case 3072: PM_FS_M(12);
-    default: PM_FS_M(16);
+    case 1024: return fs_launch_m4(a);
+    case 2048: return fs_launch_m8(a);
+    case 3072: return fs_launch_m12(a);
+    default: return fs_launch_m16(a);
     }
-#undef PM_FS_M
-#undef PM_FS_ARGS
 }
 
 } // namespace pm
