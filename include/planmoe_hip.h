@@ -276,8 +276,8 @@ int planmoe_forward_int8(const void *x, const void *wg, int dtype, int fp32_gate
  * of a second choice needs the first-choice counts of the whole batch).  One work-group per compute
  * unit holds the codes of its tokens on chip (LDS and registers) until every work-group has
  * published its expert histogram, then writes them to their slots.  Served shapes: bf16, model_dim
- * 1024, 2048, 3072 or 4096, experts <= 16, top_k <= 4, samples <= 64 x the number of compute units; any other shape is
- * an error here (planmoe_forward_int8 picks between the two on its own).  Outputs as
+ * a multiple of 256 up to 4096, experts <= 16, top_k <= 4, samples <= 64 x the number of compute
+ * units; any other shape is an error here (planmoe_forward_int8 picks between the two on its own).  Outputs as
  * planmoe_forward_int8 (logits may differ from it in the last bit: another summation order).
  * The wait between the work-groups is bounded: spin_limit polls (0 = the default, about a second);
  * a work-group that gives up writes none of its rows, marks its tokens dropped (locations =

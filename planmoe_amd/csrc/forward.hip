@@ -929,12 +929,13 @@ static void single_order_after(SingleOrder &order, hipStream_t st, bool ordered)
 }
 
 #ifdef PM_FS_TRACE
-// measurement build: the one-launch kernel's four translation units folded into this one, so that its
-// stamps and the ceiling kernels' land in one array
-PM_FS_DEFINE(4)
-PM_FS_DEFINE(8)
-PM_FS_DEFINE(12)
+// measurement build: the stamps of the one-launch kernel and of the ceiling kernels land in one array, so
+// the kernel is instantiated in this translation unit, for rows of 4096 values only (what is measured)
 PM_FS_DEFINE(16)
+#define PM_FS_ABSENT(n) int fs_launch_m##n(const FsLaunch &) { return 2; }
+PM_FS_ABSENT(1) PM_FS_ABSENT(2) PM_FS_ABSENT(3) PM_FS_ABSENT(4) PM_FS_ABSENT(5) PM_FS_ABSENT(6) PM_FS_ABSENT(7) PM_FS_ABSENT(8)
+PM_FS_ABSENT(9) PM_FS_ABSENT(10) PM_FS_ABSENT(11) PM_FS_ABSENT(12) PM_FS_ABSENT(13) PM_FS_ABSENT(14) PM_FS_ABSENT(15)
+#undef PM_FS_ABSENT
 #endif
 
 // 0: launched; 2: the shape is not served by the one-launch kernel (nothing was enqueued)
@@ -945,7 +946,7 @@ static int run_forward_single(const void *x, const void *wg, int dtype, int fp32
                               void *scale, void *workspace, int spin_limit, int32_t *gave_up, hipStream_t st)
 {
     const int k = top_k < experts ? top_k : experts;
-    if (dtype != PLANMOE_BF16 || model_dim % 1024 != 0 || model_dim > 4096 || experts > 16 || k > 4 || samples < 1) return 2;
+    if (dtype != PLANMOE_BF16 || model_dim % 256 != 0 || model_dim < 256 || model_dim > 4096 || experts > 16 || k > 4 || samples < 1) return 2;
     if (!aligned16(codes) && capacity > 0) return 2;
     int cus = 0, dev = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -958,12 +959,11 @@ static int run_forward_single(const void *x, const void *wg, int dtype, int fp32
     const FsLaunch a{rounds, groups, st, x, wg, logit_bias, samples, experts, k, normalize_gate, capacity, indices,
                      locations, gates, stride, logits_out, scores_out, l_aux, counts, codes, bias, scale, workspace,
                      process_salt(), spin_limit, gave_up, fp32_gate};
-    switch (model_dim) {                        // rows of 256 NMMA values: every wave owns an eighth of a row
-    case 1024: return fs_launch_m4(a);
-    case 2048: return fs_launch_m8(a);
-    case 3072: return fs_launch_m12(a);
-    default: return fs_launch_m16(a);
-    }
+    // rows of 256 NMMA values: every wave owns an eighth of a row
+    static int (*const launch[16])(const FsLaunch &) = {
+        fs_launch_m1, fs_launch_m2, fs_launch_m3, fs_launch_m4, fs_launch_m5, fs_launch_m6, fs_launch_m7, fs_launch_m8,
+        fs_launch_m9, fs_launch_m10, fs_launch_m11, fs_launch_m12, fs_launch_m13, fs_launch_m14, fs_launch_m15, fs_launch_m16};
+    return launch[model_dim / 256 - 1](a);
 }
 
 } // namespace pm
@@ -1092,7 +1092,7 @@ extern "C" int planmoe_forward_int8_single(const void *x, const void *wg, int dt
                                       spin_limit > 0 ? spin_limit : (1 << 20), gave_up, st);
     if (rc == 0) single_order_after(order, st, ordered);
     hold.unlock();
-    PM_REQUIRE(rc != 2, "planmoe_forward_int8_single: the one-launch kernel serves bf16 rows of 1024, 2048, 3072 or 4096 values, up to 16 "
+    PM_REQUIRE(rc != 2, "planmoe_forward_int8_single: the one-launch kernel serves bf16 rows of 256 to 4096 values in steps of 256, up to 16 "
                "experts, top_k <= 4 and at most 64 tokens per compute unit; use planmoe_forward_int8");
     PM_LAUNCH_CHECK("planmoe_forward_int8_single");
     return rc;

@@ -65,7 +65,10 @@ template <int NMMA> struct FsGeom {
     static constexpr int NV = M / 8;              // 16-byte vectors per row
     static constexpr int RS = M + 16;             // bytes per parked code row in LDS: lanes of different
                                                   // rows fall into different banks
-    static constexpr int RV = M / 16 / WAVE;      // 16-byte pieces of a code row per lane
+    static constexpr int PIECES = M / 16;         // 16-byte pieces of a code row
+    static constexpr int RV = (PIECES + WAVE - 1) / WAVE;          // ... per lane (a wave stores a whole row)
+    // piece i of this lane exists (rows whose length is no multiple of 1024 end inside the last pass)
+    static __device__ __forceinline__ bool piece(int i, int lane) { return PIECES % WAVE == 0 || i * WAVE + lane < PIECES; }
 };
 
 // four 8-bit counts -> four 16-bit fields (sums over up to 512 groups of counts up to 64 fit)
@@ -90,7 +93,7 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
     using G = FsGeom<NMMA>;
     static_assert(CAP == 8 || CAP == 16, "experts per token tile");
     static_assert(ROUNDS >= 1 && ROUNDS <= 4, "one lane per token in the ranking step");
-    static_assert(NMMA % 4 == 0 && G::RV >= 1, "rows are dealt out in 16-byte pieces");
+    static_assert(NMMA >= 1 && NMMA <= 16, "a lane holds NMMA 16-byte vectors of each of its rows");
     constexpr int TOK = 16 * ROUNDS;
     constexpr int REG_ROUNDS = ROUNDS < 2 ? ROUNDS : 2;    // the last rounds keep their codes in registers
     constexpr int LDS_ROUNDS = ROUNDS - REG_ROUNDS;        // the first rounds park theirs in LDS
@@ -433,14 +436,14 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
         uint4 v[G::RV];
         const uint4 *src = reinterpret_cast<const uint4 *>(park + prow * G::RS) + lane;
 #pragma unroll
-        for (int i = 0; i < G::RV; ++i) v[i] = src[i * WAVE];
+        for (int i = 0; i < G::RV; ++i) v[i] = G::piece(i, lane) ? src[i * WAVE] : make_uint4(0u, 0u, 0u, 0u);
         if (slot >= 0) { B16::store(bias_out, slot, s_mn[tok]); B16::store(scale_out, slot, s_sc[tok]); }
         for (int j = 0; j < k; ++j) {
             const int s = rl_i(slot, j);
             if (s < 0) continue;
             uint4 *dst = reinterpret_cast<uint4 *>(codes + (int64_t)s * G::M) + lane;
 #pragma unroll
-            for (int i = 0; i < G::RV; ++i) stream_store(dst + i * WAVE, v[i]);
+            for (int i = 0; i < G::RV; ++i) if (G::piece(i, lane)) stream_store(dst + i * WAVE, v[i]);
         }
     };
 
@@ -500,7 +503,7 @@ __global__ __launch_bounds__(FS_THREADS) void forward_single_kernel(
             const int slot = e * capacity + __builtin_amdgcn_readlane(z_used, e) + (int)(idx - (uint32_t)__builtin_amdgcn_readlane(z_beg, e));
             uint4 *dst = reinterpret_cast<uint4 *>(codes + (int64_t)slot * G::M) + lane;
 #pragma unroll
-            for (int i = 0; i < G::RV; ++i) stream_store(dst + i * WAVE, make_uint4(0u, 0u, 0u, 0u));
+            for (int i = 0; i < G::RV; ++i) if (G::piece(i, lane)) stream_store(dst + i * WAVE, make_uint4(0u, 0u, 0u, 0u));
             if (lane == 0) { B16::store(bias_out, slot, 0.f); B16::store(scale_out, slot, 0.f); }
         };
         const uint32_t total = (uint32_t)__builtin_amdgcn_readlane(z_upto, CAP - 1);

@@ -1,8 +1,8 @@
-// Host side of the one-launch forward kernel.  The kernel is instantiated for four row lengths (NMMA =
-// model_dim / 256), two score dtypes, two expert bounds and one to four rounds of 16 tokens: 64 kernels,
-// two thirds of the library's compile time.  So each row length is a translation unit of its own
-// (forward_single_m.hip, compiled once per NMMA) that exports one function, fs_launch_m<NMMA>, and the
-// four compile side by side; forward.hip picks the function by model_dim.
+// Host side of the one-launch forward kernel.  The kernel is instantiated for sixteen row lengths (NMMA =
+// model_dim / 256 = 1 .. 16), two score dtypes, two expert bounds and one to four rounds of 16 tokens: 256
+// kernels, most of the library's compile time.  So each row length is a translation unit of its own
+// (forward_single_m.hip, compiled once per NMMA) that exports one function, fs_launch_m<NMMA>, and they
+// compile side by side; forward.hip picks the function by model_dim.
 #pragma once
 #include "forward_single.hpp"
 
@@ -29,10 +29,10 @@ struct FsLaunch {
 };
 
 // 0: launched; 2: more work-groups than are resident at once (nothing was enqueued)
-int fs_launch_m4(const FsLaunch &a);
-int fs_launch_m8(const FsLaunch &a);
-int fs_launch_m12(const FsLaunch &a);
-int fs_launch_m16(const FsLaunch &a);
+#define PM_FS_DECLARE(n) int fs_launch_m##n(const FsLaunch &a);
+PM_FS_DECLARE(1) PM_FS_DECLARE(2) PM_FS_DECLARE(3) PM_FS_DECLARE(4) PM_FS_DECLARE(5) PM_FS_DECLARE(6) PM_FS_DECLARE(7) PM_FS_DECLARE(8)
+PM_FS_DECLARE(9) PM_FS_DECLARE(10) PM_FS_DECLARE(11) PM_FS_DECLARE(12) PM_FS_DECLARE(13) PM_FS_DECLARE(14) PM_FS_DECLARE(15) PM_FS_DECLARE(16)
+#undef PM_FS_DECLARE
 
 // Whether every work-group of the launch is resident at once (asked of the runtime once per kernel and device).
 template <int SDT, int CAP, int NMMA, int ROUNDS>

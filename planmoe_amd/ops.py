@@ -452,9 +452,9 @@ def forward_plain(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, norm
 
 
 def forward_int8_single_serves(x, wg, top_k):
-    """The shapes planmoe_forward_int8_single takes: bf16 rows of 1024, 2048, 3072 or 4096 values, up to
+    """The shapes planmoe_forward_int8_single takes: bf16 rows of 256 to 4096 values in steps of 256, up to
     16 experts, top_k <= 4, at most 64 tokens per compute unit."""
-    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.shape[1] in (1024, 2048, 3072, 4096) and
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.shape[1] % 256 == 0 and 256 <= x.shape[1] <= 4096 and
             x.shape[0] >= 1):
         return False
     cus = torch.cuda.get_device_properties(x.device).multi_processor_count
@@ -463,7 +463,7 @@ def forward_int8_single_serves(x, wg, top_k):
 
 def forward_int8_single(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
                         want_logits=False, want_scores=False, want_l_aux=True, want_counts=False, spin_limit=0):
-    """forward_int8 in one launch that reads x once (bf16 rows of 1024 / 2048 / 3072 / 4096 values, up to 16 experts,
+    """forward_int8 in one launch that reads x once (bf16 rows of 256 .. 4096 values in steps of 256, up to 16 experts,
     top_k <= 4, at most 64 tokens per compute unit; anything else raises).  Adds `gave_up`, a device
     int32 that is 1 when a work-group ran out of `spin_limit` polls waiting for the others."""
     x, wg, T, M, E, k, bias, out, ws = _forward_common(x, wg, top_k, fp32_gate, logit_bias, want_logits,

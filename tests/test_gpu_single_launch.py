@@ -51,9 +51,14 @@ def test_single_launch_forward(T, E, k, cf, fp32_gate, M=4096):
 @pytest.mark.parametrize("T,M,E,k,cf,fp32_gate", [(16384, 2048, 8, 2, 1.25, True), (9000, 2048, 16, 3, 0.5, False),
                                                   (16384, 1024, 8, 2, 1.25, True), (5000, 1024, 4, 1, 1.0, True),
                                                   (12000, 3072, 8, 2, 1.25, True), (100, 3072, 12, 4, 2.0, False),
-                                                  (1, 2048, 3, 2, 1.0, True)])
+                                                  (1, 2048, 3, 2, 1.0, True),
+                                                  # rows that end inside a wave's last pass over the codes
+                                                  (16384, 768, 8, 2, 1.25, True), (7000, 1280, 16, 2, 1.0, False),
+                                                  (16000, 2560, 8, 2, 1.25, True), (9000, 3584, 6, 3, 1.0, True),
+                                                  (3000, 256, 4, 2, 1.0, True), (12345, 1792, 8, 1, 1.5, False),
+                                                  (500, 3840, 16, 4, 2.0, True), (16384, 512, 8, 2, 1.25, True)])
 def test_single_launch_forward_other_row_lengths(T, M, E, k, cf, fp32_gate):
-    """The one-launch kernel at rows of 1024, 2048 and 3072 values: the same checks against the oracle."""
+    """The one-launch kernel at other row lengths (multiples of 256 values): the same checks against the oracle."""
     test_single_launch_forward(T, E, k, cf, fp32_gate, M)
 
 
