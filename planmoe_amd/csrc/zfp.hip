@@ -44,7 +44,9 @@ struct BitWriter {
 // The decoder looks at the stream by bit position: the block's words sit in LDS (NW words per
 // thread and three zero words behind them: an odd stride) and a look is neighbouring words
 // funnel-shifted, so there is no refill state to carry and no branch in the reader.  A bit plane
-// takes one look of 64 bits (a plane never uses more than 48) and is then parsed in registers.
+// takes one look of 64 bits (a plane never uses more than 48) and is then parsed in registers: the
+// group tests of a 2-D block eight stream bits at a time by table (gt16_step), except the plane the
+// block's budget ends in, which is walked bit by bit.
 // Streams of one or two words stay in a register pair that is shifted as bits are consumed.
 template <int NW>
 struct BitReader {
@@ -277,8 +279,119 @@ __device__ __forceinline__ void encode_block(const float *f, BitWriter<NW> &bw, 
     bw.finish();
 }
 
+// ---- group tests of a 2-D block's bit plane, eight stream bits at a time
+// The group-test bits of a plane are a walk with two states: a test bit is due (T), or the zeros of
+// a run up to the next one bit are being read (R).  What eight stream bits do to that walk depends
+// on the state and on how far away the block's last value is (its one is implied, and after it the
+// plane ends without another test bit).  gt16_step works that out once per (state, distance, byte):
+// bits 0..7 the one bits found (relative to the first value that was not significant), bits 8..11
+// the values passed, bits 12..15 a code c: c <= 8 = the plane ended after c bits; 9 / 10 = all eight
+// bits used and the walk goes on in state T / R.  The walk is zfp's own (decode_ints), minus the
+// budget: a step that would use up the budget is not taken, see fast_plane16.
+__host__ __device__ constexpr uint16_t gt16_step(int state, int r, uint32_t byte)
+{
+    const int last = r < 8 ? r : 99;            // the block's last value, if this step can reach it
+    int n = 0, used = 0, st = state;
+    uint32_t mask = 0;
+    bool done = false;
+    while (true) {
+        if (st == 0) {
+            if (n > last) { done = true; break; }
+            if (used == 8) break;
+            const uint32_t b = (byte >> used) & 1u; ++used;
+            if (!b) { done = true; break; }
+            st = 1;
+        }
+        bool out_of_bits = false;
+        while (n != last) {
+            if (used == 8) { out_of_bits = true; break; }
+            const uint32_t b = (byte >> used) & 1u; ++used;
+            if (b) break;
+            ++n;
+        }
+        if (out_of_bits) break;
+        mask |= 1u << n; ++n; st = 0;
+        if (n > last) { done = true; break; }
+    }
+    const int c = done ? used : (st ? 10 : 9);
+    return (uint16_t)(mask | ((uint32_t)n << 8) | ((uint32_t)c << 12));
+}
+constexpr int GT16_ENTRIES = 9 * 2 * 256;      // [min(15 - nsig, 8)][state][byte]
+struct Gt16Table {
+    uint16_t step[GT16_ENTRIES];
+    constexpr Gt16Table() : step()
+    {
+        for (int i = 0; i < GT16_ENTRIES; ++i) step[i] = gt16_step((i >> 8) & 1, i >> 9, (uint32_t)i & 255u);
+    }
+};
+__constant__ const Gt16Table gt16_table = Gt16Table();
+
+// all 256 threads of the work-group copy the table into LDS (9 KB); a barrier follows
+__device__ __forceinline__ void gt16_load(uint16_t *tab)
+{
+    const uint32_t *src = reinterpret_cast<const uint32_t *>(gt16_table.step);
+    uint32_t *dst = reinterpret_cast<uint32_t *>(tab);
+#pragma unroll
+    for (int i = 0; i < GT16_ENTRIES / 2 / 256; ++i) dst[threadIdx.x + 256 * i] = src[threadIdx.x + 256 * i];
+    __syncthreads();
+}
+
+// One bit plane of a 2-D block, bit by bit as zfp walks it: look = the next 64 stream bits (a plane
+// never uses more than 48), bits = what is left of the block's budget, nsig = values significant so
+// far.  nsig verbatim bits, then segment by segment the test bit and the zeros up to the next one
+// bit (cut short by the budget or by the block's last value, whose one is implied).
+__device__ __forceinline__ uint32_t slow_plane16(uint64_t look, int &bits, int &nsig)
+{
+    constexpr int N = 16;
+    const int mm = min(nsig, bits);
+    bits -= mm;
+    uint32_t x = (uint32_t)look & ((1u << mm) - 1u);
+    look >>= mm;
+    while (nsig < N && bits > 0) {
+        const uint32_t lo = (uint32_t)look;
+        if (!(lo & 1u)) { --bits; break; }
+        const int lim = min(N - 1 - nsig, bits - 1);
+        const uint32_t win = (lo >> 1) & ((1u << lim) - 1u);
+        const int z = win != 0u ? __builtin_ctz(win) : lim;       // zeros read
+        const int used = 1 + (win != 0u ? z + 1 : lim);
+        look >>= used; bits -= used; nsig += z;
+        x |= 1u << nsig;
+        ++nsig;
+    }
+    return x;
+}
+
+// The same plane by table, as long as the budget does not end inside it: false = it would (bits and
+// nsig are then whatever the walk left them at: the caller keeps its own copies and has
+// slow_plane16 do that plane, the block's last).  One exit and selects instead of branches: the
+// lanes of a wave are at different points of their walks.
+__device__ __forceinline__ bool fast_plane16(uint64_t look, int &bits, int &nsig, uint32_t &x, const uint16_t *tab)
+{
+    const int mm = min(nsig, bits);
+    bits -= mm;
+    x = (uint32_t)look & ((1u << mm) - 1u);
+    look >>= mm;
+    bool over = false, go = nsig < 16 && bits > 0;
+    uint32_t st = 0u;                          // state * 256
+    while (go) {
+        const uint32_t r = (uint32_t)min(15 - nsig, 8);
+        const uint32_t e = tab[(r << 9) | st | ((uint32_t)look & 255u)];
+        const uint32_t c = e >> 12;
+        const int used = (int)min(c, 8u);
+        over = used >= bits;
+        const int u = over ? 0 : used;
+        x |= (over ? 0u : (e & 255u)) << nsig;
+        nsig += over ? 0 : (int)((e >> 8) & 15u);
+        look >>= u; bits -= u;
+        st = (c & 1u) ? 0u : 256u;             // c = 9: state T, c = 10: state R (other values end the walk)
+        go = !over && c >= 9u;
+    }
+    return !over;
+}
+
+// tab: the group-test table in LDS (gt16_load), used by 2-D blocks only
 template <int N, int NW>
-__device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f)
+__device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f, const uint16_t *tab = nullptr)
 {
     if (!br.get(1)) {
 #pragma unroll
@@ -310,26 +423,9 @@ __device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f)
             }
             return x;
         } else {
-            // one look at the stream per plane: nsig verbatim bits, then segment by segment the test
-            // bit and the zeros up to the next one bit (cut short by the budget or by the block's
-            // last value, whose one is implied), at most 16 + 32 bits in all
-            uint64_t look = br.peek64();
+            // one look at the stream per plane
             const int before = bits;
-            const int mm = min(nsig, bits);
-            bits -= mm;
-            uint32_t x = (uint32_t)look & ((1u << mm) - 1u);
-            look >>= mm;
-            while (nsig < N && bits > 0) {
-                const uint32_t lo = (uint32_t)look;
-                if (!(lo & 1u)) { --bits; break; }
-                const int lim = min(N - 1 - nsig, bits - 1);
-                const uint32_t win = (lo >> 1) & ((1u << lim) - 1u);
-                const int z = win != 0u ? __builtin_ctz(win) : lim;       // zeros read
-                const int used = 1 + (win != 0u ? z + 1 : lim);
-                look >>= used; bits -= used; nsig += z;
-                x |= 1u << nsig;
-                ++nsig;
-            }
+            const uint32_t x = slow_plane16(br.peek64(), bits, nsig);
             br.skip(before - bits);
             return x;
         }
@@ -339,9 +435,32 @@ __device__ __forceinline__ void decode_block(BitReader<NW> &br, float *f)
         uint32_t w[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) w[j] = 0u;
+        // by table, up to the plane the budget ends in: that one is set aside (every lane has one, each
+        // at a plane of its own) and walked bit by bit afterwards, by all lanes at once
+        int last_k = -1, last_bits = 0, last_nsig = 0;
+        uint64_t last_look = 0;
 #pragma unroll
-        for (int k = 15; k >= 0; --k)
-            if (bits > 0) w[k >> 1] |= read_plane() << (16 * (k & 1));
+        for (int k = 15; k >= 0; --k) {
+            // (a branch of the whole wave; a lane whose budget is spent walks a plane of no bits)
+            if (__builtin_amdgcn_ballot_w64(bits > 0) != 0) {
+                const uint64_t look = br.peek64();
+                const int before = bits, nsig0 = nsig;
+                uint32_t x;
+                const bool ok = fast_plane16(look, bits, nsig, x, tab);
+                br.skip(ok ? before - bits : 0);
+                w[k >> 1] |= ok ? x << (16 * (k & 1)) : 0u;
+                last_k = ok ? last_k : k;
+                last_look = ok ? last_look : look;
+                last_bits = ok ? last_bits : before;
+                last_nsig = ok ? last_nsig : nsig0;
+                bits = ok ? bits : 0;
+            }
+        }
+        if (last_k >= 0) {
+            const uint32_t x = slow_plane16(last_look, last_bits, last_nsig) << (16 * (last_k & 1));
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w[j] |= (last_k >> 1) == j ? x : 0u;
+        }
         transpose16(w);
 #pragma unroll
         for (int j = 0; j < 8; ++j) { u[2 * j] = w[j] << 16; u[2 * j + 1] = w[j] & 0xffff0000u; }
@@ -663,25 +782,33 @@ __global__ __launch_bounds__(256) void zfp_encode2_kernel(const float *__restric
     store_words<NW>(out + b * NW, w);
 }
 
+// blocks per thread: the group-test table (9 KB) is copied into LDS once per work-group
+constexpr int ZD2_PER_THREAD = 4;
+
 template <int NW>
 __global__ __launch_bounds__(256) void zfp_decode2_kernel(const uint32_t *__restrict__ in, int64_t nx,
                                                           int64_t nbx, int64_t blocks,
                                                           float *__restrict__ field)
 {
-    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (b >= blocks) return;
     __shared__ uint32_t lds[NW <= 2 ? 1 : BitReader<NW>::STRIDE * 256];
-    uint32_t w[NW];
-    load_words<NW>(in + b * NW, w);
-    BitReader<NW> br;
-    br.init(lds, w);
-    float f[16];
-    decode_block<16, NW>(br, f);
-    const int64_t by = b / nbx, bx = b - by * nbx;
-    float *p = field + 4 * by * nx + 4 * bx;
+    __shared__ uint16_t tab[GT16_ENTRIES];
+    gt16_load(tab);
+    const int64_t b0 = (int64_t)blockIdx.x * (256 * ZD2_PER_THREAD) + threadIdx.x;
+    for (int it = 0; it < ZD2_PER_THREAD; ++it) {
+        const int64_t b = b0 + 256 * it;
+        if (b >= blocks) break;
+        uint32_t w[NW];
+        load_words<NW>(in + b * NW, w);
+        BitReader<NW> br;
+        br.init(lds, w);
+        float f[16];
+        decode_block<16, NW>(br, f, tab);
+        const int64_t by = b / nbx, bx = b - by * nbx;
+        float *p = field + 4 * by * nx + 4 * bx;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-        *reinterpret_cast<float4 *>(p + j * nx) = make_float4(f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]);
+        for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<float4 *>(p + j * nx) = make_float4(f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]);
+    }
 }
 
 // ---------------------------------------------------------------- dispatch fused with the 2-D encoder
@@ -766,16 +893,22 @@ __global__ __launch_bounds__(256) void combine_zfp2_kernel(const uint32_t *__res
                                                           int64_t model_dim, int64_t nbx, int64_t blocks,
                                                           float *__restrict__ out)
 {
-    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (b >= blocks) return;
+    // (one block per thread: with four, so that the table is copied once per 1024 blocks, the launch
+    // takes 10 % longer: half the work-groups leave early and the rest run four times as long)
     __shared__ uint32_t lds[NW <= 2 ? 1 : BitReader<NW>::STRIDE * 256];
-    const int64_t by = b / nbx, bx = b - by * nbx;
+    __shared__ uint16_t tab[GT16_ENTRIES];
+    const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool in_field = b < blocks;
+    const int64_t by = (in_field ? b : blocks - 1) / nbx, bx = b - by * nbx;
     const int4 tok = *reinterpret_cast<const int4 *>(src + 4 * by);
     const int4 pl = *reinterpret_cast<const int4 *>(splane + 4 * by);
     const int t[4] = {tok.x, tok.y, tok.z, tok.w};
-    const bool mine[4] = {tok.x >= 0 && pl.x == plane, tok.y >= 0 && pl.y == plane,
-                          tok.z >= 0 && pl.z == plane, tok.w >= 0 && pl.w == plane};
-    if (!(mine[0] || mine[1] || mine[2] || mine[3])) return;
+    const bool mine[4] = {in_field && tok.x >= 0 && pl.x == plane, in_field && tok.y >= 0 && pl.y == plane,
+                          in_field && tok.z >= 0 && pl.z == plane, in_field && tok.w >= 0 && pl.w == plane};
+    const bool any_mine = mine[0] || mine[1] || mine[2] || mine[3];
+    if (!__syncthreads_or(any_mine)) return;          // a work-group without a row of this plane leaves before the table
+    gt16_load(tab);
+    if (!any_mine) return;
     float g[4] = {1.f, 1.f, 1.f, 1.f};
     if (sgate) {
         const float4 gv = *reinterpret_cast<const float4 *>(sgate + 4 * by);
@@ -793,7 +926,7 @@ __global__ __launch_bounds__(256) void combine_zfp2_kernel(const uint32_t *__res
     BitReader<NW> br;
     br.init(lds, w);
     float f[16];
-    decode_block<16, NW>(br, f);
+    decode_block<16, NW>(br, f, tab);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         if (!mine[j]) continue;
@@ -819,10 +952,12 @@ __global__ __launch_bounds__(256) void bwd_gate_zfp2_kernel(const uint32_t *__re
 {
     __shared__ uint32_t lds[NW <= 2 ? 1 : BitReader<NW>::STRIDE * 256];
     __shared__ float s_part[4][4];
+    __shared__ uint16_t tab[GT16_ENTRIES];
     const int64_t by = blockIdx.x;
     const int4 tok = *reinterpret_cast<const int4 *>(src + 4 * by);
     const int t[4] = {tok.x, tok.y, tok.z, tok.w};
     if (t[0] < 0 && t[1] < 0 && t[2] < 0 && t[3] < 0) return;        // four empty slots (the whole work-group leaves)
+    gt16_load(tab);
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     for (int64_t bx0 = 0; bx0 < nbx; bx0 += 256) {
         const int64_t bx = bx0 + threadIdx.x;
@@ -837,7 +972,7 @@ __global__ __launch_bounds__(256) void bwd_gate_zfp2_kernel(const uint32_t *__re
         BitReader<NW> br;
         br.init(lds, w);
         float f[16];
-        decode_block<16, NW>(br, f);
+        decode_block<16, NW>(br, f, tab);
         if (in_row) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
@@ -980,7 +1115,8 @@ extern "C" int planmoe_zfp_decompress(const void *stream_in, int dims, int64_t n
     }
     PM_NW_SWITCH(nw, NW, {
         if (dims == 1) zfp_decode1_kernel<NW><<<grid, 256, 0, st>>>((const uint32_t *)stream_in, blocks, field);
-        else zfp_decode2_kernel<NW><<<grid, 256, 0, st>>>((const uint32_t *)stream_in, nx, nx / 4, blocks, field);
+        else zfp_decode2_kernel<NW><<<(unsigned)((blocks + 256 * ZD2_PER_THREAD - 1) / (256 * ZD2_PER_THREAD)), 256, 0, st>>>(
+                 (const uint32_t *)stream_in, nx, nx / 4, blocks, field);
     });
     PM_LAUNCH_CHECK("planmoe_zfp_decompress");
     return 0;
