@@ -216,6 +216,32 @@ def _config5_field(rows, nx, seed=0):
     return (v / v.std()).contiguous()
 
 
+@pytest.mark.parametrize("rate", [2, 4, 8, 16])
+def test_zfp_2d_field_kinds_and_rates(rate):
+    """The 2-D coder at every block size it is built for, on fields that take the decoder's group-test
+    walk through long zero runs, the block's last value, budgets that end in a run, all-zero blocks
+    and planes below the sixteenth: streams and decoded fields against the oracle, bit for bit."""
+    from planmoe_amd import ops
+    rng = np.random.default_rng(3 + rate)
+    ny, nx = 64, 512
+    fields = {
+        "gauss": rng.standard_normal((ny, nx)),
+        "smooth": np.sin(np.arange(nx) / 37.0)[None, :] * np.cos(np.arange(ny) / 11.0)[:, None],
+        "tiny": rng.standard_normal((ny, nx)) * 1e-30,
+        "sparse": rng.standard_normal((ny, nx)) * (rng.random((ny, nx)) < 0.05),
+        "spiky": rng.standard_normal((ny, nx)) * 10.0 ** rng.integers(-6, 6, (ny, nx)),
+        "const": np.full((ny, nx), 3.25),
+    }
+    for name, f in fields.items():
+        f = f.astype(np.float32)
+        st = oracle.zfp_compress(f, 2, float(rate))
+        want = oracle.zfp_decompress(st, ny, nx, 2, float(rate))
+        got = ops.zfp_compress(torch.from_numpy(f).to(DEV), nx, ny, 2, float(rate)).cpu().numpy()
+        assert np.array_equal(got[:len(st)], st), name
+        dec = ops.zfp_decompress(torch.from_numpy(np.concatenate([st, np.zeros(16, np.uint8)])).to(DEV), nx, ny, 2, float(rate))
+        assert np.array_equal(dec.cpu().numpy().view(np.uint32), want.view(np.uint32)), name
+
+
 @pytest.mark.parametrize("dims", [2, 1])
 def test_zfp_config5_full_size(dims):
     """[16, 8192, 1024] fp32 (65536 tokens x top-2 slots): whole stream against the oracle."""
