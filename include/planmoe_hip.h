@@ -276,8 +276,9 @@ int planmoe_forward_int8(const void *x, const void *wg, int dtype, int fp32_gate
  * of a second choice needs the first-choice counts of the whole batch).  One work-group per compute
  * unit holds the codes of its tokens on chip (LDS and registers) until every work-group has
  * published its expert histogram, then writes them to their slots.  Served shapes: bf16, model_dim
- * a multiple of 256 up to 4096, experts <= 16, top_k <= 4, samples <= 64 x the number of compute
- * units; any other shape is an error here (planmoe_forward_int8 picks between the two on its own).  Outputs as
+ * a multiple of 256 up to 4096, experts <= 16, top_k <= 4, samples <= 64 x the number of work-groups
+ * that are resident at once (one per compute unit, two for rows of up to 1792 values:
+ * planmoe_forward_int8_single_serves tells); any other shape is an error here (planmoe_forward_int8 picks between the two on its own).  Outputs as
  * planmoe_forward_int8 (logits may differ from it in the last bit: another summation order).
  * The wait between the work-groups is bounded: spin_limit polls (0 = the default, about a second);
  * a work-group that gives up writes none of its rows, marks its tokens dropped (locations =
@@ -300,6 +301,13 @@ int planmoe_forward_int8_single(const void *x, const void *wg, int dtype, int fp
                                 int32_t *expert_counts, uint8_t *codes, void *bias, void *scale,
                                 void *workspace, size_t workspace_bytes, int spin_limit,
                                 int32_t *gave_up, void *stream);
+
+/* 1 if planmoe_forward_int8_single takes the shape on the current device, else 0: the limits above,
+ * and every work-group of the launch resident at once (work-groups of at most 64 tokens; rows of up
+ * to 1792 values leave room for two of them per compute unit, so twice the tokens).  Asks the
+ * runtime once per kernel and device; launches nothing.  No counterpart in the reference: for
+ * callers that pick between the two forward entry points (the Python layer does). */
+int planmoe_forward_int8_single_serves(int dtype, int fp32_gate, int samples, int model_dim, int experts, int top_k);
 
 /* A measuring stick for planmoe_forward_int8_single, not a product path: one launch with that
  * kernel's grid, its loads of x, one exchange of tagged words between all work-groups and its

@@ -943,22 +943,24 @@ static int run_forward_single(const void *x, const void *wg, int dtype, int fp32
                               int samples, int model_dim, int experts, int top_k, int normalize_gate, int capacity,
                               int32_t *indices, int32_t *locations, void *gates, int64_t stride, void *logits_out,
                               void *scores_out, float *l_aux, int32_t *counts, uint8_t *codes, void *bias,
-                              void *scale, void *workspace, int spin_limit, int32_t *gave_up, hipStream_t st)
+                              void *scale, void *workspace, int spin_limit, int32_t *gave_up, hipStream_t st,
+                              bool ask_only = false)
 {
     const int k = top_k < experts ? top_k : experts;
     if (dtype != PLANMOE_BF16 || model_dim % 256 != 0 || model_dim < 256 || model_dim > 4096 || experts > 16 || k > 4 || samples < 1) return 2;
-    if (!aligned16(codes) && capacity > 0) return 2;
+    if (!ask_only && !aligned16(codes) && capacity > 0) return 2;
     int cus = 0, dev = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) return 2;
-    // as few tokens per work-group as it takes to put one work-group on every compute unit
-    const int rounds = (samples + 16 * cus - 1) / (16 * cus);
-    if (rounds > 4) return 2;
+    // as few tokens per work-group as it takes to put one work-group on every compute unit; beyond 64
+    // tokens per compute unit, work-groups of 64 tokens, which short rows allow two of per compute unit
+    // (the launch goes ahead only if the runtime says that all of them are resident at once)
+    const int rounds = min((samples + 16 * cus - 1) / (16 * cus), 4);
     const int groups = (samples + 16 * rounds - 1) / (16 * rounds);
     if (groups > FS_MAX_GROUPS) return 2;
     const FsLaunch a{rounds, groups, st, x, wg, logit_bias, samples, experts, k, normalize_gate, capacity, indices,
                      locations, gates, stride, logits_out, scores_out, l_aux, counts, codes, bias, scale, workspace,
-                     process_salt(), spin_limit, gave_up, fp32_gate};
+                     process_salt(), spin_limit, gave_up, fp32_gate, ask_only};
     // rows of 256 NMMA values: every wave owns an eighth of a row
     static int (*const launch[16])(const FsLaunch &) = {
         fs_launch_m1, fs_launch_m2, fs_launch_m3, fs_launch_m4, fs_launch_m5, fs_launch_m6, fs_launch_m7, fs_launch_m8,
@@ -1093,9 +1095,18 @@ extern "C" int planmoe_forward_int8_single(const void *x, const void *wg, int dt
     if (rc == 0) single_order_after(order, st, ordered);
     hold.unlock();
     PM_REQUIRE(rc != 2, "planmoe_forward_int8_single: the one-launch kernel serves bf16 rows of 256 to 4096 values in steps of 256, up to 16 "
-               "experts, top_k <= 4 and at most 64 tokens per compute unit; use planmoe_forward_int8");
+               "experts, top_k <= 4 and as many tokens as its work-groups of 64 hold while all resident at once "
+               "(planmoe_forward_int8_single_serves tells); use planmoe_forward_int8");
     PM_LAUNCH_CHECK("planmoe_forward_int8_single");
     return rc;
+}
+
+extern "C" int planmoe_forward_int8_single_serves(int dtype, int fp32_gate, int samples, int model_dim, int experts, int top_k)
+{
+    if (samples < 1 || model_dim < 1 || experts < 1 || top_k < 1) return 0;
+    return run_forward_single(nullptr, nullptr, dtype, fp32_gate, nullptr, samples, model_dim, experts, top_k, 1, 0,
+                              nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                              nullptr, nullptr, 0, nullptr, nullptr, true) == 0;
 }
 
 extern "C" int planmoe_forward_int8_single_ceiling(const void *x, int samples, int model_dim, int experts, int top_k,

@@ -26,9 +26,10 @@ struct FsLaunch {
     int spin_limit;
     int32_t *gave_up;
     int fp32_gate;
+    bool ask_only;          // do not launch: only say whether the launch would go ahead
 };
 
-// 0: launched; 2: more work-groups than are resident at once (nothing was enqueued)
+// 0: launched (or, with ask_only, would be); 2: more work-groups than are resident at once (nothing was enqueued)
 #define PM_FS_DECLARE(n) int fs_launch_m##n(const FsLaunch &a);
 PM_FS_DECLARE(1) PM_FS_DECLARE(2) PM_FS_DECLARE(3) PM_FS_DECLARE(4) PM_FS_DECLARE(5) PM_FS_DECLARE(6) PM_FS_DECLARE(7) PM_FS_DECLARE(8)
 PM_FS_DECLARE(9) PM_FS_DECLARE(10) PM_FS_DECLARE(11) PM_FS_DECLARE(12) PM_FS_DECLARE(13) PM_FS_DECLARE(14) PM_FS_DECLARE(15) PM_FS_DECLARE(16)
@@ -57,6 +58,7 @@ static int launch_single(const FsLaunch &a)
 #define PM_FS(ROUNDS)                                                                                              \
     do {                                                                                                           \
         if (!single_fits<SDT, CAP, NMMA, ROUNDS>(a.groups)) return 2;                                              \
+        if (a.ask_only) return 0;                                                                                  \
         forward_single_kernel<SDT, CAP, NMMA, ROUNDS><<<a.groups, FS_THREADS, 0, a.st>>>(                          \
             (const uint4 *)a.x, (const uint4 *)a.wg, a.bias, a.samples, a.experts, a.k, a.normalize, a.capacity,   \
             a.indices, a.locations, a.gates, a.stride, a.logits_out, a.scores_out, a.l_aux, a.counts, a.codes,     \

@@ -451,20 +451,21 @@ def forward_plain(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, norm
     return out
 
 
-def forward_int8_single_serves(x, wg, top_k):
+def forward_int8_single_serves(x, wg, top_k, fp32_gate=True):
     """The shapes planmoe_forward_int8_single takes: bf16 rows of 256 to 4096 values in steps of 256, up to
-    16 experts, top_k <= 4, at most 64 tokens per compute unit."""
-    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.shape[1] % 256 == 0 and 256 <= x.shape[1] <= 4096 and
-            x.shape[0] >= 1):
+    16 experts, top_k <= 4, and so few tokens that all its work-groups are resident at once (64 per compute
+    unit; 128 for rows of up to 1792 values).  The library is asked (planmoe_forward_int8_single_serves)."""
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.shape[0] >= 1):
         return False
-    cus = torch.cuda.get_device_properties(x.device).multi_processor_count
-    return wg.shape[0] <= 16 and min(int(top_k), wg.shape[0]) <= 4 and x.shape[0] <= 64 * cus
+    with torch.cuda.device(x.device):
+        return bool(lib.planmoe_forward_int8_single_serves(_dt(x, "forward_int8_single"), int(bool(fp32_gate)), x.shape[0],
+                                                           x.shape[1], wg.shape[0], int(top_k)))
 
 
 def forward_int8_single(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
                         want_logits=False, want_scores=False, want_l_aux=True, want_counts=False, spin_limit=0):
     """forward_int8 in one launch that reads x once (bf16 rows of 256 .. 4096 values in steps of 256, up to 16 experts,
-    top_k <= 4, at most 64 tokens per compute unit; anything else raises).  Adds `gave_up`, a device
+    top_k <= 4, as many tokens as forward_int8_single_serves allows; anything else raises).  Adds `gave_up`, a device
     int32 that is 1 when a work-group ran out of `spin_limit` polls waiting for the others."""
     x, wg, T, M, E, k, bias, out, ws = _forward_common(x, wg, top_k, fp32_gate, logit_bias, want_logits,
                                                        want_scores, want_l_aux, want_counts)

@@ -173,7 +173,7 @@ def forward_int8_send_side(x, w, top_k, capacity, fp32_gate, normalize_gate, sin
     the caller to ask later (and to run the pass again with single=False if it is set); without, the
     flag is read here and the two launches run in its place if need be.  Never hands out a partial
     result unchecked."""
-    if (single and FORWARD_SINGLE_LAUNCH and ops.forward_int8_single_serves(x, w, top_k) and
+    if (single and FORWARD_SINGLE_LAUNCH and ops.forward_int8_single_serves(x, w, top_k, fp32_gate) and
             not torch.cuda.is_current_stream_capturing()):
         out = ops.forward_int8_single(x, w, top_k, capacity, fp32_gate=fp32_gate, normalize_gate=normalize_gate, **want)
         flag = out.pop("gave_up")

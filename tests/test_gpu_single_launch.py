@@ -56,10 +56,39 @@ def test_single_launch_forward(T, E, k, cf, fp32_gate, M=4096):
                                                   (16384, 768, 8, 2, 1.25, True), (7000, 1280, 16, 2, 1.0, False),
                                                   (16000, 2560, 8, 2, 1.25, True), (9000, 3584, 6, 3, 1.0, True),
                                                   (3000, 256, 4, 2, 1.0, True), (12345, 1792, 8, 1, 1.5, False),
-                                                  (500, 3840, 16, 4, 2.0, True), (16384, 512, 8, 2, 1.25, True)])
+                                                  (500, 3840, 16, 4, 2.0, True), (16384, 512, 8, 2, 1.25, True),
+                                                  # two work-groups per compute unit: short rows, up to 128 tokens per unit
+                                                  (32768, 1024, 8, 2, 1.25, True), (30000, 1792, 8, 2, 1.0, False),
+                                                  (20000, 1536, 8, 3, 1.25, True)])
 def test_single_launch_forward_other_row_lengths(T, M, E, k, cf, fp32_gate):
     """The one-launch kernel at other row lengths (multiples of 256 values): the same checks against the oracle."""
     test_single_launch_forward(T, E, k, cf, fp32_gate, M)
+
+
+def test_the_library_says_which_shapes_the_single_launch_takes():
+    """planmoe_forward_int8_single_serves against what the entry point then does: it launches exactly the
+    shapes the query admits and refuses the others with an error (nothing enqueued)."""
+    from planmoe_amd import ops
+    from planmoe_amd._lib import PlanMoEError
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    cases = [(64 * cus, 4096, 8, 2, True), (64 * cus + 1, 4096, 8, 2, False), (128 * cus, 1024, 8, 2, True),
+             (128 * cus + 1, 1024, 8, 2, False), (100, 4352, 8, 2, False), (100, 1000, 8, 2, False),
+             (100, 1024, 17, 2, False), (100, 1024, 16, 5, False), (100, 1024, 3, 5, True), (1, 256, 1, 1, True)]
+    for T, M, E, k, want in cases:
+        print("case", T, M, E, k, flush=True)
+        x = torch.randn(T, M, device=DEV).bfloat16()
+        wg = (torch.randn(E, M, device=DEV) * M ** -0.5).bfloat16()
+        assert ops.forward_int8_single_serves(x, wg, k) == want
+        C = ops.capacity(T, E, k, 1.0, 4)
+        if want:
+            out = ops.forward_int8_single(x, wg, k, C)
+            ref = ops.forward_int8(x, wg, k, C)
+            torch.cuda.synchronize()
+            assert int(out["gave_up"]) == 0 and torch.equal(out["codes"], ref["codes"]) and torch.equal(out["locations"], ref["locations"])
+        else:
+            with pytest.raises(PlanMoEError):
+                ops.forward_int8_single(x, wg, k, C)
+    assert not ops.forward_int8_single_serves(torch.randn(64, 1024, device=DEV), torch.randn(8, 1024, device=DEV), 2)   # fp32 rows
 
 
 def test_single_launch_gives_up_cleanly_when_told_to():
