@@ -454,7 +454,8 @@ __global__ __launch_bounds__(LZ_WAVES * WAVE) void lz_place_kernel(
         *reinterpret_cast<uint16_t *>(dst + data_bytes - 2) = stage[data_bytes / 2 - 1];
 }
 
-// ---- launch 5: zero flags[flag_off[blocks] ..) and data[data_off[blocks] ..), 64 bytes per step
+// ---- launch 5: zero flags[flag_off[blocks] ..) and data[data_off[blocks] ..): 16 bytes per lane and step,
+// neighbouring lanes at neighbouring addresses (the piece the used part ends in byte by byte)
 __global__ __launch_bounds__(256) void lz_clear_slack_kernel(const int32_t *__restrict__ flag_off,
                                                             const int32_t *__restrict__ data_off,
                                                             int64_t blocks, uint8_t *__restrict__ flags,
@@ -466,13 +467,11 @@ __global__ __launch_bounds__(256) void lz_clear_slack_kernel(const int32_t *__re
         uint8_t *buf = a ? data : flags;
         const int64_t size = a ? blocks * LZ_BLOCK_BYTES : blocks * (LZ_SYMS / 8);     // multiples of 64
         const int64_t used = min(max((int64_t)(a ? data_off[blocks] : flag_off[blocks]), (int64_t)0), size);
-        for (int64_t lo = (used / 64 + tid) * 64; lo < size; lo += nthreads * 64) {
+        for (int64_t lo = (used / 16 + tid) * 16; lo < size; lo += nthreads * 16) {
             if (lo >= used) {
-                uint4 *p = reinterpret_cast<uint4 *>(buf + lo);
-                const uint4 z = make_uint4(0, 0, 0, 0);
-                p[0] = z; p[1] = z; p[2] = z; p[3] = z;
+                *reinterpret_cast<uint4 *>(buf + lo) = make_uint4(0, 0, 0, 0);
             } else {
-                for (int64_t q = used; q < lo + 64; ++q) buf[q] = 0;
+                for (int64_t q = used; q < lo + 16; ++q) buf[q] = 0;
             }
         }
     }
@@ -718,7 +717,7 @@ extern "C" int planmoe_lz_compress(const void *input, int64_t nbytes, int32_t *f
     lz_scan_totals_kernel<<<1, LZ_MAX_CHUNKS, 0, st>>>(totals, chunks, bases);
     lz_place_kernel<<<(unsigned)groups, LZ_WAVES * WAVE, 0, st>>>((const uint32_t *)input, nbytes / 4, blocks,
                                                                 flag_offsets, data_offsets, cls, bases, flags, data);
-    const int64_t slack_chunks = (blocks * LZ_BLOCK_BYTES / 64 + 255) / 256;          // enough for all of data
+    const int64_t slack_chunks = (blocks * LZ_BLOCK_BYTES / 16 + 255) / 256;          // enough for all of data
     lz_clear_slack_kernel<<<(unsigned)min(slack_chunks, (int64_t)4096), 256, 0, st>>>(flag_offsets, data_offsets,
                                                                                    blocks, flags, data);
     PM_LAUNCH_CHECK("planmoe_lz_compress");
