@@ -73,10 +73,7 @@ def test_forward_entry_point(T, M, E, k, cf):
     C = ops.capacity(T, E, k, cf, 4)
     out = ops.forward_int8(x, wg, k, C, want_scores=True, want_counts=True)
     scores = out["scores"].cpu().numpy()
-    top = np.sort(scores, axis=1)[:, ::-1][:, :min(k + 1, E)]
-    if E > 1 and not (top[:, :-1] > top[:, 1:]).all():
-        pytest.skip("tied scores in this draw: the lower-index rule is covered elsewhere")
-    idx, loc, gates, counts = oracle.route_topk(scores, k)
+    idx, loc, gates, counts = oracle.route_topk(scores, k)        # (equal scores: the lower expert id, here as there)
     assert np.array_equal(out["indices"].cpu().numpy(), idx) and np.array_equal(out["locations"].cpu().numpy(), loc)
     assert np.array_equal(raw(out["gates"]), np_raw(gates)) and np.array_equal(out["counts"].cpu().numpy(), counts)
     c2, b2, s2 = ops.dispatch_int8(x, list(out["indices"]), list(out["locations"]), None, E, C)
