@@ -451,15 +451,26 @@ def forward_plain(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, norm
     return out
 
 
+_single_serves = {}
+
+
 def forward_int8_single_serves(x, wg, top_k, fp32_gate=True):
     """The shapes planmoe_forward_int8_single takes: bf16 rows of 256 to 4096 values in steps of 256, up to
     16 experts, top_k <= 4, and so few tokens that all its work-groups are resident at once (64 per compute
-    unit; 128 for rows of up to 1792 values).  The library is asked (planmoe_forward_int8_single_serves)."""
+    unit; 128 for rows of up to 1792 values).  The library is asked (planmoe_forward_int8_single_serves),
+    once per shape and device."""
     if not (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 2 and x.shape[0] >= 1):
         return False
-    with torch.cuda.device(x.device):
-        return bool(lib.planmoe_forward_int8_single_serves(_dt(x, "forward_int8_single"), int(bool(fp32_gate)), x.shape[0],
-                                                           x.shape[1], wg.shape[0], int(top_k)))
+    key = (x.device.index, x.shape[0], x.shape[1], wg.shape[0], int(top_k), bool(fp32_gate))
+    hit = _single_serves.get(key)
+    if hit is None:
+        with torch.cuda.device(x.device):
+            hit = bool(lib.planmoe_forward_int8_single_serves(_dt(x, "forward_int8_single"), int(bool(fp32_gate)), x.shape[0],
+                                                              x.shape[1], wg.shape[0], int(top_k)))
+        if len(_single_serves) > 4096:
+            _single_serves.clear()
+        _single_serves[key] = hit
+    return hit
 
 
 def forward_int8_single(x, wg, top_k, capacity_, fp32_gate=True, logit_bias=None, normalize_gate=True,
