@@ -278,7 +278,8 @@ int planmoe_forward_int8(const void *x, const void *wg, int dtype, int fp32_gate
  * published its expert histogram, then writes them to their slots.  Served shapes: bf16, model_dim
  * a multiple of 256 up to 4096, experts <= 16, top_k <= 4, samples <= 64 x the number of work-groups
  * that are resident at once (one per compute unit, two for rows of up to 1792 values:
- * planmoe_forward_int8_single_serves tells); any other shape is an error here (planmoe_forward_int8 picks between the two on its own).  Outputs as
+ * planmoe_forward_int8_single_serves tells); any other shape is an error here, and nothing is enqueued (planmoe_forward_int8
+ * takes every shape; the Python layer asks the query and picks).  Outputs as
  * planmoe_forward_int8 (logits may differ from it in the last bit: another summation order).
  * The wait between the work-groups is bounded: spin_limit polls (0 = the default, about a second);
  * a work-group that gives up writes none of its rows, marks its tokens dropped (locations =
