@@ -273,9 +273,9 @@ int planmoe_forward_int8(const void *x, const void *wg, int dtype, int fp32_gate
                          void *workspace, size_t workspace_bytes, void *stream);
 
 /* The same chain in ONE launch that reads x once (the two launches above read it twice: the slot
- * of a second choice needs the first-choice counts of the whole batch).  One work-group per compute
- * unit holds the codes of its tokens on chip (LDS and registers) until every work-group has
- * published its expert histogram, then writes them to their slots.  Served shapes: bf16, model_dim
+ * of a second choice needs the first-choice counts of the whole batch).  Work-groups of up to 64
+ * tokens, all resident at once, hold the codes of their tokens on chip (LDS and registers) until
+ * every work-group has published its expert histogram, then write them to their slots.  Served shapes: bf16, model_dim
  * a multiple of 256 up to 4096, experts <= 16, top_k <= 4, samples <= 64 x the number of work-groups
  * that are resident at once (one per compute unit, two for rows of up to 1792 values:
  * planmoe_forward_int8_single_serves tells); any other shape is an error here, and nothing is enqueued (planmoe_forward_int8
